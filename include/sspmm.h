@@ -1,0 +1,115 @@
+/*
+ * C ABI of libsspmm_amd.so: vector-sparse SpMM and Sparse Vector Compression (RowMerge) on
+ * AMD gfx950.  Plain pointers and sizes only; every pointer is a DEVICE pointer owned by the
+ * caller unless a comment says otherwise.  All entry points are asynchronous on the given
+ * HIP stream (NULL = the default stream), never synchronise, and return 0 on success or a
+ * non-zero hipError_t value (1 = invalid value for rejected arguments).
+ *
+ * The "CVSE" format (reference RowMerge/sparse_matrix_format.py:152-175 and
+ * SSpMM/sspmm_test.cpp:28-70):
+ *   m_vec                     number of vector-rows, = ceil(M / V); the SpMM treats M = m_vec*V
+ *   row_offsets[m_vec+1]      int32, start of each vector-row in col_idx (non-decreasing)
+ *   col_idx[nvec]             int32, column of each non-zero V x 1 vector, nvec = row_offsets[m_vec]
+ *   values[nvec*V]            fp16, vector-major: values[j*V + v] = A[i*V + v, col_idx[j]]
+ *   row_indices[m_vec]        int32 permutation of vector-rows (processing order), may be NULL
+ */
+#ifndef SSPMM_AMD_SSPMM_H
+#define SSPMM_AMD_SSPMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* IEEE binary16 bit pattern (same memory as _Float16 / __half / torch.float16). */
+typedef uint16_t sspmm_half_t;
+
+/* Library version, (major << 16) | minor. */
+int sspmm_version(void);
+
+/* Static text for a return code of this library. */
+const char *sspmm_error_string(int code);
+
+/*
+ * C[m_vec*V, N] = A_cvse[m_vec*V, K] * B[K, N]; fp16 inputs, fp32 accumulation, fp32 output.
+ * Replaces spmm::SSpMM(..., float* output_matrix), reference SSpMM/include/sspmm.cuh:31-37
+ * (launcher SSpMM/src/sspmm.cu:548-587, 626-635).  Argument order m_vec, V, N, K as the
+ * reference's callers pass it (SSpMM/sspmm_test.cpp:189).
+ *   V must be 8 or 16; any N >= 0 (the reference silently required N % 64 == 0);
+ *   B and C are row-major and dense; C is fully overwritten, all-zero vector-rows included;
+ *   K*N and nvec*V must be below 2^31.  row_indices may be NULL (natural order); results do
+ *   not depend on it.
+ */
+int sspmm_f16_f32(int m_vec, int V, int N, int K, const int32_t *row_indices, const int32_t *row_offsets,
+                  const int32_t *col_idx, const sspmm_half_t *values, const sspmm_half_t *B, float *C,
+                  void *hip_stream);
+
+/*
+ * Same with fp16 output (the fp32 sum rounded to nearest even).  Replaces
+ * spmm::SSpMM(..., half* output_matrix), reference SSpMM/include/sspmm.cuh:39-45
+ * (launcher SSpMM/src/sspmm.cu:588-623, 638-648) and the kernel behind sptrans.spmm.spmm,
+ * end2end/sspmm_e2e/src/cuda/spmm_kernel.cu:460-514.
+ */
+int sspmm_f16_f16(int m_vec, int V, int N, int K, const int32_t *row_indices, const int32_t *row_offsets,
+                  const int32_t *col_idx, const sspmm_half_t *values, const sspmm_half_t *B, sspmm_half_t *C,
+                  void *hip_stream);
+
+/*
+ * Batched SpMM with one sparsity pattern shared by the whole batch; per-batch values, B and C
+ * at the given element strides.  Replaces batched_spmm_cuda / batchedWmmaSpmmKernel8,
+ * reference end2end/sspmm_e2e/src/cuda/spmm_kernel.cu:145-169, 516-586 (strides :532-534).
+ */
+int sspmm_batched_f16_f16(int batch, int m_vec, int V, int N, int K, const int32_t *row_indices,
+                          const int32_t *row_offsets, const int32_t *col_idx, const sspmm_half_t *values,
+                          int64_t stride_values, const sspmm_half_t *B, int64_t stride_B, sspmm_half_t *C,
+                          int64_t stride_C, void *hip_stream);
+
+/* Batched form with fp32 output (no counterpart kernel in the reference, which only batches the
+ * fp16 output; same semantics as sspmm_f16_f32 per batch element). */
+int sspmm_batched_f16_f32(int batch, int m_vec, int V, int N, int K, const int32_t *row_indices,
+                          const int32_t *row_offsets, const int32_t *col_idx, const sspmm_half_t *values,
+                          int64_t stride_values, const sspmm_half_t *B, int64_t stride_B, float *C,
+                          int64_t stride_C, void *hip_stream);
+
+/*
+ * row_indices = vector-rows ordered by descending length (ties: ascending row).  Replaces
+ * SortedRowSwizzle, reference SSpMM/include/bm_test_utils.h:210-225 (a host std::sort there).
+ * No scratch memory is needed.
+ */
+int sspmm_sorted_row_swizzle(int m_vec, const int32_t *row_offsets, int32_t *row_indices, void *hip_stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Sparse Vector Compression (RowMerge): CSR -> CVSE.  Replaces the Python pass
+ * CVSE.__init__, reference RowMerge/sparse_matrix_format.py:94-123 (merge at :110), and adds
+ * the value packing its consumers define (SSpMM/sspmm_test.cpp:90).
+ *
+ * Two phases so the caller can size the outputs:
+ *   1. svc_count  writes vec_row_ptr[m_vec+1]; nvec = vec_row_ptr[m_vec] (read it back, or
+ *                 skip the read and size the outputs for the bound nvec <= nnz).
+ *   2. svc_fill   writes vec_col[nvec] and, when csr_val != NULL, vec_val[nvec*V] (zero filled).
+ * Both phases take the same workspace of svc_workspace_bytes(M, nnz, V) bytes; svc_fill
+ * consumes what svc_count left there.
+ *
+ * order: SVC_ORDER_CPYTHON reproduces the column order of the reference's output files (the
+ * iteration order of CPython's set in `list(set(acc + row))`), bit for bit;
+ * SVC_ORDER_SORTED stores each vector-row's columns ascending.
+ * Column indices must lie in [0, K); a CSR row must not repeat a column.
+ * ---------------------------------------------------------------------------------------- */
+#define SVC_ORDER_CPYTHON 0
+#define SVC_ORDER_SORTED 1
+
+size_t svc_workspace_bytes(int M, int64_t nnz, int V);
+
+int svc_count(int M, int K, int V, const int32_t *row_ptr, const int32_t *col_ind, int64_t nnz, int order,
+              int32_t *vec_row_ptr, void *workspace, void *hip_stream);
+
+int svc_fill(int M, int K, int V, const int32_t *row_ptr, const int32_t *col_ind, const sspmm_half_t *csr_val,
+             int64_t nnz, int order, const int32_t *vec_row_ptr, void *workspace, int32_t *vec_col,
+             sspmm_half_t *vec_val, void *hip_stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SSPMM_AMD_SSPMM_H */

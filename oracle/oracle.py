@@ -1,0 +1,155 @@
+"""ctypes/numpy front end of the C oracle plus the pure-Python RowMerge restatement.
+
+TEST INFRASTRUCTURE ONLY (see sspmm_oracle.c for what each function follows and
+what pins it).  Nothing in sspmm_amd/ imports this module.
+"""
+import ctypes
+import math
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+_lib = None
+
+
+def build(force=False):
+    """Compile liboracle.so with gcc (seconds)."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.check_call(["make", "-C", _HERE, "-B" if force else "-s", "liboracle.so"])
+    return _LIB_PATH
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        L = ctypes.CDLL(_LIB_PATH)
+        i32p = ctypes.POINTER(ctypes.c_int32)
+        u16p = ctypes.POINTER(ctypes.c_uint16)
+        f32p = ctypes.POINTER(ctypes.c_float)
+        L.oracle_pyset_order.restype = ctypes.c_int64
+        L.oracle_pyset_order.argtypes = [i32p, ctypes.c_int64, i32p]
+        L.oracle_svc.restype = ctypes.c_int64
+        L.oracle_svc.argtypes = [ctypes.c_int32] * 3 + [i32p, i32p, u16p, ctypes.c_int32, i32p, i32p, u16p]
+        L.oracle_spmm_f32.restype = None
+        L.oracle_spmm_f32.argtypes = [ctypes.c_int32] * 4 + [i32p, i32p, u16p, u16p, f32p, ctypes.c_int32]
+        L.oracle_spmm_f16.restype = None
+        L.oracle_spmm_f16.argtypes = [ctypes.c_int32] * 4 + [i32p, i32p, u16p, u16p, u16p, ctypes.c_int32]
+        L.oracle_sorted_row_swizzle.restype = None
+        L.oracle_sorted_row_swizzle.argtypes = [ctypes.c_int32, i32p, i32p]
+        L.oracle_h2f.restype = ctypes.c_float
+        L.oracle_h2f.argtypes = [ctypes.c_uint16]
+        L.oracle_f2h.restype = ctypes.c_uint16
+        L.oracle_f2h.argtypes = [ctypes.c_float]
+        _lib = L
+    return _lib
+
+
+def _p(a, ct):
+    return None if a is None else a.ctypes.data_as(ctypes.POINTER(ct))
+
+
+def _i32(a):
+    return np.ascontiguousarray(a, dtype=np.int32)
+
+
+def _u16(a):
+    """fp16 array -> its bit pattern as uint16 (no copy when already contiguous)."""
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.float16:
+        return a.view(np.uint16)
+    return np.ascontiguousarray(a, dtype=np.uint16)
+
+
+def pyset_order(keys):
+    """C model of list(set(keys)) for non-negative ints."""
+    keys = _i32(keys)
+    out = np.empty(max(len(keys), 1), dtype=np.int32)
+    n = lib().oracle_pyset_order(_p(keys, ctypes.c_int32), len(keys), _p(out, ctypes.c_int32))
+    return out[:n].copy()
+
+
+def svc(M, K, V, row_ptr, col_ind, csr_val=None, order="cpython"):
+    """RowMerge.  Returns (vec_row_ptr[int32 m_vec+1], vec_col[int32 nvec], vec_val[fp16 nvec*V] or None)."""
+    row_ptr, col_ind = _i32(row_ptr), _i32(col_ind)
+    nnz = int(row_ptr[M]) if M > 0 else 0
+    m_vec = (M + V - 1) // V
+    vrp = np.zeros(m_vec + 1, dtype=np.int32)
+    vcol = np.empty(max(nnz, 1), dtype=np.int32)
+    vval = None
+    cv = None
+    if csr_val is not None:
+        cv = _u16(csr_val)
+        vval = np.empty(max(nnz, 1) * V, dtype=np.uint16)
+    nvec = lib().oracle_svc(M, K, V, _p(row_ptr, ctypes.c_int32), _p(col_ind, ctypes.c_int32),
+                            _p(cv, ctypes.c_uint16), {"cpython": 0, "sorted": 1}[order],
+                            _p(vrp, ctypes.c_int32), _p(vcol, ctypes.c_int32), _p(vval, ctypes.c_uint16))
+    if nvec < 0:
+        raise ValueError("oracle_svc: bad arguments")
+    return vrp, vcol[:nvec].copy(), (None if vval is None else vval[:nvec * V].copy().view(np.float16))
+
+
+def spmm(m_vec, V, N, K, row_offsets, col_idx, values, B, out_dtype=np.float32, threads=1):
+    """Host SpMM check loop of the reference harness; values/B are fp16 arrays."""
+    row_offsets, col_idx = _i32(row_offsets), _i32(col_idx)
+    vals, Bb = _u16(values), _u16(B)
+    M = m_vec * V
+    if out_dtype == np.float32:
+        C = np.empty((M, N), dtype=np.float32)
+        lib().oracle_spmm_f32(m_vec, V, N, K, _p(row_offsets, ctypes.c_int32), _p(col_idx, ctypes.c_int32),
+                              _p(vals, ctypes.c_uint16), _p(Bb, ctypes.c_uint16), _p(C, ctypes.c_float), threads)
+        return C
+    C = np.empty((M, N), dtype=np.uint16)
+    lib().oracle_spmm_f16(m_vec, V, N, K, _p(row_offsets, ctypes.c_int32), _p(col_idx, ctypes.c_int32),
+                          _p(vals, ctypes.c_uint16), _p(Bb, ctypes.c_uint16), _p(C, ctypes.c_uint16), threads)
+    return C.view(np.float16)
+
+
+def sorted_row_swizzle(row_offsets):
+    row_offsets = _i32(row_offsets)
+    rows = len(row_offsets) - 1
+    out = np.empty(max(rows, 1), dtype=np.int32)
+    lib().oracle_sorted_row_swizzle(rows, _p(row_offsets, ctypes.c_int32), _p(out, ctypes.c_int32))
+    return out[:rows].copy()
+
+
+def rowmerge_python(M, V, col_lists):
+    """Pure-Python RowMerge, the reference's own algorithm on the language runtime's set.
+
+    Follows CVSE.__init__ (RowMerge/sparse_matrix_format.py:100-123): per vector-row,
+    fold `list(set(acc + row))` over its V member rows (rows >= M skipped), then the
+    running total becomes the next row pointer.  This is the timed "Python RowMerge"
+    CPU baseline and the ground truth for column order.
+    """
+    m_vec = math.ceil(M / V)
+    ptr = [0]
+    flat = []
+    total = 0
+    for i in range(m_vec):
+        acc = []
+        for j in range(V):
+            if V * i + j < M:
+                acc = list(set(acc + col_lists[V * i + j]))
+        total += len(acc)
+        ptr.append(total)
+        flat.extend(acc)
+    return ptr, flat
+
+
+def csr_col_lists(M, row_ptr, col_ind):
+    """colInd_list_array of the reference (sparse_matrix_format.py:41-53): per-row python lists."""
+    ci = [int(c) for c in col_ind]
+    return [ci[int(row_ptr[i]):int(row_ptr[i + 1])] for i in range(M)]
+
+
+def densify(m_vec, V, K, row_offsets, col_idx, values):
+    """csr2dense of the reference (end2end/sspmm_e2e/verify/static_mask.py:29-45), fp16 [m_vec*V, K]."""
+    A = np.zeros((m_vec * V, K), dtype=np.float16)
+    values = np.asarray(values).reshape(-1, V)
+    for i in range(m_vec):
+        for j in range(int(row_offsets[i]), int(row_offsets[i + 1])):
+            A[i * V:(i + 1) * V, int(col_idx[j])] = values[j]
+    return A

@@ -1,0 +1,140 @@
+// extern "C" boundary of libsspmm_amd.so: argument checks and dispatch to the kernels.
+// The declarations and their contracts are in include/sspmm.h.
+#include <hip/hip_runtime.h>
+
+#include "../../include/sspmm.h"
+#include "spmm_kernels.h"
+#include "svc_kernels.h"
+
+namespace {
+
+constexpr int kInvalid = (int)hipErrorInvalidValue;
+
+int spmm_entry(int batch, int m_vec, int V, int N, int K, const int32_t *row_indices, const int32_t *row_offsets,
+               const int32_t *col_idx, const sspmm_half_t *values, int64_t stride_values, const sspmm_half_t *B,
+               int64_t stride_B, void *C, int64_t stride_C, bool out_f16, void *stream) {
+  if (V != 8 && V != 16) return kInvalid;
+  if (batch < 0 || m_vec < 0 || N < 0 || K < 0) return kInvalid;
+  if (batch == 0 || m_vec == 0 || N == 0) return 0;  // nothing to write
+  if (!row_offsets || !C) return kInvalid;
+  // col_idx / values / B are only dereferenced when some vector-row is non-empty, which the host
+  // cannot see (row_offsets is device memory): empty matrices may pass null for them.
+  if ((int64_t)K * N >= (1ll << 31)) return kInvalid;
+  if ((int64_t)m_vec * V >= (1ll << 31)) return kInvalid;
+  const int64_t tiles = ((int64_t)N + 63) / 64;
+  if ((int64_t)m_vec * tiles * batch >= (1ll << 31) - 8) return kInvalid;
+  if (batch > 1 && (stride_values < 0 || stride_B < 0 || stride_C < (int64_t)m_vec * V * N)) return kInvalid;
+  sspmm::SpmmArgs a{};
+  a.m_vec = m_vec;
+  a.N = N;
+  a.K = K;
+  a.batch = batch;
+  a.row_indices = row_indices;
+  a.row_offsets = row_offsets;
+  a.col_idx = col_idx;
+  a.values = values;
+  a.B = B;
+  a.C = C;
+  a.stride_values = stride_values;
+  a.stride_B = stride_B;
+  a.stride_C = stride_C;
+  return (int)sspmm::launch_spmm(a, V, out_f16, /*force_generic=*/false, static_cast<hipStream_t>(stream));
+}
+
+}  // namespace
+
+extern "C" {
+
+int sspmm_version(void) { return (0 << 16) | 1; }
+
+const char *sspmm_error_string(int code) {
+  if (code == 0) return "success";
+  if (code == kInvalid) return "invalid argument (unsupported V, negative size, null pointer or index range)";
+  return hipGetErrorString(static_cast<hipError_t>(code));
+}
+
+int sspmm_f16_f32(int m_vec, int V, int N, int K, const int32_t *row_indices, const int32_t *row_offsets,
+                  const int32_t *col_idx, const sspmm_half_t *values, const sspmm_half_t *B, float *C,
+                  void *hip_stream) {
+  return spmm_entry(1, m_vec, V, N, K, row_indices, row_offsets, col_idx, values, 0, B, 0, C, 0, false, hip_stream);
+}
+
+int sspmm_f16_f16(int m_vec, int V, int N, int K, const int32_t *row_indices, const int32_t *row_offsets,
+                  const int32_t *col_idx, const sspmm_half_t *values, const sspmm_half_t *B, sspmm_half_t *C,
+                  void *hip_stream) {
+  return spmm_entry(1, m_vec, V, N, K, row_indices, row_offsets, col_idx, values, 0, B, 0, C, 0, true, hip_stream);
+}
+
+int sspmm_batched_f16_f16(int batch, int m_vec, int V, int N, int K, const int32_t *row_indices,
+                          const int32_t *row_offsets, const int32_t *col_idx, const sspmm_half_t *values,
+                          int64_t stride_values, const sspmm_half_t *B, int64_t stride_B, sspmm_half_t *C,
+                          int64_t stride_C, void *hip_stream) {
+  return spmm_entry(batch, m_vec, V, N, K, row_indices, row_offsets, col_idx, values, stride_values, B, stride_B, C,
+                    stride_C, true, hip_stream);
+}
+
+int sspmm_batched_f16_f32(int batch, int m_vec, int V, int N, int K, const int32_t *row_indices,
+                          const int32_t *row_offsets, const int32_t *col_idx, const sspmm_half_t *values,
+                          int64_t stride_values, const sspmm_half_t *B, int64_t stride_B, float *C,
+                          int64_t stride_C, void *hip_stream) {
+  return spmm_entry(batch, m_vec, V, N, K, row_indices, row_offsets, col_idx, values, stride_values, B, stride_B, C,
+                    stride_C, false, hip_stream);
+}
+
+int sspmm_sorted_row_swizzle(int m_vec, const int32_t *row_offsets, int32_t *row_indices, void *hip_stream) {
+  if (m_vec < 0) return kInvalid;
+  if (m_vec == 0) return 0;
+  if (!row_offsets || !row_indices) return kInvalid;
+  return (int)sspmm::launch_sorted_row_swizzle(m_vec, row_offsets, row_indices, static_cast<hipStream_t>(hip_stream));
+}
+
+size_t svc_workspace_bytes(int M, int64_t nnz, int V) {
+  (void)M;
+  (void)V;
+  return sspmm::svc_workspace_layout(nnz, nullptr, nullptr);
+}
+
+static int svc_args(int M, int K, int V, const int32_t *row_ptr, const int32_t *col_ind, int64_t nnz, void *workspace,
+                    sspmm::SvcArgs *a) {
+  if (M < 0 || K < 0 || V < 1 || V > 64 || nnz < 0 || nnz >= (1ll << 28)) return kInvalid;
+  if (!row_ptr || !workspace || (nnz > 0 && !col_ind)) return kInvalid;
+  size_t off_pos, off_tables;
+  sspmm::svc_workspace_layout(nnz, &off_pos, &off_tables);
+  unsigned char *w = static_cast<unsigned char *>(workspace);
+  a->M = M;
+  a->K = K;
+  a->V = V;
+  a->row_ptr = row_ptr;
+  a->col_ind = col_ind;
+  a->tmp_cols = reinterpret_cast<int32_t *>(w);
+  a->pos = reinterpret_cast<int32_t *>(w + off_pos);
+  a->big_tables = reinterpret_cast<unsigned long long *>(w + off_tables);
+  a->lds_table_slots = 0;
+  return 0;
+}
+
+int svc_count(int M, int K, int V, const int32_t *row_ptr, const int32_t *col_ind, int64_t nnz, int order,
+              int32_t *vec_row_ptr, void *workspace, void *hip_stream) {
+  sspmm::SvcArgs a{};
+  if (order != SVC_ORDER_CPYTHON && order != SVC_ORDER_SORTED) return kInvalid;
+  if (!vec_row_ptr) return kInvalid;
+  const int rc = svc_args(M, K, V, row_ptr, col_ind, nnz, workspace, &a);
+  if (rc) return rc;
+  a.vec_row_ptr = vec_row_ptr;
+  return (int)sspmm::launch_svc_count(a, order, static_cast<hipStream_t>(hip_stream));
+}
+
+int svc_fill(int M, int K, int V, const int32_t *row_ptr, const int32_t *col_ind, const sspmm_half_t *csr_val,
+             int64_t nnz, int order, const int32_t *vec_row_ptr, void *workspace, int32_t *vec_col,
+             sspmm_half_t *vec_val, void *hip_stream) {
+  (void)order;
+  sspmm::SvcArgs a{};
+  if (!vec_row_ptr) return kInvalid;
+  if (csr_val && !vec_val) return kInvalid;
+  const int rc = svc_args(M, K, V, row_ptr, col_ind, nnz, workspace, &a);
+  if (rc) return rc;
+  if (M == 0) return 0;
+  return (int)sspmm::launch_svc_fill(a, csr_val, vec_row_ptr, vec_col, vec_val, static_cast<hipStream_t>(hip_stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,31 @@
+// Launch interface between the C ABI layer and the SVC (RowMerge) kernels.
+#ifndef SSPMM_AMD_SVC_KERNELS_H
+#define SSPMM_AMD_SVC_KERNELS_H
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace sspmm {
+
+struct SvcArgs {
+  int M, K, V;
+  const int32_t *row_ptr;
+  const int32_t *col_ind;
+  int32_t *vec_row_ptr;          // svc_count output
+  // workspace views
+  int32_t *tmp_cols;             // [nnz]   ordered columns of group g at row_ptr[g*V]
+  int32_t *pos;                  // [nnz]   position of every non-zero's column inside its group
+  unsigned long long *big_tables;  // [8*nnz] hash tables of groups too large for LDS
+  int lds_table_slots;           // filled by the launcher
+};
+
+// Total workspace bytes; optional byte offsets of the pos and table views.
+size_t svc_workspace_layout(int64_t nnz, size_t *off_pos, size_t *off_tables);
+
+hipError_t launch_svc_count(const SvcArgs &a, int order, hipStream_t stream);
+hipError_t launch_svc_fill(const SvcArgs &a, const uint16_t *csr_val, const int32_t *vec_row_ptr, int32_t *vec_col,
+                           uint16_t *vec_val, hipStream_t stream);
+
+}  // namespace sspmm
+#endif

@@ -1,0 +1,390 @@
+// Sparse Vector Compression (RowMerge) on the GPU: CSR -> CVSE.
+//
+// The reference does this in Python (reference RowMerge/sparse_matrix_format.py:94-123): for every
+// group of V consecutive rows it folds  acc = list(set(acc + row))  over the member rows, so the
+// column order of a vector-row is the iteration order of a CPython set, rebuilt from an empty
+// table once per member row.  SVC_ORDER_CPYTHON reproduces that order bit for bit.
+//
+// How a set construction is replayed in parallel.  For non-negative int keys hash(k) = k, and a
+// CPython set (Objects/setobject.c, 3.7 - 3.12) is an open-addressed table: look at slot
+// i = k & mask, then, when i + 9 <= mask, at the nine slots after it; if none is free continue
+// with perturb >>= 5, i = (5 i + 1 + perturb) & mask.  The table starts with 8 slots and, as
+// soon as 5 * fill >= 3 * mask after an insert, is rebuilt into the smallest power of two above
+// 4 * fill (2 * fill beyond 50 000 keys) by re-inserting the keys in slot order.  Inserting a key
+// that is present changes nothing, so duplicates are dropped first; after that the number of
+// keys alone fixes where the rebuilds happen, and a construction is a short sequence of phases:
+//     phase with S slots: keys[0 .. min(n, thr(S))) are inserted into an empty S-slot table,
+//     where keys[0 .. thr(previous S)) have been put into the previous table's slot order.
+// Within a phase the final table is the unique first-come-first-served placement: every key sits
+// in the first slot of its probe sequence not held by an earlier key.  That fixed point is
+// reached by any interleaving of threads that claim slots with a 64-bit atomic min on
+// (insertion index << 32 | key): a later key that is displaced by an earlier one resumes its own
+// probe sequence behind that slot.  So one thread per key inserts a whole phase at once.
+//
+// One workgroup owns one vector-row group.  The list and the table live in LDS (64-thread groups
+// for up to 306 keys, 256 threads up to 1228, 1024 threads up to 4914) or, beyond that, in the
+// caller's workspace.  svc_count runs the replay and leaves the ordered columns and every
+// non-zero's position in the workspace; svc_fill copies them to their final offsets and scatters
+// the values into zero-filled V-wide vectors.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "svc_kernels.h"
+
+namespace sspmm {
+
+typedef unsigned long long u64;
+static constexpr u64 kEmpty = ~0ull;
+
+__device__ __forceinline__ void probe_start(uint32_t key, uint32_t mask, uint32_t &i, uint32_t &perturb,
+                                            uint32_t &lin) {
+  i = key & mask;
+  perturb = key;
+  lin = 0;
+}
+
+__device__ __forceinline__ void probe_next(uint32_t mask, uint32_t &i, uint32_t &perturb, uint32_t &lin) {
+  const uint32_t window = (i + 9u <= mask) ? 9u : 0u;
+  if (lin < window) {
+    ++lin;
+  } else {
+    perturb >>= 5;
+    i = (i * 5u + 1u + perturb) & mask;
+    lin = 0;
+  }
+}
+
+// Slot that holds `key`, or -1.  The table always keeps free slots, so the walk ends.
+__device__ __forceinline__ int find_slot(const u64 *table, uint32_t mask, uint32_t key) {
+  uint32_t i, perturb, lin;
+  probe_start(key, mask, i, perturb, lin);
+  for (;;) {
+    const u64 x = table[i + lin];
+    if (x == kEmpty) return -1;
+    if ((uint32_t)x == key) return (int)(i + lin);
+    probe_next(mask, i, perturb, lin);
+  }
+}
+
+// First-come-first-served placement of (order, key) by atomic min; see the file header.
+__device__ __forceinline__ void place(u64 *table, uint32_t mask, uint32_t key, uint32_t order) {
+  u64 mine = ((u64)order << 32) | key;
+  uint32_t i, perturb, lin;
+  probe_start(key, mask, i, perturb, lin);
+  for (;;) {
+    const uint32_t s = i + lin;
+    const u64 old = atomicMin(&table[s], mine);
+    if (old == kEmpty) return;
+    // The same key twice can only come from a CSR row that repeats a column (invalid input):
+    // keep one copy so the output stays a valid pattern.
+    if ((uint32_t)old == (uint32_t)mine) return;
+    if (old > mine) {
+      // An entry inserted later than mine was sitting here: it moves on.  It reached this slot
+      // on the first visit of its own probe sequence, so replay that sequence up to here.
+      mine = old;
+      key = (uint32_t)old;
+      probe_start(key, mask, i, perturb, lin);
+      while (i + lin != s) probe_next(mask, i, perturb, lin);
+    }
+    probe_next(mask, i, perturb, lin);
+  }
+}
+
+// Exclusive prefix sum of one int per thread over the workgroup; *total = sum.  `scratch` holds
+// THREADS / 64 + 1 ints of LDS.  Contains barriers: every thread of the group must call it.
+template <int THREADS>
+__device__ __forceinline__ int block_exclusive_scan(int x, int *total, int *scratch) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int incl = x;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int y = __shfl_up(incl, d, 64);
+    if (lane >= d) incl += y;
+  }
+  constexpr int WAVES = THREADS / 64;
+  if (WAVES == 1) {
+    *total = __shfl(incl, 63, 64);
+    return incl - x;
+  }
+  __syncthreads();  // scratch may still be read from a previous call
+  if (lane == 63) scratch[wave] = incl;
+  __syncthreads();
+  int base = 0, sum = 0;
+#pragma unroll
+  for (int wv = 0; wv < WAVES; ++wv) {
+    const int t = scratch[wv];
+    if (wv < wave) base += t;
+    sum += t;
+  }
+  *total = sum;
+  return base + incl - x;
+}
+
+__device__ __forceinline__ uint32_t resize_threshold(uint32_t slots) { return (3u * (slots - 1u) + 4u) / 5u; }
+
+__device__ __forceinline__ uint32_t resized_slots(uint32_t fill) {
+  const uint32_t minused = fill > 50000u ? fill * 2u : fill * 4u;
+  uint32_t s = 8;
+  while (s <= minused) s <<= 1;
+  return s;
+}
+
+// Writes the keys of table[0..slots) to list[0..) in slot order; when `final` also replaces each
+// entry's insertion index by its position in that order.
+template <int THREADS>
+__device__ __forceinline__ int extract_slot_order(u64 *table, uint32_t slots, int *list, bool final, int *scratch) {
+  const uint32_t per = (slots + THREADS - 1) / THREADS;
+  const uint32_t lo = min(slots, threadIdx.x * per), hi = min(slots, lo + per);
+  int mine = 0;
+  for (uint32_t s = lo; s < hi; ++s) mine += table[s] != kEmpty;
+  int total;
+  int at = block_exclusive_scan<THREADS>(mine, &total, scratch);
+  for (uint32_t s = lo; s < hi; ++s) {
+    const u64 x = table[s];
+    if (x != kEmpty) {
+      list[at] = (int)(uint32_t)x;
+      if (final) table[s] = ((u64)(uint32_t)at << 32) | (uint32_t)x;
+      ++at;
+    }
+  }
+  return total;
+}
+
+// list(set(list[0..n))) for distinct keys: on return list holds the set's iteration order and
+// table (slot count returned) maps each key to its position.  n is updated to the number of keys
+// in the table (it only changes for invalid input with repeated keys).
+template <int THREADS>
+__device__ __forceinline__ uint32_t rebuild_set(u64 *table, int *list, int &n, int *scratch) {
+  uint32_t slots = 8;
+  for (;;) {
+    const uint32_t thr = resize_threshold(slots);
+    const int cnt = min(n, (int)thr);
+    for (uint32_t s = threadIdx.x; s < slots; s += THREADS) table[s] = kEmpty;
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < cnt; idx += THREADS) place(table, slots - 1u, (uint32_t)list[idx], (uint32_t)idx);
+    __syncthreads();
+    const bool final = n < (int)thr;
+    const int kept = extract_slot_order<THREADS>(table, slots, list, final, scratch);
+    __syncthreads();
+    if (final) {
+      n = kept;
+      return slots;
+    }
+    slots = resized_slots(thr);
+  }
+}
+
+// Class of a vector-row group by its key bound: which kernel instance handles it.
+__device__ __forceinline__ bool in_class(int bound, int lo, int hi) { return bound > lo && bound <= hi; }
+
+template <int THREADS, bool IN_LDS>
+__global__ __launch_bounds__(THREADS) void svc_merge_cpython_kernel(const SvcArgs a, int class_lo, int class_hi,
+                                                                    int list_cap) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int grp = blockIdx.x;
+  const int r0 = grp * a.V, r1 = min(a.M, r0 + a.V);
+  const int e0 = a.row_ptr[r0], e1 = a.row_ptr[r1];
+  const int bound = min(e1 - e0, a.K);
+  if (!in_class(bound, class_lo, class_hi)) return;  // uniform over the group
+
+  int *scratch = reinterpret_cast<int *>(smem);  // 32 ints
+  int *list;
+  u64 *table;
+  if (IN_LDS) {
+    table = reinterpret_cast<u64 *>(smem + 128);
+    list = reinterpret_cast<int *>(smem + 128 + (size_t)a.lds_table_slots * 8);
+  } else {
+    list_cap = e1 - e0;
+    list = a.tmp_cols + e0;
+    table = a.big_tables + (int64_t)e0 * 8;
+  }
+
+  int n = 0;
+  uint32_t slots = 0;
+  for (int r = r0; r < r1; ++r) {
+    const int b = a.row_ptr[r], e = a.row_ptr[r + 1];
+    // acc + row: append the row's columns that are not in acc yet, in row order.
+    int appended = 0;
+    for (int base = b; base < e; base += THREADS) {
+      const int idx = base + (int)threadIdx.x;
+      bool is_new = false;
+      int key = 0;
+      if (idx < e) {
+        key = a.col_ind[idx];
+        is_new = (slots == 0) || find_slot(table, slots - 1u, (uint32_t)key) < 0;
+      }
+      int total;
+      const int rank = block_exclusive_scan<THREADS>(is_new ? 1 : 0, &total, scratch);
+      if (is_new && n + appended + rank < list_cap) list[n + appended + rank] = key;
+      appended += total;
+    }
+    n = min(n + appended, list_cap);  // the cap only bites for invalid input (repeated columns)
+    __syncthreads();
+    slots = rebuild_set<THREADS>(table, list, n, scratch);
+  }
+
+  if (threadIdx.x == 0) a.vec_row_ptr[grp + 1] = n;
+  if (IN_LDS)
+    for (int p = threadIdx.x; p < n; p += THREADS) a.tmp_cols[e0 + p] = list[p];
+  if (n > 0)
+    for (int idx = e0 + (int)threadIdx.x; idx < e1; idx += THREADS) {
+      const int s = find_slot(table, slots - 1u, (uint32_t)a.col_ind[idx]);
+      a.pos[idx] = s >= 0 ? (int)(table[s] >> 32) : 0;  // s < 0 only for invalid (capped) input
+    }
+}
+
+// Ascending order: a K-bit occupancy bitmap per group plus a per-word running popcount.
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void svc_merge_sorted_kernel(const SvcArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int grp = blockIdx.x;
+  const int r0 = grp * a.V, r1 = min(a.M, r0 + a.V);
+  const int e0 = a.row_ptr[r0], e1 = a.row_ptr[r1];
+  const int words = (a.K + 31) / 32;
+  int *scratch = reinterpret_cast<int *>(smem);
+  uint32_t *bits = reinterpret_cast<uint32_t *>(smem + 128);
+  int *prefix = reinterpret_cast<int *>(smem + 128 + (size_t)words * 4);
+  for (int w = threadIdx.x; w < words; w += THREADS) bits[w] = 0;
+  __syncthreads();
+  for (int idx = e0 + (int)threadIdx.x; idx < e1; idx += THREADS) {
+    const uint32_t c = (uint32_t)a.col_ind[idx];
+    atomicOr(&bits[c >> 5], 1u << (c & 31u));
+  }
+  __syncthreads();
+  const int per = (words + THREADS - 1) / THREADS;
+  const int lo = min(words, (int)threadIdx.x * per), hi = min(words, lo + per);
+  int mine = 0;
+  for (int w = lo; w < hi; ++w) mine += __popc(bits[w]);
+  int total;
+  int at = block_exclusive_scan<THREADS>(mine, &total, scratch);
+  for (int w = lo; w < hi; ++w) {
+    prefix[w] = at;
+    uint32_t x = bits[w];
+    while (x) {
+      const int b = __ffs(x) - 1;
+      x &= x - 1;
+      a.tmp_cols[e0 + at++] = w * 32 + b;
+    }
+  }
+  if (threadIdx.x == 0) a.vec_row_ptr[grp + 1] = total;
+  __syncthreads();
+  for (int idx = e0 + (int)threadIdx.x; idx < e1; idx += THREADS) {
+    const uint32_t c = (uint32_t)a.col_ind[idx];
+    a.pos[idx] = prefix[c >> 5] + __popc(bits[c >> 5] & ((1u << (c & 31u)) - 1u));
+  }
+}
+
+// In-place inclusive scan of vec_row_ptr[1..m_vec], vec_row_ptr[0] = 0.  One workgroup walks the
+// array in tiles of 1024: m_vec is the row count divided by V, a few thousand to a few hundred
+// thousand entries, far too little to be worth a multi-pass scan.
+__global__ __launch_bounds__(1024) void svc_scan_kernel(int m_vec, int32_t *vec_row_ptr) {
+  __shared__ int scratch[32];
+  int carry = 0;
+  if (threadIdx.x == 0) vec_row_ptr[0] = 0;
+  for (int base = 0; base < m_vec; base += 1024) {
+    const int i = base + (int)threadIdx.x;
+    const int x = i < m_vec ? vec_row_ptr[i + 1] : 0;
+    int total;
+    const int ex = block_exclusive_scan<1024>(x, &total, scratch);
+    if (i < m_vec) vec_row_ptr[i + 1] = carry + ex + x;
+    carry += total;
+  }
+}
+
+// One workgroup per vector-row group: copy its ordered columns to their final offset, clear its
+// value vectors and scatter the group's non-zeros into them.
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void svc_fill_kernel(const SvcArgs a, const uint16_t *csr_val,
+                                                          const int32_t *vec_row_ptr, int32_t *vec_col,
+                                                          uint16_t *vec_val) {
+  const int grp = blockIdx.x;
+  const int r0 = grp * a.V, r1 = min(a.M, r0 + a.V);
+  const int e0 = a.row_ptr[r0];
+  const int v0 = vec_row_ptr[grp], n = vec_row_ptr[grp + 1] - v0;
+  if (vec_col)
+    for (int p = threadIdx.x; p < n; p += THREADS) vec_col[v0 + p] = a.tmp_cols[e0 + p];
+  if (!vec_val) return;
+  // A group's value region starts at v0 * V halfs: a multiple of 4 bytes whenever V is even.
+  const int64_t halfs = (int64_t)n * a.V;
+  uint16_t *out = vec_val + (int64_t)v0 * a.V;
+  if ((a.V & 1) == 0) {
+    uint32_t *out32 = reinterpret_cast<uint32_t *>(out);
+    for (int64_t t = threadIdx.x; t < halfs / 2; t += THREADS) out32[t] = 0u;
+  } else {
+    for (int64_t t = threadIdx.x; t < halfs; t += THREADS) out[t] = 0;
+  }
+  __syncthreads();
+  for (int r = r0; r < r1; ++r) {
+    const int b = a.row_ptr[r], e = a.row_ptr[r + 1];
+    for (int idx = b + (int)threadIdx.x; idx < e; idx += THREADS)
+      out[(int64_t)a.pos[idx] * a.V + (r - r0)] = csr_val[idx];
+  }
+}
+
+static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+size_t svc_workspace_layout(int64_t nnz, size_t *off_pos, size_t *off_tables) {
+  const size_t n = (size_t)(nnz > 0 ? nnz : 1);
+  const size_t cols = align256(n * 4);
+  const size_t pos = align256(n * 4);
+  const size_t tables = align256(n * 64);
+  if (off_pos) *off_pos = cols;
+  if (off_tables) *off_tables = cols + pos;
+  return cols + pos + tables;
+}
+
+static constexpr int kSmallKeys = 306, kMediumKeys = 1228, kLargeKeys = 4914;
+
+template <int THREADS>
+static hipError_t launch_lds_class(const SvcArgs &base, int m_vec, int lo, int hi, int slots, hipStream_t stream) {
+  SvcArgs a = base;
+  a.lds_table_slots = slots;
+  const size_t lds = 128 + (size_t)slots * 8 + (size_t)hi * 4;
+  auto kern = svc_merge_cpython_kernel<THREADS, true>;
+  if (lds > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(kern, dim3(m_vec), dim3(THREADS), lds, stream, a, lo, hi, hi);
+  return hipGetLastError();
+}
+
+hipError_t launch_svc_count(const SvcArgs &a, int order, hipStream_t stream) {
+  const int m_vec = (a.M + a.V - 1) / a.V;
+  hipError_t e;
+  if (order == 0) {
+    // Four passes over the groups, each taking the groups of its size class; a group's class is
+    // decided from min(non-zeros of the group, K), an upper bound of its distinct columns.
+    if ((e = launch_lds_class<64>(a, m_vec, -1, kSmallKeys, 512, stream)) != hipSuccess) return e;
+    if ((e = launch_lds_class<256>(a, m_vec, kSmallKeys, kMediumKeys, 2048, stream)) != hipSuccess) return e;
+    if ((e = launch_lds_class<1024>(a, m_vec, kMediumKeys, kLargeKeys, 8192, stream)) != hipSuccess) return e;
+    hipLaunchKernelGGL((svc_merge_cpython_kernel<1024, false>), dim3(m_vec), dim3(1024), 128, stream, a, kLargeKeys,
+                       0x7fffffff, 0);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+  } else {
+    const int words = (a.K + 31) / 32;
+    const size_t lds = 128 + (size_t)words * 8;
+    if (lds > 160 * 1024) return hipErrorInvalidValue;
+    auto kern = svc_merge_sorted_kernel<256>;
+    if (lds > 64 * 1024) {
+      e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)lds);
+      if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL(kern, dim3(m_vec), dim3(256), lds, stream, a);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(svc_scan_kernel, dim3(1), dim3(1024), 0, stream, m_vec, a.vec_row_ptr);
+  return hipGetLastError();
+}
+
+hipError_t launch_svc_fill(const SvcArgs &a, const uint16_t *csr_val, const int32_t *vec_row_ptr, int32_t *vec_col,
+                           uint16_t *vec_val, hipStream_t stream) {
+  const int m_vec = (a.M + a.V - 1) / a.V;
+  hipLaunchKernelGGL((svc_fill_kernel<256>), dim3(m_vec), dim3(256), 0, stream, a, csr_val, vec_row_ptr, vec_col,
+                     csr_val ? vec_val : nullptr);
+  return hipGetLastError();
+}
+
+}  // namespace sspmm

@@ -1,0 +1,90 @@
+"""Python operator surface of the SpMM, mirroring the reference's torch extension
+`sptrans.spmm` (reference end2end/sspmm_e2e/src/cuda/spmm.cpp:11-46): same names, same
+argument order, same shape inference (reference end2end/sspmm_e2e/src/cuda/spmm_kernel.cu:
+468-475 and 524-538).  Tensors are torch-ROCm device tensors; torch only provides the device
+memory and the stream, the arithmetic happens in the HIP kernels behind the C ABI.
+"""
+import torch
+
+from . import _lib
+
+
+def _ptr(t):
+    return 0 if t is None else t.data_ptr()
+
+
+def _check_inputs(row_indices, row_offsets, column_indices, values, rhs_matrix, vec_length):
+    if vec_length not in (8, 16):
+        raise ValueError("vec_length must be 8 or 16, got %r" % (vec_length,))
+    for name, t, dt in (("row_offsets", row_offsets, torch.int32), ("column_indices", column_indices, torch.int32),
+                        ("values", values, torch.float16), ("rhs_matrix", rhs_matrix, torch.float16)):
+        if t.dtype != dt:
+            raise TypeError("%s must be %s, got %s" % (name, dt, t.dtype))
+        if not t.is_cuda:
+            raise ValueError("%s must live on the GPU" % name)
+        if not t.is_contiguous():
+            raise ValueError("%s must be contiguous" % name)
+    if row_indices is not None:
+        if row_indices.dtype != torch.int32 or not row_indices.is_cuda or not row_indices.is_contiguous():
+            raise TypeError("row_indices must be a contiguous int32 GPU tensor")
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def spmm(row_indices, row_offsets, column_indices, values, rhs_matrix, vec_length, out_dtype=torch.float16):
+    """C[m_vec*V, N] = A_cvse @ rhs_matrix[K, N].
+
+    Same call as the reference's `spmm(row_indices, row_offsets, column_indices, values,
+    rhs_matrix, vec_length)`; returns a new fp16 tensor like the reference, or fp32 when
+    out_dtype=torch.float32 (the reference's C++ `float*` overload, SSpMM/include/sspmm.cuh:31-37).
+    """
+    _check_inputs(row_indices, row_offsets, column_indices, values, rhs_matrix, vec_length)
+    if rhs_matrix.dim() != 2:
+        raise ValueError("rhs_matrix must be [K, N]")
+    m_vec = row_offsets.size(-1) - 1
+    K, N = rhs_matrix.size(0), rhs_matrix.size(1)
+    out = torch.empty((m_vec * vec_length, N), dtype=out_dtype, device=rhs_matrix.device)
+    fn = {torch.float16: _lib.lib().sspmm_f16_f16, torch.float32: _lib.lib().sspmm_f16_f32}[out_dtype]
+    with torch.cuda.device(rhs_matrix.device):
+        rc = fn(m_vec, vec_length, N, K, _ptr(row_indices), _ptr(row_offsets), _ptr(column_indices), _ptr(values),
+                _ptr(rhs_matrix), _ptr(out), _stream())
+    _lib.check(rc, "sspmm")
+    return out
+
+
+def bspmm(row_indices, row_offsets, column_indices, values, rhs_matrix, vec_length, out_dtype=torch.float16):
+    """Batched SpMM with one pattern for the whole batch: values [batch, nvec*V],
+    rhs_matrix [batch, K, N] -> [batch, m_vec*V, N] (reference batched_spmm_cuda,
+    end2end/sspmm_e2e/src/cuda/spmm_kernel.cu:516-586)."""
+    _check_inputs(row_indices, row_offsets, column_indices, values, rhs_matrix, vec_length)
+    m_vec = row_offsets.size(-1) - 1
+    K, N = rhs_matrix.size(-2), rhs_matrix.size(-1)
+    batch = rhs_matrix.numel() // (K * N) if K * N > 0 else (rhs_matrix.size(0) if rhs_matrix.dim() > 2 else 1)
+    nvec = column_indices.numel()
+    if values.numel() != batch * nvec * vec_length:
+        raise ValueError("values must hold batch * nvec * vec_length = %d elements, got %d"
+                         % (batch * nvec * vec_length, values.numel()))
+    M = m_vec * vec_length
+    out = torch.empty((batch, M, N), dtype=out_dtype, device=rhs_matrix.device)
+    fn = {torch.float16: _lib.lib().sspmm_batched_f16_f16,
+          torch.float32: _lib.lib().sspmm_batched_f16_f32}[out_dtype]
+    with torch.cuda.device(rhs_matrix.device):
+        rc = fn(batch, m_vec, vec_length, N, K, _ptr(row_indices), _ptr(row_offsets), _ptr(column_indices),
+                _ptr(values), nvec * vec_length, _ptr(rhs_matrix), K * N, _ptr(out), M * N, _stream())
+    _lib.check(rc, "sspmm_batched")
+    return out
+
+
+def sorted_row_swizzle(row_offsets):
+    """Vector-rows ordered by descending length (reference SortedRowSwizzle,
+    SSpMM/include/bm_test_utils.h:210-225), computed on the GPU."""
+    if row_offsets.dtype != torch.int32 or not row_offsets.is_cuda:
+        raise TypeError("row_offsets must be an int32 GPU tensor")
+    m_vec = row_offsets.numel() - 1
+    out = torch.empty(max(m_vec, 0), dtype=torch.int32, device=row_offsets.device)
+    with torch.cuda.device(row_offsets.device):
+        rc = _lib.lib().sspmm_sorted_row_swizzle(m_vec, _ptr(row_offsets), _ptr(out), _stream())
+    _lib.check(rc, "sspmm_sorted_row_swizzle")
+    return out

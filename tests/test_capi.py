@@ -1,0 +1,68 @@
+"""The C ABI library loads without a GPU, exports every symbol include/sspmm.h declares, and
+rejects bad arguments before touching the device."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "sspmm.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b((?:sspmm|svc)_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound(built_library):
+    from sspmm_amd import _lib
+    L = ctypes.CDLL(built_library)
+    names = _declared_symbols()
+    assert len(names) >= 10
+    for n in names:
+        assert hasattr(L, n), "library does not export %s" % n
+        assert n in _lib.SIGNATURES, "ctypes binding misses %s" % n
+    assert sorted(_lib.SIGNATURES) == names
+
+
+def test_argument_errors_without_device_work(built_library):
+    from sspmm_amd import _lib
+    L = _lib.lib()
+    assert L.sspmm_version() >= 1
+    one = 1  # any non-null pointer value; rejected calls never dereference it
+    # unsupported vector length (the reference prints and carries on: sspmm.cu:582-583)
+    assert L.sspmm_f16_f32(4, 4, 64, 64, None, one, one, one, one, one, None) == 1
+    assert L.sspmm_f16_f16(4, 2, 64, 64, None, one, one, one, one, one, None) == 1
+    # negative sizes, null outputs
+    assert L.sspmm_f16_f32(-1, 8, 64, 64, None, one, one, one, one, one, None) == 1
+    assert L.sspmm_f16_f32(4, 8, 64, 64, None, None, one, one, one, one, None) == 1
+    assert L.sspmm_f16_f32(4, 8, 64, 64, None, one, one, one, one, None, None) == 1
+    assert L.sspmm_f16_f32(4, 8, 1 << 20, 1 << 12, None, one, one, one, one, one, None) == 1  # K*N >= 2^31
+    # nothing to do is success
+    assert L.sspmm_f16_f32(0, 8, 64, 64, None, None, None, None, None, None, None) == 0
+    assert L.sspmm_f16_f16(4, 16, 0, 64, None, one, one, one, one, one, None) == 0
+    assert L.sspmm_batched_f16_f16(0, 4, 8, 64, 64, None, one, one, one, 0, one, 0, one, 0, None) == 0
+    assert L.sspmm_batched_f16_f16(2, 4, 8, 64, 64, None, one, one, one, 0, one, 0, one, 5, None) == 1  # C overlaps
+    assert L.sspmm_sorted_row_swizzle(-3, one, one, None) == 1
+    assert L.sspmm_sorted_row_swizzle(0, None, None, None) == 0
+    assert L.svc_count(8, 8, 8, one, one, 4, 7, one, one, None) == 1  # unknown order
+    assert L.svc_count(8, 8, 0, one, one, 4, 0, one, one, None) == 1  # V < 1
+    assert L.svc_count(8, 8, 8, one, one, 4, 0, one, None, None) == 1  # no workspace
+    assert L.svc_fill(8, 8, 8, one, one, one, 4, 0, one, one, one, None, None) == 1  # values in, no values out
+    assert L.svc_workspace_bytes(16, 100, 8) >= 100 * 8
+    assert b"invalid" in L.sspmm_error_string(1)
+    assert L.sspmm_error_string(0) == b"success"
+
+
+def test_python_operator_rejects_bad_arguments(built_library):
+    import torch
+    import sspmm_amd
+    t = torch.zeros(4, dtype=torch.int32)
+    h = torch.zeros(4, dtype=torch.float16)
+    with pytest.raises(ValueError):
+        sspmm_amd.spmm(None, t, t, h, h.reshape(2, 2), 4)
+    with pytest.raises(TypeError):
+        sspmm_amd.spmm(None, t.long(), t, h, h.reshape(2, 2), 8)
+    with pytest.raises(ValueError):  # CPU tensors: there is no CPU path
+        sspmm_amd.spmm(None, t, t, h, h.reshape(2, 2), 8)

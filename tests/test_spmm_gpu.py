@@ -1,0 +1,185 @@
+"""GPU parity of the SpMM through the C ABI (via the ctypes operator) against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+import sspmm_amd
+from sspmm_amd import synth
+from gpu_util import PARITY_TOL, TIGHT_F16, TIGHT_F32, dev, max_rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def run(vs, B, out_dtype, row_indices=None):
+    out = sspmm_amd.spmm(row_indices, dev(vs.row_offsets), dev(vs.col_idx), dev(vs.values), dev(B), vs.V,
+                         out_dtype=out_dtype)
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+def check(oracle, vs, B, out_dtype=torch.float32, row_indices=None):
+    K, N = B.shape
+    print("case M=%d K=%d N=%d V=%d nvec=%d out=%s" % (vs.M, K, N, vs.V, vs.col_idx.size, out_dtype), flush=True)
+    got = run(vs, B, out_dtype, row_indices)
+    want = oracle.spmm(vs.m_vec, vs.V, N, K, vs.row_offsets, vs.col_idx, vs.values, B, threads=8)
+    assert got.shape == (vs.m_vec * vs.V, N)
+    err = max_rel_err(got, want)
+    assert err <= PARITY_TOL, err
+    assert err <= (TIGHT_F32 if out_dtype == torch.float32 else TIGHT_F16), err
+    return got, want
+
+
+# BASELINE configs at their real shapes (the oracle runs each in well under a second with 8 threads)
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
+def test_cfg1_512x512_v8(oracle, built_library, out_dtype):
+    vs = synth.vector_sparse(512, 512, 8, 0.9, seed=1)
+    check(oracle, vs, synth.dense_rhs(512, 256, seed=11), out_dtype)
+
+
+@pytest.mark.parametrize("shape", [(2048, 512), (512, 2048)])
+@pytest.mark.parametrize("sparsity", [0.7, 0.9, 0.98])
+def test_cfg2_ffn_v8(oracle, built_library, shape, sparsity):
+    vs = synth.vector_sparse(shape[0], shape[1], 8, sparsity, seed=2, std=0.02)
+    check(oracle, vs, synth.dense_rhs(shape[1], 256, seed=12))
+
+
+@pytest.mark.parametrize("shape,sparsity,N", [((1024, 2304), 0.8, 256), ((2048, 1024), 0.95, 256),
+                                             ((1024, 2304), 0.95, 3136), ((2048, 1024), 0.8, 3136)])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
+def test_cfg3_conv_v16(oracle, built_library, shape, sparsity, N, out_dtype):
+    vs = synth.vector_sparse(shape[0], shape[1], 16, sparsity, seed=3, std=0.05)
+    check(oracle, vs, synth.dense_rhs(shape[1], N, seed=13), out_dtype)
+
+
+@pytest.mark.parametrize("V", [8, 16])
+@pytest.mark.parametrize("N", [8, 24, 64, 120, 128, 136, 200, 264])
+def test_column_tails(oracle, built_library, V, N):
+    """N that is not a multiple of the 128-column tile (the reference needs N % 64 == 0)."""
+    vs = synth.vector_sparse(6 * V, 80, V, 0.6, seed=20 + N)
+    check(oracle, vs, synth.dense_rhs(80, N, seed=N))
+
+
+@pytest.mark.parametrize("V", [8, 16])
+@pytest.mark.parametrize("N", [1, 3, 17, 66, 130])
+def test_odd_widths_take_the_generic_kernel_and_match_the_oracle_bit_for_bit(oracle, built_library, V, N):
+    """N % 8 != 0 runs the scalar kernel, which adds in the oracle's order: fp32 results are identical."""
+    vs = synth.vector_sparse(5 * V, 70, V, 0.5, seed=40 + N)
+    got, want = check(oracle, vs, synth.dense_rhs(70, N, seed=N))
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("V", [8, 16])
+@pytest.mark.parametrize("per_row", [0, 1, 7, 31, 32, 33, 63, 64, 65, 97])
+def test_row_length_tails(oracle, built_library, V, per_row):
+    """Vector-row lengths around the 32-vector step of the kernel."""
+    K = 128
+    rng = np.random.default_rng(per_row)
+    m_vec = 5
+    cols = np.concatenate([np.sort(rng.choice(K, per_row, replace=False)) for _ in range(m_vec)] or [[]]).astype(np.int32)
+    vs = synth.VectorSparse(m_vec * V, K, V, m_vec, (np.arange(m_vec + 1) * per_row).astype(np.int32), cols,
+                            rng.standard_normal(m_vec * per_row * V).astype(np.float16), m_vec * per_row * V)
+    check(oracle, vs, synth.dense_rhs(K, 128, seed=3))
+
+
+def test_ragged_rows_empty_rows_and_unsorted_columns(oracle, built_library):
+    rng = np.random.default_rng(77)
+    K, V, N = 300, 8, 256
+    lens = np.array([0, 5, 0, 0, 200, 33, 1, 0, 64, 0])
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cols = np.concatenate([rng.permutation(K)[:n] for n in lens]).astype(np.int32)  # not sorted
+    vs = synth.VectorSparse(len(lens) * V, K, V, len(lens), off, cols,
+                            rng.standard_normal(cols.size * V).astype(np.float16), cols.size * V)
+    B = synth.dense_rhs(K, N, seed=5)
+    got, want = check(oracle, vs, B)
+    for i in np.flatnonzero(lens == 0):
+        assert not got[i * V:(i + 1) * V].any()
+
+
+def test_inf_in_unreferenced_row_of_B_does_not_leak(oracle, built_library):
+    """Padding slots of a partial step must not multiply a real row of B."""
+    V, K, N = 8, 64, 128
+    vs = synth.vector_sparse(4 * V, K, V, 0.9, seed=9)  # 6 vectors per row, none is a full step
+    B = synth.dense_rhs(K, N, seed=9)
+    unused = sorted(set(range(K)) - set(vs.col_idx.tolist()))
+    B[unused] = np.inf
+    got = run(vs, B, torch.float32)
+    assert np.isfinite(got).all()
+
+
+def test_result_does_not_depend_on_row_indices(oracle, built_library):
+    vs = synth.vector_sparse(40 * 8, 256, 8, 0.85, seed=31)
+    B = synth.dense_rhs(256, 256, seed=32)
+    base = run(vs, B, torch.float32)
+    perm = np.random.default_rng(1).permutation(vs.m_vec).astype(np.int32)
+    assert np.array_equal(run(vs, B, torch.float32, dev(perm)), base)
+    swz = sspmm_amd.sorted_row_swizzle(dev(vs.row_offsets))
+    assert np.array_equal(run(vs, B, torch.float32, swz), base)
+
+
+def test_special_patterns(oracle, built_library):
+    V, K, N = 16, 32, 128
+    B = synth.dense_rhs(K, N, seed=6)
+    # one vector: outer product, exact
+    vals = np.arange(1, V + 1).astype(np.float16)
+    vs = synth.VectorSparse(V, K, V, 1, np.array([0, 1], np.int32), np.array([7], np.int32), vals, V)
+    got = run(vs, B, torch.float32)
+    assert np.array_equal(got, np.outer(vals.astype(np.float32), B[7].astype(np.float32)))
+    # identity-like pattern with ones: every row of slab i equals B[i]
+    m_vec = 8
+    vs = synth.VectorSparse(m_vec * V, K, V, m_vec, np.arange(m_vec + 1, dtype=np.int32),
+                            np.arange(m_vec, dtype=np.int32), np.ones(m_vec * V, np.float16), m_vec * V)
+    got = run(vs, B, torch.float16)
+    for i in range(m_vec):
+        assert np.array_equal(got[i * V:(i + 1) * V], np.tile(B[i], (V, 1)))
+
+
+def test_linearity_at_full_size(built_library):
+    """cfg3 at N = 3136 without the oracle: spmm(A, B1 + B2) == spmm(A, B1) + spmm(A, B2) when the
+    sums are exact (small integers), and scaling the values by 2 doubles the result exactly."""
+    V = 16
+    vs = synth.vector_sparse(1024, 2304, V, 0.8, seed=3)
+    rng = np.random.default_rng(0)
+    vals = rng.integers(-2, 3, vs.values.size).astype(np.float16)
+    vs = vs._replace(values=vals)
+    B1 = rng.integers(-3, 4, (2304, 3136)).astype(np.float16)
+    B2 = rng.integers(-3, 4, (2304, 3136)).astype(np.float16)
+    c1, c2, c12 = run(vs, B1, torch.float32), run(vs, B2, torch.float32), run(vs, B1 + B2, torch.float32)
+    assert np.array_equal(c12, c1 + c2)
+    c1d = run(vs._replace(values=vals * np.float16(2)), B1, torch.float32)
+    assert np.array_equal(c1d, 2 * c1)
+    # and against an exact dense integer matmul on a slab of rows
+    A = np.zeros((vs.m_vec * V, 2304), np.float32)
+    vv = vals.reshape(-1, V).astype(np.float32)
+    for i in range(4):
+        for j in range(vs.row_offsets[i], vs.row_offsets[i + 1]):
+            A[i * V:(i + 1) * V, vs.col_idx[j]] = vv[j]
+    assert np.array_equal(c1[:4 * V], A[:4 * V] @ B1.astype(np.float32))
+
+
+@pytest.mark.parametrize("V", [8, 16])
+@pytest.mark.parametrize("out_dtype", [torch.float16, torch.float32])
+def test_bspmm_matches_looped_spmm(oracle, built_library, V, out_dtype):
+    """Pattern shared by the batch, per-batch values / B / C (reference spmm_kernel.cu:532-534)."""
+    batch, K, N = 3, 96, 192
+    vs = synth.vector_sparse(12 * V, K, V, 0.75, seed=50)
+    rng = np.random.default_rng(51)
+    vals = rng.standard_normal((batch, vs.values.size)).astype(np.float16)
+    B = rng.standard_normal((batch, K, N)).astype(np.float16)
+    out = sspmm_amd.bspmm(None, dev(vs.row_offsets), dev(vs.col_idx), dev(vals), dev(B), V, out_dtype=out_dtype)
+    torch.cuda.synchronize()
+    out = out.cpu().numpy()
+    assert out.shape == (batch, vs.m_vec * V, N)
+    for b in range(batch):
+        single = run(vs._replace(values=vals[b]), B[b], out_dtype)
+        assert np.array_equal(out[b], single)
+        want = oracle.spmm(vs.m_vec, V, N, K, vs.row_offsets, vs.col_idx, vals[b], B[b])
+        assert max_rel_err(out[b], want) <= (TIGHT_F32 if out_dtype == torch.float32 else TIGHT_F16)
+
+
+def test_row_swizzle_matches_oracle(oracle, built_library):
+    rng = np.random.default_rng(3)
+    for m_vec in [1, 5, 255, 256, 257, 3000]:
+        lens = rng.integers(0, 50, m_vec)
+        off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        got = sspmm_amd.sorted_row_swizzle(dev(off)).cpu().numpy()
+        assert np.array_equal(got, oracle.sorted_row_swizzle(off))

@@ -1,0 +1,136 @@
+"""GPU parity of the SVC (RowMerge) through the C ABI: bit-exact against the files the reference
+wrote, the CPU oracle and the Python runtime's own set."""
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import sspmm_amd
+from sspmm_amd import formats, synth
+from gpu_util import dev
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+CASES = sorted(os.path.basename(p)[:-5] for p in glob.glob(os.path.join(GOLDEN, "*.smtx"))
+               if ".v" not in os.path.basename(p))
+
+
+def gpu_svc(M, K, V, row_ptr, col_ind, vals=None, order="cpython"):
+    r = sspmm_amd.svc(dev(row_ptr), dev(col_ind), None if vals is None else dev(vals), M, K, V, order=order)
+    torch.cuda.synchronize()
+    return (r.vec_row_ptr.cpu().numpy(), r.vec_col.cpu().numpy(),
+            None if r.vec_val is None else r.vec_val.cpu().numpy(), r.num_vec)
+
+
+@pytest.mark.parametrize("name", CASES)
+@pytest.mark.parametrize("V", [8, 16])
+def test_reference_files_byte_for_byte(built_library, name, V):
+    print("case", name, V, flush=True)
+    M, K, nnz, row_ptr, col_ind = formats.read_smtx(os.path.join(GOLDEN, name + ".smtx"))
+    vrp, vcol, _, nvec = gpu_svc(M, K, V, row_ptr, col_ind)
+    with open(os.path.join(GOLDEN, "%s.v%d.smtx" % (name, V))) as f:
+        want = f.read()
+    assert formats.cvse_text(len(vrp) - 1, K, nnz, vrp, vcol) == want
+    assert nvec == vcol.size
+
+
+def _compare_with_oracle(oracle, csr, V, order="cpython"):
+    print("case M=%d K=%d nnz=%d V=%d %s" % (csr.M, csr.K, csr.col_ind.size, V, order), flush=True)
+    vrp, vcol, vval, _ = gpu_svc(csr.M, csr.K, V, csr.row_ptr, csr.col_ind, csr.values, order)
+    wrp, wcol, wval = oracle.svc(csr.M, csr.K, V, csr.row_ptr, csr.col_ind, csr.values, order=order)
+    assert np.array_equal(vrp, wrp)
+    assert np.array_equal(vcol, wcol)
+    assert np.array_equal(vval.view(np.uint16), wval.view(np.uint16))
+    return vrp, vcol, vval
+
+
+def _random_csr(rng, M, K, max_len, sort=True):
+    lens = rng.integers(0, min(K, max_len) + 1, M)
+    ptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cols = np.concatenate([(np.sort if sort else (lambda x: x))(rng.permutation(K)[:n]) for n in lens] +
+                          [np.zeros(0, np.int64)]).astype(np.int32)
+    vals = rng.standard_normal(cols.size).astype(np.float16)
+    return synth.Csr(M, K, ptr, cols, vals)
+
+
+@pytest.mark.parametrize("V", [1, 3, 8, 16])
+@pytest.mark.parametrize("order", ["cpython", "sorted"])
+def test_random_small_matrices(oracle, built_library, V, order):
+    rng = np.random.default_rng(1000 + V)
+    for trial in range(6):
+        csr = _random_csr(rng, int(rng.integers(1, 90)), int(rng.choice([8, 33, 512, 5000])), 60, sort=bool(trial % 2))
+        _compare_with_oracle(oracle, csr, V, order)
+
+
+@pytest.mark.parametrize("V", [8, 16])
+def test_against_python_set_directly(oracle, built_library, V):
+    """The reference's one-line merge evaluated by the Python runtime itself."""
+    rng = np.random.default_rng(5)
+    csr = _random_csr(rng, 70, 3000, 120)
+    vrp, vcol, _, _ = gpu_svc(csr.M, csr.K, V, csr.row_ptr, csr.col_ind)
+    ptr, flat = oracle.rowmerge_python(csr.M, V, oracle.csr_col_lists(csr.M, csr.row_ptr, csr.col_ind))
+    assert vrp.tolist() == ptr and vcol.tolist() == flat
+
+
+@pytest.mark.parametrize("keys", [300, 310, 1200, 1240, 4800, 5000, 9000])
+def test_every_group_size_class(oracle, built_library, keys):
+    """Groups whose distinct-column bound falls into each kernel class (LDS 64 / 256 / 1024 threads,
+    and tables in the workspace), next to empty and tiny groups."""
+    rng = np.random.default_rng(keys)
+    V, K = 8, 40000
+    lens = np.zeros(40, np.int64)
+    lens[8:16] = keys // 8 + 1
+    lens[17] = 3
+    lens[24:27] = [keys // 2, 2, keys // 3]
+    ptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cols = np.concatenate([np.sort(rng.permutation(K)[:n]) for n in lens]).astype(np.int32)
+    csr = synth.Csr(40, K, ptr, cols, rng.standard_normal(cols.size).astype(np.float16))
+    _compare_with_oracle(oracle, csr, V)
+    _compare_with_oracle(oracle, csr, 16)
+
+
+def test_cfg1_rowmerge_returns_the_vector_pattern(oracle, built_library):
+    vs = synth.vector_sparse(512, 512, 8, 0.9, seed=1)
+    csr = synth.expand_to_csr(vs)
+    vrp, vcol, vval, _ = gpu_svc(csr.M, csr.K, 8, csr.row_ptr, csr.col_ind, csr.values, "sorted")
+    assert np.array_equal(vrp, vs.row_offsets) and np.array_equal(vcol, vs.col_idx)
+    assert np.array_equal(vval.view(np.uint16), vs.values.view(np.uint16))
+    _compare_with_oracle(oracle, csr, 8)
+
+
+def test_cfg4_zipf_16384(oracle, built_library):
+    csr = synth.zipf_csr(16384, 16384, seed=4)
+    vrp, vcol, vval = _compare_with_oracle(oracle, csr, 8)
+    # size-independent properties: densify(svc(A)) == A on sampled groups, nvec <= nnz, counts == distinct columns
+    assert vrp[-1] <= csr.col_ind.size
+    vv = vval.reshape(-1, 8)
+    for g in [0, 1, 777, 2047] + list(np.argsort(np.diff(vrp))[-2:]):
+        cols = vcol[vrp[g]:vrp[g + 1]]
+        assert len(set(cols.tolist())) == cols.size
+        for v in range(8):
+            r = g * 8 + v
+            b, e = csr.row_ptr[r], csr.row_ptr[r + 1]
+            where = {c: p for p, c in enumerate(cols.tolist())}
+            dense_row = np.zeros(cols.size, np.float16)
+            for c, x in zip(csr.col_ind[b:e].tolist(), csr.values[b:e]):
+                dense_row[where[c]] = x
+            assert np.array_equal(vv[vrp[g]:vrp[g + 1], v], dense_row)
+    _compare_with_oracle(oracle, csr, 16, "sorted")
+
+
+def test_svc_then_spmm_equals_csr_matmul(oracle, built_library):
+    """End of the pipe: unstructured CSR -> SVC (GPU) -> SpMM (GPU) == dense(A) @ B."""
+    rng = np.random.default_rng(8)
+    csr = _random_csr(rng, 128, 200, 30)
+    B = synth.dense_rhs(200, 64, seed=8)
+    r = sspmm_amd.svc(dev(csr.row_ptr), dev(csr.col_ind), dev(csr.values), csr.M, csr.K, 8)
+    out = sspmm_amd.spmm(None, r.vec_row_ptr, r.vec_col, r.vec_val, dev(B), 8, out_dtype=torch.float32)
+    torch.cuda.synchronize()
+    A = np.zeros((csr.M, csr.K), np.float64)
+    for i in range(csr.M):
+        A[i, csr.col_ind[csr.row_ptr[i]:csr.row_ptr[i + 1]]] = csr.values[csr.row_ptr[i]:csr.row_ptr[i + 1]]
+    want = A @ B.astype(np.float64)
+    assert np.abs(out.cpu().numpy() - want).max() <= 2e-5 * np.abs(want).max()

@@ -1,0 +1,231 @@
+#!/usr/bin/env python3
+"""Benchmark of the SVC -> SpMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Prints ONE JSON line.  A "step" is one pass of the SpMM over one batch of synthetic inputs
+already resident in HBM: the FFN-shaped configuration (A 2048x512 fp16, V=8, 90 % vector
+sparsity, B 512x256 fp16, C fp32), run bspmm-style over a batch of independent value / B / C
+sets that share the pattern, so that one launch moves more bytes than the last-level cache
+holds.  `value` is useful TFLOP/s = 2 * nnz * N * batch / t (the reference's convention,
+SSpMM/sspmm_test.cpp:197, with nnz the scalar non-zeros).
+
+`roofline` prices the SpMM kernel against the 8 TB/s HBM peak with the algorithmic bytes of one
+launch (every operand read once, C written once).  `cpu_baseline` times the CPU oracle (a port of
+the reference's host loop) on one batch element, single thread.  `extra` carries the other
+configurations (single launches, V=16 shapes, the SVC against the Python RowMerge, the dense GEMM
+comparator).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+HBM_PEAK_GBPS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--batch", type=int, default=128, help="independent value/B/C sets per step")
+    ap.add_argument("--quick", action="store_true", help="skip the extra configurations and CPU legs")
+    return ap.parse_args()
+
+
+def time_launches(fn, steps, warmup):
+    """Average milliseconds per call over `steps` calls, HIP events on the launch stream."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / steps
+
+
+def spmm_case(L, torch, synth, M, K, V, sparsity, N, batch, out_f32, std, seed, steps, warmup, dense=False):
+    """Times one SpMM configuration; returns a dict of figures."""
+    vs = synth.vector_sparse(M, K, V, sparsity, seed=seed, std=std)
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    ro = torch.from_numpy(vs.row_offsets).cuda()
+    ci = torch.from_numpy(vs.col_idx).cuda()
+    nv = vs.col_idx.size
+    vals = (torch.randn(batch, nv * V, generator=g, device="cuda") * std).half()
+    B = torch.randn(batch, K, N, generator=g, device="cuda").half()
+    C = torch.empty(batch, vs.m_vec * V, N, dtype=torch.float32 if out_f32 else torch.float16, device="cuda")
+    fn = L.sspmm_batched_f16_f32 if out_f32 else L.sspmm_batched_f16_f16
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def launch():
+        rc = fn(batch, vs.m_vec, V, N, K, None, ro.data_ptr(), ci.data_ptr(), vals.data_ptr(), nv * V, B.data_ptr(),
+                K * N, C.data_ptr(), vs.m_vec * V * N, stream)
+        if rc:
+            raise RuntimeError("sspmm failed: %d" % rc)
+
+    ms = time_launches(launch, steps, warmup)
+    bytes_alg = batch * synth.spmm_algorithmic_bytes(vs.m_vec, V, nv, K, N, 4 if out_f32 else 2) \
+        - (batch - 1) * (4 * nv + 4 * (vs.m_vec + 1))  # the pattern is shared by the batch
+    flops = 2.0 * vs.nnz * N * batch
+    out = {
+        "workload": "A %dx%d V=%d s=%.2f, B %dx%d, C %s, batch %d" % (M, K, V, sparsity, K, N,
+                                                                       "fp32" if out_f32 else "fp16", batch),
+        "ms": ms, "useful_tflops": flops / ms / 1e9, "alg_bytes": bytes_alg, "hbm_gbps": bytes_alg / ms / 1e6,
+        "hbm_frac": bytes_alg / ms / 1e6 / HBM_PEAK_GBPS,
+        "gather_bytes_no_reuse": batch * 2 * nv * N,
+    }
+    if dense:
+        A = torch.zeros(vs.m_vec * V, K, dtype=torch.float16, device="cuda")
+        Ad = A.unsqueeze(0).expand(batch, -1, -1).contiguous()
+        dms = time_launches(lambda: torch.bmm(Ad, B), max(10, steps // 4), 3)
+        out["dense_gemm_ms"] = dms
+        out["dense_gemm_effective_tflops"] = flops / dms / 1e9
+        out["speedup_vs_dense"] = dms / ms
+        del A, Ad
+    handles = (vs, vals, B, C)
+    return out, handles
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no multi-GPU leg (vector-rows shard without "
+              "communication); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    from sspmm_amd import _lib, synth
+    import sspmm_amd
+    L = _lib.lib()
+    torch.cuda.set_device(0)
+
+    M, K, V, sparsity, N = 2048, 512, 8, 0.9, 256
+    main_res, (vs, vals, B, C) = spmm_case(L, torch, synth, M, K, V, sparsity, N, args.batch, True, 0.02, 2,
+                                           args.steps, args.warmup, dense=not args.quick)
+    torch.cuda.synchronize()
+
+    # parity of batch element 0 against the CPU oracle, and the CPU baseline on the same element
+    cpu = None
+    parity = None
+    if not args.quick:
+        from oracle import oracle as O
+        O.build()
+        v0 = vals[0].cpu().numpy()
+        b0 = B[0].cpu().numpy()
+        t0 = time.perf_counter()
+        reps = 0
+        while True:
+            want = O.spmm(vs.m_vec, V, N, K, vs.row_offsets, vs.col_idx, v0, b0, threads=1)
+            reps += 1
+            if time.perf_counter() - t0 > 10.0 or reps >= 200:
+                break
+        cpu_s = (time.perf_counter() - t0) / reps
+        got = C[0].cpu().numpy()
+        parity = float(np.abs(got - want).max() / max(np.abs(want).max(), 1e-30))
+        ncores = os.cpu_count()
+        t0 = time.perf_counter()
+        O.spmm(vs.m_vec, V, N, K, vs.row_offsets, vs.col_idx, v0, b0, threads=min(ncores, 16))
+        cpu_mt_s = time.perf_counter() - t0
+        cpu = {"value": 2.0 * vs.nnz * N / cpu_s / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+               "sample": "%d repeats of one batch element (A 2048x512 V=8 s=0.9, B 512x256), host loop of "
+                         "sspmm_test.cpp:75-95 in C, -O2, single thread; %.1f ms each" % (reps, cpu_s * 1e3),
+               "all_cores_value": 2.0 * vs.nnz * N / cpu_mt_s / 1e12, "all_cores": min(ncores, 16),
+               "host_cpus": ncores}
+    del vals, B, C
+
+    extra = {}
+    if not args.quick:
+        st, wu = max(20, args.steps // 4), 5
+        cases = {
+            "cfg2_single_launch": dict(M=2048, K=512, V=8, sparsity=0.9, N=256, batch=1, out_f32=True, std=0.02, seed=2),
+            "cfg2_batched_fp16_out": dict(M=2048, K=512, V=8, sparsity=0.9, N=256, batch=args.batch, out_f32=False,
+                                          std=0.02, seed=2),
+            "cfg3_1024x2304_v16_s0.8_n3136": dict(M=1024, K=2304, V=16, sparsity=0.8, N=3136, batch=1, out_f32=True,
+                                                  std=0.05, seed=3),
+            "cfg3_2048x1024_v16_s0.95_n3136": dict(M=2048, K=1024, V=16, sparsity=0.95, N=3136, batch=1,
+                                                   out_f32=True, std=0.05, seed=3),
+            "cfg5_ffn1_3072x768_v16_s0.9_n4096": dict(M=3072, K=768, V=16, sparsity=0.9, N=4096, batch=1,
+                                                      out_f32=False, std=0.02, seed=5),
+            "cfg5_ffn2_768x3072_v16_s0.9_n4096": dict(M=768, K=3072, V=16, sparsity=0.9, N=4096, batch=1,
+                                                      out_f32=False, std=0.02, seed=5),
+            "cfg5_ffn1_batched8": dict(M=3072, K=768, V=16, sparsity=0.9, N=4096, batch=8, out_f32=False, std=0.02,
+                                       seed=5),
+        }
+        for name, kw in cases.items():
+            res, handles = spmm_case(L, torch, synth, steps=st, warmup=wu, dense=True, **kw)
+            del handles
+            torch.cuda.empty_cache()
+            extra[name] = res
+
+        # SVC: cfg4 (Zipf CSR 16384^2) on the GPU against the Python RowMerge and the C oracle
+        from oracle import oracle as O
+        csr = synth.zipf_csr(16384, 16384, seed=4)
+        rp, ci, cv = (torch.from_numpy(x).cuda() for x in (csr.row_ptr, csr.col_ind, csr.values))
+        r = sspmm_amd.svc(rp, ci, cv, csr.M, csr.K, 8)
+        torch.cuda.synchronize()
+        svc_ms = time_launches(lambda: sspmm_amd.svc(rp, ci, cv, csr.M, csr.K, 8), 20, 3)
+        # kernels only (no allocation, no host read-back)
+        ws = torch.empty(L.svc_workspace_bytes(csr.M, csr.col_ind.size, 8), dtype=torch.uint8, device="cuda")
+        vrp = torch.zeros(csr.M // 8 + 1, dtype=torch.int32, device="cuda")
+        vcol = torch.empty(r.num_vec, dtype=torch.int32, device="cuda")
+        vval = torch.empty(r.num_vec * 8, dtype=torch.float16, device="cuda")
+        stream = torch.cuda.current_stream().cuda_stream
+
+        def svc_kernels():
+            L.svc_count(csr.M, csr.K, 8, rp.data_ptr(), ci.data_ptr(), csr.col_ind.size, 0, vrp.data_ptr(),
+                        ws.data_ptr(), stream)
+            L.svc_fill(csr.M, csr.K, 8, rp.data_ptr(), ci.data_ptr(), cv.data_ptr(), csr.col_ind.size, 0,
+                       vrp.data_ptr(), ws.data_ptr(), vcol.data_ptr(), vval.data_ptr(), stream)
+
+        svc_k_ms = time_launches(svc_kernels, 20, 3)
+        lists = O.csr_col_lists(csr.M, csr.row_ptr, csr.col_ind)
+        t0 = time.perf_counter()
+        ptr, flat = O.rowmerge_python(csr.M, 8, lists)
+        py_ms = (time.perf_counter() - t0) * 1e3
+        t0 = time.perf_counter()
+        O.svc(csr.M, csr.K, 8, csr.row_ptr, csr.col_ind, csr.values)
+        c_ms = (time.perf_counter() - t0) * 1e3
+        same = (r.vec_row_ptr.cpu().numpy().tolist() == ptr) and (r.vec_col.cpu().numpy().tolist() == flat)
+        nnz = csr.col_ind.size
+        svc_bytes = synth.svc_algorithmic_bytes(csr.M, nnz, csr.M // 8, r.num_vec, 8)
+        extra["svc_cfg4_zipf_16384_v8"] = {
+            "gpu_ms_with_alloc_and_readback": svc_ms, "gpu_ms_kernels": svc_k_ms, "python_rowmerge_ms": py_ms,
+            "c_oracle_ms": c_ms, "speedup_vs_python": py_ms / svc_k_ms, "bit_exact_vs_python": bool(same),
+            "nnz": int(nnz), "nvec": int(r.num_vec), "fill_ratio": nnz / (r.num_vec * 8.0),
+            "max_vector_row": int(np.diff(r.vec_row_ptr.cpu().numpy()).max()),
+            "alg_bytes": svc_bytes, "hbm_gbps": svc_bytes / svc_k_ms / 1e6,
+        }
+
+    line = {
+        "metric": "SpMM useful TFLOP/s (2*nnz*N/t), V=8 @90% sparsity, fp16 in / fp32 accumulate",
+        "value": main_res["useful_tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": main_res["ms"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": main_res["workload"] + " (one launch, pattern shared by the batch)",
+                   "hbm_gbps": main_res["hbm_gbps"]},
+        "roofline": {"bound": "hbm", "achieved": main_res["hbm_gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": main_res["hbm_frac"], "traffic": None,
+                     "kernel": "spmm_gather_kernel<8,float>", "alg_bytes_per_launch": main_res["alg_bytes"]},
+        "cpu_baseline": cpu,
+        "parity_max_rel_err": parity,
+        "dense_gemm": {k: main_res[k] for k in main_res if k.startswith("dense") or k.startswith("speedup")},
+        "extra": extra,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

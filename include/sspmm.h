@@ -29,6 +29,14 @@ typedef uint16_t sspmm_half_t;
 /* Library version, (major << 16) | minor. */
 int sspmm_version(void);
 
+/*
+ * Testing and tuning hook without a counterpart in the reference: forces one SpMM kernel wherever
+ * its preconditions hold.  0 = automatic choice (default), 1 = scalar kernel (any shape),
+ * 2 = one-wave gather kernel, 3 = LDS-slab kernel.  Process-wide, not thread-safe.  Returns the
+ * previous setting, or -1 for an unknown value.
+ */
+int sspmm_select_kernel(int which);
+
 /* Static text for a return code of this library. */
 const char *sspmm_error_string(int code);
 

@@ -38,7 +38,7 @@ int spmm_entry(int batch, int m_vec, int V, int N, int K, const int32_t *row_ind
   a.stride_values = stride_values;
   a.stride_B = stride_B;
   a.stride_C = stride_C;
-  return (int)sspmm::launch_spmm(a, V, out_f16, /*force_generic=*/false, static_cast<hipStream_t>(stream));
+  return (int)sspmm::launch_spmm(a, V, out_f16, static_cast<hipStream_t>(stream));
 }
 
 }  // namespace
@@ -46,6 +46,11 @@ int spmm_entry(int batch, int m_vec, int V, int N, int K, const int32_t *row_ind
 extern "C" {
 
 int sspmm_version(void) { return (0 << 16) | 1; }
+
+int sspmm_select_kernel(int which) {
+  if (which < 0 || which > 3) return -1;
+  return sspmm::set_kernel_override(which);
+}
 
 const char *sspmm_error_string(int code) {
   if (code == 0) return "success";

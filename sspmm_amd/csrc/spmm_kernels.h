@@ -18,11 +18,17 @@ struct SpmmArgs {
   int64_t stride_values, stride_B, stride_C;  // per-batch strides in elements
   // filled by the launcher
   uint32_t n_tiles, total_work, per_xcd;
+  uint32_t n_slabs, row_blocks, rows_per_block;  // slab kernel
 };
 
-// V must be 8 or 16.  force_generic selects the shape-agnostic kernel even when the MFMA
-// kernel's alignment conditions hold (used by tests to cross-check the two).
-hipError_t launch_spmm(const SpmmArgs &args, int V, bool out_f16, bool force_generic, hipStream_t stream);
+// V must be 8 or 16.  Picks the kernel from the shape: the scalar kernel for widths or alignments
+// the MFMA kernels cannot take, the LDS-slab kernel when K is small and the problem is large,
+// the gather kernel otherwise.
+hipError_t launch_spmm(const SpmmArgs &args, int V, bool out_f16, hipStream_t stream);
+
+// Forces a kernel where its preconditions hold: 0 automatic, 1 scalar, 2 gather, 3 LDS slab.
+// Process-wide and not thread-safe: meant for tests and tuning.  Returns the previous value.
+int set_kernel_override(int which);
 
 hipError_t launch_sorted_row_swizzle(int m_vec, const int32_t *row_offsets, int32_t *row_indices,
                                      hipStream_t stream);

@@ -43,8 +43,14 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_srd(const void *base, uin
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, (int)kSrdWord3);
 }
 
-__device__ __forceinline__ uint32_t pack_lo(uint32_t x, uint32_t y) { return (x & 0xffffu) | (y << 16); }
-__device__ __forceinline__ uint32_t pack_hi(uint32_t x, uint32_t y) { return (x >> 16) | (y & 0xffff0000u); }
+// v_perm_b32 picks each result byte from the 8 bytes {y (bytes 4-7), x (bytes 0-3)}.
+// pack_lo = low half of x | low half of y << 16; pack_hi the same with the high halves.
+__device__ __forceinline__ uint32_t pack_lo(uint32_t x, uint32_t y) {
+  return __builtin_amdgcn_perm(y, x, 0x05040100u);
+}
+__device__ __forceinline__ uint32_t pack_hi(uint32_t x, uint32_t y) {
+  return __builtin_amdgcn_perm(y, x, 0x07060302u);
+}
 
 union Half8Bits {
   half8 h;
@@ -196,6 +202,189 @@ __global__ __launch_bounds__(64) void spmm_gather_kernel(const SpmmArgs p) {
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// Slab kernel: B resident in LDS.
+//
+// When K is small enough that a 64-column slab of B (K rows x 128 bytes) fits in the 160 KB of
+// LDS, a workgroup of 8 waves copies the slab into LDS once with coalesced 16-byte loads and
+// then walks a block of vector-rows against it: every gather of a row of B becomes a
+// ds_read_b64 (16 lanes read one 128-byte row segment, so the reads are bank-conflict free),
+// and HBM/L2 only see each slab once per row block, the value vectors, the column indices and
+// the stores of C.  Waves draw vector-rows from a counter in LDS, so ragged rows balance
+// inside the workgroup; the value/index loads of the next 32 vectors (possibly of the next
+// vector-row) are issued before the current 32 are contracted.  Row K of the slab is all
+// zeros: unused k slots of a partial step point there.
+static constexpr int kSlabWaves = 8;
+static constexpr int kSlabThreads = kSlabWaves * 64;
+static constexpr int kSlabRowBytes = 128;  // 64 columns of fp16
+
+struct SlabRegs {
+  uintx4 c0, c1;    // column indices of k slots 8g .. 8g+7
+  uint16_t a16[8];  // values[(k slot 8g+j), v = m]
+};
+
+template <int V>
+__device__ __forceinline__ void slab_issue(SlabRegs &r, int kc, int end, int g, const int32_t *col_idx,
+                                           const uint16_t *vals, uint32_t vals_lane_off) {
+  const __amdgpu_buffer_rsrc_t srd_cols = make_srd(col_idx, (uint32_t)end * 4u);
+  const __amdgpu_buffer_rsrc_t srd_vals = make_srd(vals, (uint32_t)end * (V * 2u));
+  const int kb = kc + 8 * g;
+  r.c0 = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_cols, kb * 4, 0, 0));
+  r.c1 = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_cols, kb * 4 + 16, 0, 0));
+  const uint32_t voff = (uint32_t)kb * (V * 2) + vals_lane_off;
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+    r.a16[j] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(srd_vals, voff + j * V * 2, 0, 0);
+}
+
+__device__ __forceinline__ void slab_mac(const SlabRegs &r, int kc, int end, int g, uint32_t zero_row,
+                                         const unsigned char *slab, uint32_t lane_byte, floatx4 (&acc)[4]) {
+  uint32_t col[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) col[j] = j < 4 ? r.c0[j] : r.c1[j - 4];
+  if (kc + 32 > end) {  // wave-uniform: partial step
+    const int kb = kc + 8 * g;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) col[j] = (kb + j < end) ? col[j] : zero_row;
+  }
+  uintx2 raw[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j)
+    raw[j] = *reinterpret_cast<const uintx2 *>(slab + col[j] * (uint32_t)kSlabRowBytes + lane_byte);
+  Half8Bits a;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) a.u[d] = (uint32_t)r.a16[2 * d] | ((uint32_t)r.a16[2 * d + 1] << 16);
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    Half8Bits b;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const uint32_t x = raw[2 * d][q >> 1], y = raw[2 * d + 1][q >> 1];
+      b.u[d] = (q & 1) ? pack_hi(x, y) : pack_lo(x, y);
+    }
+    acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a.h, b.h, acc[q], 0, 0, 0);
+  }
+}
+
+template <typename OutT>
+struct Store4;
+template <>
+struct Store4<float> {
+  static __device__ __forceinline__ void run(float *p, float a, float b, float c, float d) {
+    *reinterpret_cast<floatx4 *>(p) = floatx4{a, b, c, d};
+  }
+};
+template <>
+struct Store4<_Float16> {
+  typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+  static __device__ __forceinline__ void run(_Float16 *p, float a, float b, float c, float d) {
+    *reinterpret_cast<half4 *>(p) = half4{(_Float16)a, (_Float16)b, (_Float16)c, (_Float16)d};
+  }
+};
+
+template <int V, typename OutT>
+__global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs p) {
+  extern __shared__ __align__(16) unsigned char lds[];
+  const uint32_t id = blockIdx.x;
+  // Blocks that share a slab differ by multiples of 8 in their id: they land on one XCD and
+  // fetch the slab from the same L2.
+  const uint32_t slab_lo = id & 7u, qd = id >> 3;
+  const uint32_t rb = qd % p.row_blocks;
+  const uint32_t slab_id = (qd / p.row_blocks) * 8u + slab_lo;
+  if (slab_id >= p.n_slabs) return;
+  const uint32_t tile = slab_id % p.n_tiles, batch = slab_id / p.n_tiles;
+
+  const int tid = threadIdx.x, lane = tid & 63, m = lane & 15, g = lane >> 4;
+  const int n0 = (int)tile * 64;
+  const uint16_t *vals = p.values + (int64_t)batch * p.stride_values;
+  const uint16_t *bmat = p.B + (int64_t)batch * p.stride_B;
+  const uint32_t b_bytes = (uint32_t)p.K * (uint32_t)p.N * 2u;
+  const __amdgpu_buffer_rsrc_t srd_b = make_srd(bmat, b_bytes);
+
+  // ---- stage the slab: unit u = 16 bytes = columns n0 + 8*(u % 8) .. +7 of row u / 8
+  const uint32_t units = (uint32_t)p.K * 8u;
+  const uint32_t n2 = (uint32_t)p.N * 2u;
+  for (uint32_t u0 = 0; u0 < units; u0 += kSlabThreads * 8) {
+    uintx4 d[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t u = u0 + i * kSlabThreads + tid;
+      const uint32_t col = (uint32_t)n0 + (u & 7u) * 8u;
+      const uint32_t off = (u < units && col < (uint32_t)p.N) ? __umul24(u >> 3, n2) + col * 2u : b_bytes;
+      d[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_b, off, 0, 0));
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t u = u0 + i * kSlabThreads + tid;
+      if (u < units) *reinterpret_cast<uintx4 *>(lds + u * 16u) = d[i];
+    }
+  }
+  const uint32_t zero_row = (uint32_t)p.K;
+  if (tid < 8) *reinterpret_cast<uintx4 *>(lds + zero_row * kSlabRowBytes + tid * 16) = uintx4{0u, 0u, 0u, 0u};
+  int *counter = reinterpret_cast<int *>(lds + (zero_row + 1u) * kSlabRowBytes);
+  if (tid == 0) *counter = 0;
+  __syncthreads();
+
+  // ---- vector-rows of this block, drawn from the counter
+  const int row_lo = (int)(rb * p.rows_per_block);
+  const int row_hi = min(p.m_vec, row_lo + (int)p.rows_per_block);
+  auto grab = [&]() -> int {
+    int r = 0;
+    if (lane == 0) r = atomicAdd(counter, 1);
+    return __builtin_amdgcn_readfirstlane(r) + row_lo;
+  };
+  const uint32_t lane_byte = (uint32_t)m * 8u;
+  const uint32_t vals_lane_off = (uint32_t)m * 2u;
+  const int ncol = n0 + m * 4;
+  const bool col_ok = ncol < p.N;
+  OutT *cbase = reinterpret_cast<OutT *>(p.C) + (int64_t)batch * p.stride_C;
+
+  int r = grab();
+  if (r >= row_hi) return;
+  int row = p.row_indices ? p.row_indices[r] : r;
+  int kc = p.row_offsets[row], end = p.row_offsets[row + 1];
+  SlabRegs cur;
+  slab_issue<V>(cur, kc, end, g, p.col_idx, vals, vals_lane_off);
+  floatx4 acc[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  for (;;) {
+    int nrow = row, nkc = kc + 32, nend = end;
+    bool more = true;
+    if (nkc >= end) {
+      const int r2 = grab();
+      more = r2 < row_hi;
+      if (more) {
+        nrow = p.row_indices ? p.row_indices[r2] : r2;
+        nkc = p.row_offsets[nrow];
+        nend = p.row_offsets[nrow + 1];
+      }
+    }
+    SlabRegs nxt = cur;
+    if (more) slab_issue<V>(nxt, nkc, nend, g, p.col_idx, vals, vals_lane_off);
+    slab_mac(cur, kc, end, g, zero_row, lds, lane_byte, acc);
+    if (kc + 32 >= end) {
+      if (col_ok) {
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr) {
+          const int v = 4 * g + rr;
+          if (v < V)
+            Store4<OutT>::run(cbase + ((int64_t)row * V + v) * p.N + ncol, acc[0][rr], acc[1][rr], acc[2][rr],
+                              acc[3][rr]);
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+    if (!more) break;
+    row = nrow;
+    kc = nkc;
+    end = nend;
+    cur = nxt;
+  }
+}
+
 // Shape-agnostic kernel: any N, any alignment.  One thread per output column, scalar gathers,
 // accumulation in ascending vector order (the order of the reference's host check loop,
 // reference SSpMM/sspmm_test.cpp:82-94).
@@ -225,10 +414,47 @@ __global__ __launch_bounds__(64) void spmm_generic_kernel(const SpmmArgs p) {
   for (int v = 0; v < V; ++v) cbase[((int64_t)row * V + v) * p.N + n] = (OutT)acc[v];
 }
 
+static int g_kernel_override = 0;  // 0 auto, 1 generic, 2 gather, 3 slab (tests and tuning)
+
+int set_kernel_override(int which) {
+  const int old = g_kernel_override;
+  g_kernel_override = which;
+  return old;
+}
+
+static constexpr int kSlabMaxK = 1248;  // (K + 1) * 128 + 16 bytes must fit in 160 KB of LDS
+
 template <int V, typename OutT>
-static hipError_t launch_v(const SpmmArgs &a, bool fast, hipStream_t stream) {
+static hipError_t launch_slab(const SpmmArgs &a, hipStream_t stream) {
   SpmmArgs p = a;
-  if (fast) {
+  p.n_tiles = (uint32_t)((a.N + 63) / 64);
+  p.n_slabs = p.n_tiles * (uint32_t)a.batch;
+  // Aim at ~4 workgroups per CU, but keep at least 32 vector-rows per workgroup so that the copy
+  // of the slab into LDS stays a small part of the workgroup's traffic.
+  const uint32_t rb_target = p.n_slabs >= 1024u ? 1u : 1024u / p.n_slabs;
+  uint32_t rows = ((uint32_t)a.m_vec + rb_target - 1u) / rb_target;
+  if (rows < 32u) rows = 32u;
+  p.rows_per_block = rows;
+  p.row_blocks = ((uint32_t)a.m_vec + rows - 1u) / rows;
+  const size_t lds = (size_t)(a.K + 1) * kSlabRowBytes + 16;
+  auto kern = spmm_slab_kernel<V, OutT>;
+  static size_t lds_allowed = 64 * 1024;  // per instantiation
+  if (lds > lds_allowed) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e != hipSuccess) return e;
+    lds_allowed = 160 * 1024;
+  }
+  const uint32_t grid = ((p.n_slabs + 7u) / 8u) * 8u * p.row_blocks;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kSlabThreads), lds, stream, p);
+  return hipGetLastError();
+}
+
+template <int V, typename OutT>
+static hipError_t launch_v(const SpmmArgs &a, int which, hipStream_t stream) {
+  SpmmArgs p = a;
+  if (which == 3) return launch_slab<V, OutT>(a, stream);
+  if (which == 2) {
     p.n_tiles = (uint32_t)((a.N + 127) / 128);
     p.total_work = (uint32_t)a.m_vec * p.n_tiles * (uint32_t)a.batch;
     p.per_xcd = (p.total_work + 7u) / 8u;
@@ -242,17 +468,28 @@ static hipError_t launch_v(const SpmmArgs &a, bool fast, hipStream_t stream) {
   return hipGetLastError();
 }
 
-hipError_t launch_spmm(const SpmmArgs &a, int V, bool out_f16, bool force_generic, hipStream_t stream) {
-  // The MFMA kernel needs 16-byte row segments of B and C: N % 8 == 0 and aligned bases/strides;
+hipError_t launch_spmm(const SpmmArgs &a, int V, bool out_f16, hipStream_t stream) {
+  // The MFMA kernels need 16-byte row segments of B and C: N % 8 == 0 and aligned bases/strides;
   // 24-bit multiplies bound K and 2N; one buffer descriptor must span B.
   const uint64_t b_bytes = (uint64_t)a.K * (uint64_t)a.N * 2u;
   const int out_size = out_f16 ? 2 : 4;
-  bool fast = !force_generic && (a.N % 8 == 0) && (reinterpret_cast<uintptr_t>(a.B) % 16 == 0) &&
-              (reinterpret_cast<uintptr_t>(a.C) % 16 == 0) && (a.stride_B % 8 == 0) &&
-              ((a.stride_C * out_size) % 16 == 0) && (a.K < (1 << 24)) && (a.N < (1 << 23)) &&
-              (b_bytes + 16 <= 0xffffffffull);
-  if (V == 8) return out_f16 ? launch_v<8, _Float16>(a, fast, stream) : launch_v<8, float>(a, fast, stream);
-  return out_f16 ? launch_v<16, _Float16>(a, fast, stream) : launch_v<16, float>(a, fast, stream);
+  const bool fast = (a.N % 8 == 0) && (reinterpret_cast<uintptr_t>(a.B) % 16 == 0) &&
+                    (reinterpret_cast<uintptr_t>(a.C) % 16 == 0) && (a.stride_B % 8 == 0) &&
+                    ((a.stride_C * out_size) % 16 == 0) && (a.K < (1 << 24)) && (a.N < (1 << 23)) &&
+                    (b_bytes + 16 <= 0xffffffffull);
+  int which = 1;
+  if (fast) {
+    // The slab kernel pays off when enough vector-rows share a slab and there are enough
+    // workgroups to fill the chip; otherwise one wave per (vector-row, 128 columns).
+    const uint64_t slabs = (uint64_t)((a.N + 63) / 64) * (uint64_t)a.batch;
+    const uint64_t blocks = slabs * (uint64_t)((a.m_vec + 31) / 32);
+    which = (a.K <= kSlabMaxK && a.m_vec >= 64 && blocks >= 1024) ? 3 : 2;
+    if (g_kernel_override == 2) which = 2;
+    if (g_kernel_override == 3 && a.K <= kSlabMaxK) which = 3;
+  }
+  if (g_kernel_override == 1) which = 1;
+  if (V == 8) return out_f16 ? launch_v<8, _Float16>(a, which, stream) : launch_v<8, float>(a, which, stream);
+  return out_f16 ? launch_v<16, _Float16>(a, which, stream) : launch_v<16, float>(a, which, stream);
 }
 
 }  // namespace sspmm

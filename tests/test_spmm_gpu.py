@@ -9,6 +9,17 @@ from gpu_util import PARITY_TOL, TIGHT_F16, TIGHT_F32, dev, max_rel_err
 
 pytestmark = pytest.mark.gpu
 
+KERNELS = {"auto": 0, "gather": 2, "slab": 3}
+
+
+@pytest.fixture(params=sorted(KERNELS))
+def kernel(request, built_library):
+    """Runs the test once per SpMM kernel (the automatic choice, and each MFMA kernel forced)."""
+    from sspmm_amd import _lib
+    _lib.lib().sspmm_select_kernel(KERNELS[request.param])
+    yield request.param
+    _lib.lib().sspmm_select_kernel(0)
+
 
 def run(vs, B, out_dtype, row_indices=None):
     out = sspmm_amd.spmm(row_indices, dev(vs.row_offsets), dev(vs.col_idx), dev(vs.values), dev(B), vs.V,
@@ -31,14 +42,14 @@ def check(oracle, vs, B, out_dtype=torch.float32, row_indices=None):
 
 # BASELINE configs at their real shapes (the oracle runs each in well under a second with 8 threads)
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
-def test_cfg1_512x512_v8(oracle, built_library, out_dtype):
+def test_cfg1_512x512_v8(oracle, kernel, out_dtype):
     vs = synth.vector_sparse(512, 512, 8, 0.9, seed=1)
     check(oracle, vs, synth.dense_rhs(512, 256, seed=11), out_dtype)
 
 
 @pytest.mark.parametrize("shape", [(2048, 512), (512, 2048)])
 @pytest.mark.parametrize("sparsity", [0.7, 0.9, 0.98])
-def test_cfg2_ffn_v8(oracle, built_library, shape, sparsity):
+def test_cfg2_ffn_v8(oracle, kernel, shape, sparsity):
     vs = synth.vector_sparse(shape[0], shape[1], 8, sparsity, seed=2, std=0.02)
     check(oracle, vs, synth.dense_rhs(shape[1], 256, seed=12))
 
@@ -53,7 +64,7 @@ def test_cfg3_conv_v16(oracle, built_library, shape, sparsity, N, out_dtype):
 
 @pytest.mark.parametrize("V", [8, 16])
 @pytest.mark.parametrize("N", [8, 24, 64, 120, 128, 136, 200, 264])
-def test_column_tails(oracle, built_library, V, N):
+def test_column_tails(oracle, kernel, V, N):
     """N that is not a multiple of the 128-column tile (the reference needs N % 64 == 0)."""
     vs = synth.vector_sparse(6 * V, 80, V, 0.6, seed=20 + N)
     check(oracle, vs, synth.dense_rhs(80, N, seed=N))
@@ -70,7 +81,7 @@ def test_odd_widths_take_the_generic_kernel_and_match_the_oracle_bit_for_bit(ora
 
 @pytest.mark.parametrize("V", [8, 16])
 @pytest.mark.parametrize("per_row", [0, 1, 7, 31, 32, 33, 63, 64, 65, 97])
-def test_row_length_tails(oracle, built_library, V, per_row):
+def test_row_length_tails(oracle, kernel, V, per_row):
     """Vector-row lengths around the 32-vector step of the kernel."""
     K = 128
     rng = np.random.default_rng(per_row)
@@ -81,7 +92,7 @@ def test_row_length_tails(oracle, built_library, V, per_row):
     check(oracle, vs, synth.dense_rhs(K, 128, seed=3))
 
 
-def test_ragged_rows_empty_rows_and_unsorted_columns(oracle, built_library):
+def test_ragged_rows_empty_rows_and_unsorted_columns(oracle, kernel):
     rng = np.random.default_rng(77)
     K, V, N = 300, 8, 256
     lens = np.array([0, 5, 0, 0, 200, 33, 1, 0, 64, 0])
@@ -95,7 +106,7 @@ def test_ragged_rows_empty_rows_and_unsorted_columns(oracle, built_library):
         assert not got[i * V:(i + 1) * V].any()
 
 
-def test_inf_in_unreferenced_row_of_B_does_not_leak(oracle, built_library):
+def test_inf_in_unreferenced_row_of_B_does_not_leak(oracle, kernel):
     """Padding slots of a partial step must not multiply a real row of B."""
     V, K, N = 8, 64, 128
     vs = synth.vector_sparse(4 * V, K, V, 0.9, seed=9)  # 6 vectors per row, none is a full step
@@ -106,7 +117,7 @@ def test_inf_in_unreferenced_row_of_B_does_not_leak(oracle, built_library):
     assert np.isfinite(got).all()
 
 
-def test_result_does_not_depend_on_row_indices(oracle, built_library):
+def test_result_does_not_depend_on_row_indices(oracle, kernel):
     vs = synth.vector_sparse(40 * 8, 256, 8, 0.85, seed=31)
     B = synth.dense_rhs(256, 256, seed=32)
     base = run(vs, B, torch.float32)
@@ -116,7 +127,7 @@ def test_result_does_not_depend_on_row_indices(oracle, built_library):
     assert np.array_equal(run(vs, B, torch.float32, swz), base)
 
 
-def test_special_patterns(oracle, built_library):
+def test_special_patterns(oracle, kernel):
     V, K, N = 16, 32, 128
     B = synth.dense_rhs(K, N, seed=6)
     # one vector: outer product, exact
@@ -131,6 +142,25 @@ def test_special_patterns(oracle, built_library):
     got = run(vs, B, torch.float16)
     for i in range(m_vec):
         assert np.array_equal(got[i * V:(i + 1) * V], np.tile(B[i], (V, 1)))
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
+def test_slab_kernel_at_k1024_v16(oracle, kernel, out_dtype):
+    vs = synth.vector_sparse(2048, 1024, 16, 0.95, seed=3, std=0.05)
+    check(oracle, vs, synth.dense_rhs(1024, 448, seed=14), out_dtype)
+
+
+def test_skewed_row_lengths(oracle, kernel):
+    """A few very long vector-rows among short ones (what the row counter in the slab kernel balances)."""
+    rng = np.random.default_rng(123)
+    K, V, N, m_vec = 1000, 8, 192, 96
+    lens = rng.integers(0, 20, m_vec)
+    lens[[3, 40, 95]] = [1000, 700, 333]
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cols = np.concatenate([rng.permutation(K)[:n] for n in lens]).astype(np.int32)
+    vs = synth.VectorSparse(m_vec * V, K, V, m_vec, off, cols,
+                            rng.standard_normal(cols.size * V).astype(np.float16), cols.size * V)
+    check(oracle, vs, synth.dense_rhs(K, N, seed=15))
 
 
 def test_linearity_at_full_size(built_library):
@@ -158,7 +188,7 @@ def test_linearity_at_full_size(built_library):
 
 @pytest.mark.parametrize("V", [8, 16])
 @pytest.mark.parametrize("out_dtype", [torch.float16, torch.float32])
-def test_bspmm_matches_looped_spmm(oracle, built_library, V, out_dtype):
+def test_bspmm_matches_looped_spmm(oracle, kernel, V, out_dtype):
     """Pattern shared by the batch, per-batch values / B / C (reference spmm_kernel.cu:532-534)."""
     batch, K, N = 3, 96, 192
     vs = synth.vector_sparse(12 * V, K, V, 0.75, seed=50)

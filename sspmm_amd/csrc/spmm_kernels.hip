@@ -203,87 +203,98 @@ __global__ __launch_bounds__(64) void spmm_gather_kernel(const SpmmArgs p) {
 }
 
 // ------------------------------------------------------------------------------------------
-// Slab kernel: B resident in LDS.
+// Slab kernel: B resident in LDS, operands formed by LDS transpose reads.
 //
 // When K is small enough that a 64-column slab of B (K rows x 128 bytes) fits in the 160 KB of
 // LDS, a workgroup of 8 waves copies the slab into LDS once with coalesced 16-byte loads and
-// then walks a block of vector-rows against it: every gather of a row of B becomes a
-// ds_read_b64 (16 lanes read one 128-byte row segment, so the reads are bank-conflict free),
-// and HBM/L2 only see each slab once per row block, the value vectors, the column indices and
-// the stores of C.  Waves draw vector-rows from a counter in LDS, so ragged rows balance
-// inside the workgroup; the value/index loads of the next 32 vectors (possibly of the next
-// vector-row) are issued before the current 32 are contracted.  Row K of the slab is all
-// zeros: unused k slots of a partial step point there.
+// then walks a block of vector-rows against it, so HBM/L2 only see each slab once per row
+// block, the value vectors, the column indices and the stores of C.
+//
+// ds_read_b64_tr_b16 is what makes this cheap.  Within 16 lanes, lane n receives element n of the
+// four 32-byte runs addressed by lanes 0-3, 4-7, 8-11, 12-15: four rows that are contiguous in the
+// column direction come back as "four k of one column", which is the MFMA operand layout.  Per
+// step of 32 vectors a wave therefore issues
+//   * 2 transpose reads of its value tile (32 vectors x V halfs, written to LDS with one
+//     16-byte store per lane from one coalesced 16-byte global load per lane), and
+//   * 8 transpose reads of the slab (two k halves x four 16-column tiles), addressed by just
+//     two column indices per lane,
+// and 4 MFMAs, with no byte shuffling in registers.  A 16-lane group of a slab read touches four
+// different rows of B at the same column offset; the 32-byte segments of slab row c are stored
+// XOR-swizzled by (c >> 1) & 3 so that those rows spread over the LDS banks.
+// Waves draw vector-rows from a counter in LDS, so ragged rows balance inside the workgroup, and
+// the loads of a step are issued two steps ahead (across vector-row boundaries).  Row K of the
+// slab is all zeros: unused k slots of a partial step point there.
 static constexpr int kSlabWaves = 8;
 static constexpr int kSlabThreads = kSlabWaves * 64;
-static constexpr int kSlabRowBytes = 128;  // 64 columns of fp16
+static constexpr int kSlabRowBytes = 128;       // 64 columns of fp16
+static constexpr int kValTileBytes = 1024 + 64;  // 32 vectors x 32 B, plus slack for the V = 8 over-read
 
-struct SlabRegs {
-  uintx4 c0, c1;    // column indices of k slots 8g .. 8g+7
-  uint16_t a16[8];  // values[(k slot 8g+j), v = m]
+typedef short shortx4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) shortx4 lds_shortx4;
+
+__device__ __forceinline__ uintx2 lds_read_tr(const unsigned char *lds_base, uint32_t byte_off) {
+  const shortx4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4 *)(lds_base + byte_off));
+  return __builtin_bit_cast(uintx2, v);
+}
+
+struct SlabDesc {  // one step: 32 vectors [kc, kc + 32) of vector-row `row`, which ends at `end`
+  int row, kc, end;
+  bool valid;
 };
 
 template <int V>
-__device__ __forceinline__ void slab_issue(SlabRegs &r, int kc, int end, int g, const int32_t *col_idx,
-                                           const uint16_t *vals, uint32_t vals_lane_off) {
-  const __amdgpu_buffer_rsrc_t srd_cols = make_srd(col_idx, (uint32_t)end * 4u);
-  const __amdgpu_buffer_rsrc_t srd_vals = make_srd(vals, (uint32_t)end * (V * 2u));
-  const int kb = kc + 8 * g;
-  r.c0 = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_cols, kb * 4, 0, 0));
-  r.c1 = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_cols, kb * 4 + 16, 0, 0));
-  const uint32_t voff = (uint32_t)kb * (V * 2) + vals_lane_off;
-#pragma unroll
-  for (int j = 0; j < 8; ++j)
-    r.a16[j] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(srd_vals, voff + j * V * 2, 0, 0);
-}
+struct SlabVals;  // the 32 x V halfs of a step, spread over the 64 lanes
+template <>
+struct SlabVals<8> {
+  typedef uintx2 type;  // 8 bytes per lane
+  static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t srd, uint32_t off) {
+    return __builtin_bit_cast(uintx2, __builtin_amdgcn_raw_buffer_load_b64(srd, off, 0, 0));
+  }
+};
+template <>
+struct SlabVals<16> {
+  typedef uintx4 type;  // 16 bytes per lane
+  static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t srd, uint32_t off) {
+    return __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd, off, 0, 0));
+  }
+};
 
-__device__ __forceinline__ void slab_mac(const SlabRegs &r, int kc, int end, int g, uint32_t zero_row,
-                                         const unsigned char *slab, uint32_t lane_byte, floatx4 (&acc)[4]) {
-  uint32_t col[8];
-#pragma unroll
-  for (int j = 0; j < 8; ++j) col[j] = j < 4 ? r.c0[j] : r.c1[j - 4];
-  if (kc + 32 > end) {  // wave-uniform: partial step
-    const int kb = kc + 8 * g;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) col[j] = (kb + j < end) ? col[j] : zero_row;
-  }
-  uintx2 raw[8];
-#pragma unroll
-  for (int j = 0; j < 8; ++j)
-    raw[j] = *reinterpret_cast<const uintx2 *>(slab + col[j] * (uint32_t)kSlabRowBytes + lane_byte);
-  Half8Bits a;
-#pragma unroll
-  for (int d = 0; d < 4; ++d) a.u[d] = (uint32_t)r.a16[2 * d] | ((uint32_t)r.a16[2 * d + 1] << 16);
-#pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    Half8Bits b;
-#pragma unroll
-    for (int d = 0; d < 4; ++d) {
-      const uint32_t x = raw[2 * d][q >> 1], y = raw[2 * d + 1][q >> 1];
-      b.u[d] = (q & 1) ? pack_hi(x, y) : pack_lo(x, y);
-    }
-    acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a.h, b.h, acc[q], 0, 0, 0);
-  }
+template <int V>
+struct SlabLoads {
+  uint32_t col[2];  // column index of k slots 8g + m/4 and 8g + 4 + m/4
+  typename SlabVals<V>::type vraw;
+};
+
+template <int V>
+__device__ __forceinline__ void slab_issue(SlabLoads<V> &r, const SlabDesc &d, int lane, uint32_t slot0,
+                                           __amdgpu_buffer_rsrc_t srd_cols, const uint16_t *vals) {
+  r.col[0] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(srd_cols, (d.kc + (int)slot0) * 4, 0, 0);
+  r.col[1] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(srd_cols, (d.kc + (int)slot0) * 4 + 16, 0, 0);
+  // The value descriptor ends with the vector-row: vectors past it read as zero.
+  const __amdgpu_buffer_rsrc_t srd_vals = make_srd(vals, (uint32_t)d.end * (V * 2u));
+  constexpr uint32_t kLaneBytes = V * 2u * 32u / 64u;
+  r.vraw = SlabVals<V>::load(srd_vals, (uint32_t)d.kc * (V * 2u) + (uint32_t)lane * kLaneBytes);
 }
 
 template <typename OutT>
-struct Store4;
+struct StoreCol;  // one output element
 template <>
-struct Store4<float> {
-  static __device__ __forceinline__ void run(float *p, float a, float b, float c, float d) {
-    *reinterpret_cast<floatx4 *>(p) = floatx4{a, b, c, d};
-  }
+struct StoreCol<float> {
+  static __device__ __forceinline__ void run(unsigned char *p, float a) { *reinterpret_cast<float *>(p) = a; }
 };
 template <>
-struct Store4<_Float16> {
-  typedef _Float16 half4 __attribute__((ext_vector_type(4)));
-  static __device__ __forceinline__ void run(_Float16 *p, float a, float b, float c, float d) {
-    *reinterpret_cast<half4 *>(p) = half4{(_Float16)a, (_Float16)b, (_Float16)c, (_Float16)d};
+struct StoreCol<_Float16> {
+  static __device__ __forceinline__ void run(unsigned char *p, float a) {
+    *reinterpret_cast<_Float16 *>(p) = (_Float16)a;
   }
 };
 
+static constexpr int kSlabRing = 8;  // steps whose loads are in flight or waiting in registers
+
 template <int V, typename OutT>
-__global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs p) {
+__global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs p,
+                                                                 const int32_t *__restrict__ row_offsets,
+                                                                 const int32_t *__restrict__ row_indices) {
   extern __shared__ __align__(16) unsigned char lds[];
   const uint32_t id = blockIdx.x;
   // Blocks that share a slab differ by multiples of 8 in their id: they land on one XCD and
@@ -294,14 +305,15 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
   if (slab_id >= p.n_slabs) return;
   const uint32_t tile = slab_id % p.n_tiles, batch = slab_id / p.n_tiles;
 
-  const int tid = threadIdx.x, lane = tid & 63, m = lane & 15, g = lane >> 4;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, m = lane & 15, g = lane >> 4;
   const int n0 = (int)tile * 64;
   const uint16_t *vals = p.values + (int64_t)batch * p.stride_values;
   const uint16_t *bmat = p.B + (int64_t)batch * p.stride_B;
   const uint32_t b_bytes = (uint32_t)p.K * (uint32_t)p.N * 2u;
   const __amdgpu_buffer_rsrc_t srd_b = make_srd(bmat, b_bytes);
 
-  // ---- stage the slab: unit u = 16 bytes = columns n0 + 8*(u % 8) .. +7 of row u / 8
+  // ---- stage the slab: unit u = 16 bytes = columns n0 + 8*(u % 8) .. +7 of row u / 8; the
+  // 32-byte segment (u % 8) / 2 of row c lands at segment ((u % 8) / 2) ^ ((c >> 1) & 3).
   const uint32_t units = (uint32_t)p.K * 8u;
   const uint32_t n2 = (uint32_t)p.N * 2u;
   for (uint32_t u0 = 0; u0 < units; u0 += kSlabThreads * 8) {
@@ -316,72 +328,156 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const uint32_t u = u0 + i * kSlabThreads + tid;
-      if (u < units) *reinterpret_cast<uintx4 *>(lds + u * 16u) = d[i];
+      const uint32_t c = u >> 3;
+      const uint32_t dst = c * kSlabRowBytes + (((u & 7u) * 16u) ^ (((c >> 1) & 3u) << 5));
+      if (u < units) *reinterpret_cast<uintx4 *>(lds + dst) = d[i];
     }
   }
   const uint32_t zero_row = (uint32_t)p.K;
   if (tid < 8) *reinterpret_cast<uintx4 *>(lds + zero_row * kSlabRowBytes + tid * 16) = uintx4{0u, 0u, 0u, 0u};
-  int *counter = reinterpret_cast<int *>(lds + (zero_row + 1u) * kSlabRowBytes);
+  const uint32_t tiles_off = (zero_row + 1u) * kSlabRowBytes;
+  int *counter = reinterpret_cast<int *>(lds + tiles_off + kSlabWaves * kValTileBytes);
   if (tid == 0) *counter = 0;
   __syncthreads();
 
-  // ---- vector-rows of this block, drawn from the counter
+  // ---- per-lane constants
+  unsigned char *val_tile = lds + tiles_off + wave * kValTileBytes;
+  constexpr uint32_t kLaneBytes = V * 2u * 32u / 64u;
+  unsigned char *val_dst = val_tile + lane * kLaneBytes;
+  // value tile rows are V*2 bytes; transpose read h picks rows 8g + 4h + m/4
+  const uint32_t a_off = (uint32_t)(8 * g + (m >> 2)) * (V * 2u) + (uint32_t)(m & 3) * 8u;
+  const uint32_t slot0 = (uint32_t)(8 * g + (m >> 2));
+  const uint32_t b_lane_off = (uint32_t)(m & 3) * 8u;
+  // accumulator q of lane (m, g) holds rows 4g .. 4g+3 of column n0 + 16q + m
+  uint32_t c_lane_off[4];
+  bool c_ok[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const int ncol = n0 + 16 * q + m;
+    c_ok[q] = ncol < p.N;
+    c_lane_off[q] = ((uint32_t)(4 * g) * (uint32_t)p.N + (uint32_t)ncol) * (uint32_t)sizeof(OutT);
+  }
+  const uint32_t c_row_stride = (uint32_t)p.N * (uint32_t)sizeof(OutT);
+  unsigned char *cbase = reinterpret_cast<unsigned char *>(reinterpret_cast<OutT *>(p.C) + (int64_t)batch * p.stride_C);
+  const int64_t c_vrow_bytes = (int64_t)V * p.N * (int64_t)sizeof(OutT);
+  // Row bookkeeping is read through the restrict-qualified kernel arguments so that it goes
+  // through the scalar cache and does not share the vector-memory counter with the stores of C.
+  const uint32_t nvec = (uint32_t)row_offsets[p.m_vec];
+  const __amdgpu_buffer_rsrc_t srd_cols = make_srd(p.col_idx, nvec * 4u);
+
+  // ---- this wave's stream of steps
   const int row_lo = (int)(rb * p.rows_per_block);
   const int row_hi = min(p.m_vec, row_lo + (int)p.rows_per_block);
+  const bool permuted = row_indices != nullptr;
   auto grab = [&]() -> int {
     int r = 0;
     if (lane == 0) r = atomicAdd(counter, 1);
     return __builtin_amdgcn_readfirstlane(r) + row_lo;
   };
-  const uint32_t lane_byte = (uint32_t)m * 8u;
-  const uint32_t vals_lane_off = (uint32_t)m * 2u;
-  const int ncol = n0 + m * 4;
-  const bool col_ok = ncol < p.N;
-  OutT *cbase = reinterpret_cast<OutT *>(p.C) + (int64_t)batch * p.stride_C;
+  // The next vector-row of this wave is fetched one row ahead of its use.
+  SlabDesc ahead;
+  auto fetch_ahead = [&]() {
+    const int r = grab();
+    ahead.valid = r < row_hi;
+    ahead.row = 0;
+    ahead.kc = 0;
+    ahead.end = 0;
+    if (ahead.valid) {
+      ahead.row = permuted ? row_indices[r] : r;
+      ahead.kc = row_offsets[ahead.row];
+      ahead.end = row_offsets[ahead.row + 1];
+    }
+  };
+  auto successor = [&](const SlabDesc &d) -> SlabDesc {
+    SlabDesc n = d;
+    if (d.valid) {
+      n.kc = d.kc + 32;
+      if (n.kc >= d.end) {
+        n = ahead;
+        if (ahead.valid) fetch_ahead();
+      }
+    }
+    return n;
+  };
 
-  int r = grab();
-  if (r >= row_hi) return;
-  int row = p.row_indices ? p.row_indices[r] : r;
-  int kc = p.row_offsets[row], end = p.row_offsets[row + 1];
-  SlabRegs cur;
-  slab_issue<V>(cur, kc, end, g, p.col_idx, vals, vals_lane_off);
+  fetch_ahead();
+  if (!ahead.valid) return;
+  SlabDesc dd[kSlabRing];
+  SlabLoads<V> ld[kSlabRing];
+  dd[0] = ahead;
+  fetch_ahead();
+  slab_issue<V>(ld[0], dd[0], lane, slot0, srd_cols, vals);
+#pragma unroll
+  for (int i = 1; i < kSlabRing - 1; ++i) {
+    dd[i] = successor(dd[i - 1]);
+    if (dd[i].valid) slab_issue<V>(ld[i], dd[i], lane, slot0, srd_cols, vals);
+  }
+  // the value tile of the first step
+  *reinterpret_cast<typename SlabVals<V>::type *>(val_dst) = ld[0].vraw;
+
   floatx4 acc[4];
-#pragma unroll
-  for (int q = 0; q < 4; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
-
+  bool first = true;  // first step of a vector-row: accumulate onto zero
   for (;;) {
-    int nrow = row, nkc = kc + 32, nend = end;
-    bool more = true;
-    if (nkc >= end) {
-      const int r2 = grab();
-      more = r2 < row_hi;
-      if (more) {
-        nrow = p.row_indices ? p.row_indices[r2] : r2;
-        nkc = p.row_offsets[nrow];
-        nend = p.row_offsets[nrow + 1];
-      }
-    }
-    SlabRegs nxt = cur;
-    if (more) slab_issue<V>(nxt, nkc, nend, g, p.col_idx, vals, vals_lane_off);
-    slab_mac(cur, kc, end, g, zero_row, lds, lane_byte, acc);
-    if (kc + 32 >= end) {
-      if (col_ok) {
 #pragma unroll
-        for (int rr = 0; rr < 4; ++rr) {
-          const int v = 4 * g + rr;
-          if (v < V)
-            Store4<OutT>::run(cbase + ((int64_t)row * V + v) * p.N + ncol, acc[0][rr], acc[1][rr], acc[2][rr],
-                              acc[3][rr]);
+    for (int u = 0; u < kSlabRing; ++u) {
+      constexpr int R = kSlabRing;
+      const int cur = u, nxt = (u + 1) % R, newest = (u + R - 2) % R, fill = (u + R - 1) % R;
+      dd[fill] = successor(dd[newest]);
+      if (dd[fill].valid) slab_issue<V>(ld[fill], dd[fill], lane, slot0, srd_cols, vals);
+      const SlabDesc d0 = dd[cur];
+
+      // A operand: this step's value tile
+      Half8Bits a;
+      {
+        const uintx2 lo = lds_read_tr(val_tile, a_off);
+        const uintx2 hi = lds_read_tr(val_tile, a_off + 4u * (V * 2u));
+        a.u[0] = lo[0]; a.u[1] = lo[1]; a.u[2] = hi[0]; a.u[3] = hi[1];
+      }
+      // B operands: two column indices per lane
+      uint32_t addr[2];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        uint32_t c = ld[cur].col[h];
+        if (d0.kc + 32 > d0.end) c = (d0.kc + (int)slot0 + 4 * h < d0.end) ? c : zero_row;  // partial step
+        const uint32_t t = c << 4;
+        addr[h] = (t << 3) | ((t & 0x60u) | b_lane_off);
+      }
+      Half8Bits b[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const uintx2 lo = lds_read_tr(lds, addr[0] ^ ((uint32_t)q << 5));
+        const uintx2 hi = lds_read_tr(lds, addr[1] ^ ((uint32_t)q << 5));
+        b[q].u[0] = lo[0]; b[q].u[1] = lo[1]; b[q].u[2] = hi[0]; b[q].u[3] = hi[1];
+      }
+      // the next step's value tile goes to LDS behind the reads above (LDS operations of a wave
+      // execute in order)
+      if (dd[nxt].valid) *reinterpret_cast<typename SlabVals<V>::type *>(val_dst) = ld[nxt].vraw;
+
+      if (first) {
+        const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a.h, b[q].h, zero, 0, 0, 0);
+      } else {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a.h, b[q].h, acc[q], 0, 0, 0);
+      }
+      first = false;
+      if (d0.kc + 32 >= d0.end) {  // last step of the vector-row: write its V x 64 tile of C
+        unsigned char *crow = cbase + (int64_t)d0.row * c_vrow_bytes;
+        if (4 * g < V) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            if (c_ok[q]) {
+#pragma unroll
+              for (int rr = 0; rr < 4; ++rr)
+                StoreCol<OutT>::run(crow + c_lane_off[q] + rr * c_row_stride, acc[q][rr]);
+            }
+          }
         }
+        first = true;
       }
-#pragma unroll
-      for (int q = 0; q < 4; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
+      if (!dd[nxt].valid) return;
     }
-    if (!more) break;
-    row = nrow;
-    kc = nkc;
-    end = nend;
-    cur = nxt;
   }
 }
 
@@ -422,7 +518,7 @@ int set_kernel_override(int which) {
   return old;
 }
 
-static constexpr int kSlabMaxK = 1248;  // (K + 1) * 128 + 16 bytes must fit in 160 KB of LDS
+static constexpr int kSlabMaxK = 1200;  // slab + zero row + 8 value tiles must fit in 160 KB of LDS
 
 template <int V, typename OutT>
 static hipError_t launch_slab(const SpmmArgs &a, hipStream_t stream) {
@@ -436,7 +532,7 @@ static hipError_t launch_slab(const SpmmArgs &a, hipStream_t stream) {
   if (rows < 32u) rows = 32u;
   p.rows_per_block = rows;
   p.row_blocks = ((uint32_t)a.m_vec + rows - 1u) / rows;
-  const size_t lds = (size_t)(a.K + 1) * kSlabRowBytes + 16;
+  const size_t lds = (size_t)(a.K + 1) * kSlabRowBytes + kSlabWaves * kValTileBytes + 16;
   auto kern = spmm_slab_kernel<V, OutT>;
   static size_t lds_allowed = 64 * 1024;  // per instantiation
   if (lds > lds_allowed) {
@@ -446,7 +542,7 @@ static hipError_t launch_slab(const SpmmArgs &a, hipStream_t stream) {
     lds_allowed = 160 * 1024;
   }
   const uint32_t grid = ((p.n_slabs + 7u) / 8u) * 8u * p.row_blocks;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(kSlabThreads), lds, stream, p);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kSlabThreads), lds, stream, p, a.row_offsets, a.row_indices);
   return hipGetLastError();
 }
 

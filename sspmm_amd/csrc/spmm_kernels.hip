@@ -227,7 +227,15 @@ __global__ __launch_bounds__(64) void spmm_gather_kernel(const SpmmArgs p) {
 static constexpr int kSlabWaves = 8;
 static constexpr int kSlabThreads = kSlabWaves * 64;
 static constexpr int kSlabRowBytes = 128;       // 64 columns of fp16
-static constexpr int kValTileBytes = 1024 + 64;  // 32 vectors x 32 B, plus slack for the V = 8 over-read
+// Per-wave LDS: the value tile of a step (32 vectors x V halfs; the V = 8 transpose read touches 16
+// bytes past its 512) and a staging tile of 8 rows x 128 bytes (+16 bytes of padding per row)
+// through which finished tiles of C are turned into row-contiguous 16-byte stores.
+static constexpr int val_tile_bytes(int V) { return V == 8 ? 528 : 1024; }
+static constexpr int kStageStride = 144;
+static constexpr int kStageBytes = 8 * kStageStride;
+static constexpr int wave_lds_bytes(int V) { return val_tile_bytes(V) + kStageBytes; }
+
+static constexpr int kSlabRing = 8;  // steps whose loads are in flight or waiting in registers
 
 typedef short shortx4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) shortx4 lds_shortx4;
@@ -236,11 +244,6 @@ __device__ __forceinline__ uintx2 lds_read_tr(const unsigned char *lds_base, uin
   const shortx4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4 *)(lds_base + byte_off));
   return __builtin_bit_cast(uintx2, v);
 }
-
-struct SlabDesc {  // one step: 32 vectors [kc, kc + 32) of vector-row `row`, which ends at `end`
-  int row, kc, end;
-  bool valid;
-};
 
 template <int V>
 struct SlabVals;  // the 32 x V halfs of a step, spread over the 64 lanes
@@ -265,31 +268,71 @@ struct SlabLoads {
   typename SlabVals<V>::type vraw;
 };
 
+// Walks one wave's sequence of steps: wave w of a row block takes the block's vector-rows
+// w, w + 8, w + 16, ...; a vector-row of n vectors is ceil(n / 32) steps, and an empty vector-row is
+// one step without vectors (its zeros still have to be written).  The offsets of the following
+// vector-row are requested one row ahead so that the scalar loads are off the critical path.
+// Two cursors run over the same sequence: one issues the loads of a step, the other, kSlabRing - 1
+// steps behind it, consumes them.
+struct SlabCursor {
+  int pos;                       // position of the current vector-row in the row block
+  int row, kc, end;              // current step: vectors [kc, min(kc + 32, end)) of vector-row `row`
+  bool valid;
+  int next_row, next_kc, next_end;
+  bool next_valid;
+};
+
+__device__ __forceinline__ void cursor_prefetch(SlabCursor &c, int pos, int row_hi,
+                                                const int32_t *__restrict__ row_offsets,
+                                                const int32_t *__restrict__ row_indices) {
+  c.next_valid = pos < row_hi;
+  c.next_row = c.next_kc = c.next_end = 0;
+  if (c.next_valid) {
+    c.next_row = row_indices ? row_indices[pos] : pos;
+    c.next_kc = row_offsets[c.next_row];
+    c.next_end = row_offsets[c.next_row + 1];
+  }
+}
+
+__device__ __forceinline__ void cursor_take_next(SlabCursor &c, int row_hi, const int32_t *__restrict__ row_offsets,
+                                                 const int32_t *__restrict__ row_indices) {
+  c.pos += kSlabWaves;
+  c.row = c.next_row;
+  c.kc = c.next_kc;
+  c.end = c.next_end;
+  c.valid = c.next_valid;
+  if (c.valid) cursor_prefetch(c, c.pos + kSlabWaves, row_hi, row_offsets, row_indices);
+}
+
+__device__ __forceinline__ void cursor_advance(SlabCursor &c, int row_hi, const int32_t *__restrict__ row_offsets,
+                                               const int32_t *__restrict__ row_indices) {
+  c.kc += 32;
+  if (c.kc >= c.end) cursor_take_next(c, row_hi, row_offsets, row_indices);
+}
+
 template <int V>
-__device__ __forceinline__ void slab_issue(SlabLoads<V> &r, const SlabDesc &d, int lane, uint32_t slot0,
+__device__ __forceinline__ void slab_issue(SlabLoads<V> &r, int kc, int end, int lane, uint32_t slot0,
                                            __amdgpu_buffer_rsrc_t srd_cols, const uint16_t *vals) {
-  r.col[0] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(srd_cols, (d.kc + (int)slot0) * 4, 0, 0);
-  r.col[1] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(srd_cols, (d.kc + (int)slot0) * 4 + 16, 0, 0);
+  r.col[0] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(srd_cols, (kc + (int)slot0) * 4, 0, 0);
+  r.col[1] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(srd_cols, (kc + (int)slot0) * 4 + 16, 0, 0);
   // The value descriptor ends with the vector-row: vectors past it read as zero.
-  const __amdgpu_buffer_rsrc_t srd_vals = make_srd(vals, (uint32_t)d.end * (V * 2u));
+  const __amdgpu_buffer_rsrc_t srd_vals = make_srd(vals, (uint32_t)end * (V * 2u));
   constexpr uint32_t kLaneBytes = V * 2u * 32u / 64u;
-  r.vraw = SlabVals<V>::load(srd_vals, (uint32_t)d.kc * (V * 2u) + (uint32_t)lane * kLaneBytes);
+  r.vraw = SlabVals<V>::load(srd_vals, (uint32_t)kc * (V * 2u) + (uint32_t)lane * kLaneBytes);
 }
 
 template <typename OutT>
-struct StoreCol;  // one output element
+struct StageElem;  // writes one accumulator element into the staging tile in the output type
 template <>
-struct StoreCol<float> {
-  static __device__ __forceinline__ void run(unsigned char *p, float a) { *reinterpret_cast<float *>(p) = a; }
+struct StageElem<float> {
+  static __device__ __forceinline__ void put(unsigned char *p, float a) { *reinterpret_cast<float *>(p) = a; }
 };
 template <>
-struct StoreCol<_Float16> {
-  static __device__ __forceinline__ void run(unsigned char *p, float a) {
-    *reinterpret_cast<_Float16 *>(p) = (_Float16)a;
+struct StageElem<_Float16> {
+  static __device__ __forceinline__ void put(unsigned char *p, float a) {
+    *reinterpret_cast<_Float16 *>(p) = (_Float16)a;  // round to nearest even
   }
 };
-
-static constexpr int kSlabRing = 8;  // steps whose loads are in flight or waiting in registers
 
 template <int V, typename OutT>
 __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs p,
@@ -305,7 +348,8 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
   if (slab_id >= p.n_slabs) return;
   const uint32_t tile = slab_id % p.n_tiles, batch = slab_id / p.n_tiles;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, m = lane & 15, g = lane >> 4;
+  const int tid = threadIdx.x, lane = tid & 63, m = lane & 15, g = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // tell the compiler it is wave-uniform
   const int n0 = (int)tile * 64;
   const uint16_t *vals = p.values + (int64_t)batch * p.stride_values;
   const uint16_t *bmat = p.B + (int64_t)batch * p.stride_B;
@@ -336,30 +380,36 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
   const uint32_t zero_row = (uint32_t)p.K;
   if (tid < 8) *reinterpret_cast<uintx4 *>(lds + zero_row * kSlabRowBytes + tid * 16) = uintx4{0u, 0u, 0u, 0u};
   const uint32_t tiles_off = (zero_row + 1u) * kSlabRowBytes;
-  int *counter = reinterpret_cast<int *>(lds + tiles_off + kSlabWaves * kValTileBytes);
-  if (tid == 0) *counter = 0;
   __syncthreads();
 
   // ---- per-lane constants
-  unsigned char *val_tile = lds + tiles_off + wave * kValTileBytes;
+  unsigned char *val_tile = lds + tiles_off + wave * wave_lds_bytes(V);
+  unsigned char *stage = val_tile + val_tile_bytes(V);
   constexpr uint32_t kLaneBytes = V * 2u * 32u / 64u;
   unsigned char *val_dst = val_tile + lane * kLaneBytes;
   // value tile rows are V*2 bytes; transpose read h picks rows 8g + 4h + m/4
   const uint32_t a_off = (uint32_t)(8 * g + (m >> 2)) * (V * 2u) + (uint32_t)(m & 3) * 8u;
   const uint32_t slot0 = (uint32_t)(8 * g + (m >> 2));
   const uint32_t b_lane_off = (uint32_t)(m & 3) * 8u;
-  // accumulator q of lane (m, g) holds rows 4g .. 4g+3 of column n0 + 16q + m
-  uint32_t c_lane_off[4];
-  bool c_ok[4];
+  // Accumulator q of lane (m, g) holds rows 4g .. 4g+3 of column n0 + 16q + m.  A finished tile goes
+  // to C in passes of 8 rows x 128 bytes: the lanes owning those rows write their elements into the
+  // staging tile, then every lane reads 16 contiguous bytes of one row and stores them, so a store
+  // instruction writes eight full 128-byte lines.
+  constexpr int kColsPerPass = 128 / (int)sizeof(OutT);  // 32 fp32 or 64 fp16 columns
+  constexpr int kTilesPerPass = kColsPerPass / 16;        // accumulators per pass
+  constexpr int kPasses = 64 / kColsPerPass;
+  unsigned char *stage_w = stage + (4 * (g & 1)) * kStageStride + m * (int)sizeof(OutT);
+  const unsigned char *stage_r = stage + (lane >> 3) * kStageStride + (lane & 7) * 16;
+  const uint32_t c_voff = ((uint32_t)(lane >> 3) * (uint32_t)p.N + (uint32_t)n0) * (uint32_t)sizeof(OutT) +
+                          (uint32_t)(lane & 7) * 16u;
+  bool pass_ok[kPasses];
 #pragma unroll
-  for (int q = 0; q < 4; ++q) {
-    const int ncol = n0 + 16 * q + m;
-    c_ok[q] = ncol < p.N;
-    c_lane_off[q] = ((uint32_t)(4 * g) * (uint32_t)p.N + (uint32_t)ncol) * (uint32_t)sizeof(OutT);
-  }
-  const uint32_t c_row_stride = (uint32_t)p.N * (uint32_t)sizeof(OutT);
-  unsigned char *cbase = reinterpret_cast<unsigned char *>(reinterpret_cast<OutT *>(p.C) + (int64_t)batch * p.stride_C);
-  const int64_t c_vrow_bytes = (int64_t)V * p.N * (int64_t)sizeof(OutT);
+  for (int ps = 0; ps < kPasses; ++ps)
+    pass_ok[ps] = n0 + ps * kColsPerPass + (lane & 7) * (16 / (int)sizeof(OutT)) < p.N;
+  // One buffer descriptor spans this batch element's C (the launcher checks it is below 4 GiB).
+  const uint32_t c_vrow_bytes = (uint32_t)V * (uint32_t)p.N * (uint32_t)sizeof(OutT);
+  const __amdgpu_buffer_rsrc_t srd_c = make_srd(reinterpret_cast<OutT *>(p.C) + (int64_t)batch * p.stride_C,
+                                                (uint32_t)p.m_vec * c_vrow_bytes);
   // Row bookkeeping is read through the restrict-qualified kernel arguments so that it goes
   // through the scalar cache and does not share the vector-memory counter with the stores of C.
   const uint32_t nvec = (uint32_t)row_offsets[p.m_vec];
@@ -368,49 +418,20 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
   // ---- this wave's stream of steps
   const int row_lo = (int)(rb * p.rows_per_block);
   const int row_hi = min(p.m_vec, row_lo + (int)p.rows_per_block);
-  const bool permuted = row_indices != nullptr;
-  auto grab = [&]() -> int {
-    int r = 0;
-    if (lane == 0) r = atomicAdd(counter, 1);
-    return __builtin_amdgcn_readfirstlane(r) + row_lo;
-  };
-  // The next vector-row of this wave is fetched one row ahead of its use.
-  SlabDesc ahead;
-  auto fetch_ahead = [&]() {
-    const int r = grab();
-    ahead.valid = r < row_hi;
-    ahead.row = 0;
-    ahead.kc = 0;
-    ahead.end = 0;
-    if (ahead.valid) {
-      ahead.row = permuted ? row_indices[r] : r;
-      ahead.kc = row_offsets[ahead.row];
-      ahead.end = row_offsets[ahead.row + 1];
-    }
-  };
-  auto successor = [&](const SlabDesc &d) -> SlabDesc {
-    SlabDesc n = d;
-    if (d.valid) {
-      n.kc = d.kc + 32;
-      if (n.kc >= d.end) {
-        n = ahead;
-        if (ahead.valid) fetch_ahead();
-      }
-    }
-    return n;
-  };
+  SlabCursor head;  // issues loads
+  head.pos = row_lo + wave - kSlabWaves;
+  cursor_prefetch(head, row_lo + wave, row_hi, row_offsets, row_indices);
+  cursor_take_next(head, row_hi, row_offsets, row_indices);
+  if (!head.valid) return;
+  SlabCursor tail = head;  // consumes them
 
-  fetch_ahead();
-  if (!ahead.valid) return;
-  SlabDesc dd[kSlabRing];
   SlabLoads<V> ld[kSlabRing];
-  dd[0] = ahead;
-  fetch_ahead();
-  slab_issue<V>(ld[0], dd[0], lane, slot0, srd_cols, vals);
 #pragma unroll
-  for (int i = 1; i < kSlabRing - 1; ++i) {
-    dd[i] = successor(dd[i - 1]);
-    if (dd[i].valid) slab_issue<V>(ld[i], dd[i], lane, slot0, srd_cols, vals);
+  for (int i = 0; i < kSlabRing - 1; ++i) {
+    if (head.valid) {
+      slab_issue<V>(ld[i], head.kc, head.end, lane, slot0, srd_cols, vals);
+      cursor_advance(head, row_hi, row_offsets, row_indices);
+    }
   }
   // the value tile of the first step
   *reinterpret_cast<typename SlabVals<V>::type *>(val_dst) = ld[0].vraw;
@@ -421,10 +442,14 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
 #pragma unroll
     for (int u = 0; u < kSlabRing; ++u) {
       constexpr int R = kSlabRing;
-      const int cur = u, nxt = (u + 1) % R, newest = (u + R - 2) % R, fill = (u + R - 1) % R;
-      dd[fill] = successor(dd[newest]);
-      if (dd[fill].valid) slab_issue<V>(ld[fill], dd[fill], lane, slot0, srd_cols, vals);
-      const SlabDesc d0 = dd[cur];
+      const int cur = u, nxt = (u + 1) % R, fill = (u + R - 1) % R;
+      if (head.valid) {
+        slab_issue<V>(ld[fill], head.kc, head.end, lane, slot0, srd_cols, vals);
+        cursor_advance(head, row_hi, row_offsets, row_indices);
+      }
+      const int row = tail.row;
+      const int left = tail.end - tail.kc;  // vectors of this vector-row from this step on
+      cursor_advance(tail, row_hi, row_offsets, row_indices);
 
       // A operand: this step's value tile
       Half8Bits a;
@@ -433,12 +458,11 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
         const uintx2 hi = lds_read_tr(val_tile, a_off + 4u * (V * 2u));
         a.u[0] = lo[0]; a.u[1] = lo[1]; a.u[2] = hi[0]; a.u[3] = hi[1];
       }
-      // B operands: two column indices per lane
+      // B operands: two column indices per lane; unused k slots of a partial step read the zero row
       uint32_t addr[2];
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        uint32_t c = ld[cur].col[h];
-        if (d0.kc + 32 > d0.end) c = (d0.kc + (int)slot0 + 4 * h < d0.end) ? c : zero_row;  // partial step
+        const uint32_t c = ((int)slot0 + 4 * h < left) ? ld[cur].col[h] : zero_row;
         const uint32_t t = c << 4;
         addr[h] = (t << 3) | ((t & 0x60u) | b_lane_off);
       }
@@ -451,7 +475,7 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
       }
       // the next step's value tile goes to LDS behind the reads above (LDS operations of a wave
       // execute in order)
-      if (dd[nxt].valid) *reinterpret_cast<typename SlabVals<V>::type *>(val_dst) = ld[nxt].vraw;
+      if (tail.valid) *reinterpret_cast<typename SlabVals<V>::type *>(val_dst) = ld[nxt].vraw;
 
       if (first) {
         const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
@@ -461,22 +485,29 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
 #pragma unroll
         for (int q = 0; q < 4; ++q) acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a.h, b[q].h, acc[q], 0, 0, 0);
       }
-      first = false;
-      if (d0.kc + 32 >= d0.end) {  // last step of the vector-row: write its V x 64 tile of C
-        unsigned char *crow = cbase + (int64_t)d0.row * c_vrow_bytes;
-        if (4 * g < V) {
+      first = left <= 32;
+      if (first) {  // last step of the vector-row: write its V x 64 tile of C
+        const uint32_t crow = (uint32_t)row * c_vrow_bytes;
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            if (c_ok[q]) {
+        for (int vh = 0; vh < V / 8; ++vh) {
 #pragma unroll
-              for (int rr = 0; rr < 4; ++rr)
-                StoreCol<OutT>::run(crow + c_lane_off[q] + rr * c_row_stride, acc[q][rr]);
+          for (int ps = 0; ps < kPasses; ++ps) {
+            if ((g >> 1) == vh) {
+#pragma unroll
+              for (int qi = 0; qi < kTilesPerPass; ++qi)
+#pragma unroll
+                for (int rr = 0; rr < 4; ++rr)
+                  StageElem<OutT>::put(stage_w + rr * kStageStride + qi * 16 * (int)sizeof(OutT),
+                                       acc[ps * kTilesPerPass + qi][rr]);
             }
+            const uintx4 line = *reinterpret_cast<const uintx4 *>(stage_r);
+            if (pass_ok[ps])
+              __builtin_amdgcn_raw_buffer_store_b128(line, srd_c, c_voff + ps * 128,
+                                                     crow + (uint32_t)vh * 8u * (uint32_t)p.N * (uint32_t)sizeof(OutT), 0);
           }
         }
-        first = true;
       }
-      if (!dd[nxt].valid) return;
+      if (!tail.valid) return;
     }
   }
 }
@@ -518,7 +549,7 @@ int set_kernel_override(int which) {
   return old;
 }
 
-static constexpr int kSlabMaxK = 1200;  // slab + zero row + 8 value tiles must fit in 160 KB of LDS
+static constexpr int kSlabMaxK = 1136;  // slab + zero row + 8 x (value tile + staging tile) must fit in 160 KB of LDS
 
 template <int V, typename OutT>
 static hipError_t launch_slab(const SpmmArgs &a, hipStream_t stream) {
@@ -532,7 +563,7 @@ static hipError_t launch_slab(const SpmmArgs &a, hipStream_t stream) {
   if (rows < 32u) rows = 32u;
   p.rows_per_block = rows;
   p.row_blocks = ((uint32_t)a.m_vec + rows - 1u) / rows;
-  const size_t lds = (size_t)(a.K + 1) * kSlabRowBytes + kSlabWaves * kValTileBytes + 16;
+  const size_t lds = (size_t)(a.K + 1) * kSlabRowBytes + kSlabWaves * wave_lds_bytes(V);
   auto kern = spmm_slab_kernel<V, OutT>;
   static size_t lds_allowed = 64 * 1024;  // per instantiation
   if (lds > lds_allowed) {
@@ -579,9 +610,11 @@ hipError_t launch_spmm(const SpmmArgs &a, int V, bool out_f16, hipStream_t strea
     // workgroups to fill the chip; otherwise one wave per (vector-row, 128 columns).
     const uint64_t slabs = (uint64_t)((a.N + 63) / 64) * (uint64_t)a.batch;
     const uint64_t blocks = slabs * (uint64_t)((a.m_vec + 31) / 32);
-    which = (a.K <= kSlabMaxK && a.m_vec >= 64 && blocks >= 1024) ? 3 : 2;
+    // The slab kernel addresses one batch element's C through a 32-bit buffer descriptor.
+    const bool slab_ok = a.K <= kSlabMaxK && (uint64_t)a.m_vec * (V == 8 ? 8u : 16u) * (uint64_t)a.N * out_size < 0xffffffffull;
+    which = (slab_ok && a.m_vec >= 64 && blocks >= 1024) ? 3 : 2;
     if (g_kernel_override == 2) which = 2;
-    if (g_kernel_override == 3 && a.K <= kSlabMaxK) which = 3;
+    if (g_kernel_override == 3 && slab_ok) which = 3;
   }
   if (g_kernel_override == 1) which = 1;
   if (V == 8) return out_f16 ? launch_v<8, _Float16>(a, which, stream) : launch_v<8, float>(a, which, stream);

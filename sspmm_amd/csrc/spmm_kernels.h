@@ -18,7 +18,7 @@ struct SpmmArgs {
   int64_t stride_values, stride_B, stride_C;  // per-batch strides in elements
   // filled by the launcher
   uint32_t n_tiles, total_work, per_xcd;
-  uint32_t n_slabs, row_blocks, rows_per_block;  // slab kernel
+  uint32_t n_slabs, row_blocks, rows_per_block, group_by_batch;  // slab kernel
 };
 
 // V must be 8 or 16.  Picks the kernel from the shape: the scalar kernel for widths or alignments

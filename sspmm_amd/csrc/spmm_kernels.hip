@@ -268,46 +268,67 @@ struct SlabLoads {
   typename SlabVals<V>::type vraw;
 };
 
-// Walks one wave's sequence of steps: wave w of a row block takes the block's vector-rows
-// w, w + 8, w + 16, ...; a vector-row of n vectors is ceil(n / 32) steps, and an empty vector-row is
-// one step without vectors (its zeros still have to be written).  The offsets of the following
-// vector-row are requested one row ahead so that the scalar loads are off the critical path.
-// Two cursors run over the same sequence: one issues the loads of a step, the other, kSlabRing - 1
-// steps behind it, consumes them.
+// Walks one wave's sequence of steps.  Waves draw the vector-rows of their row block from a counter
+// in LDS, so ragged rows and uneven memory latency balance inside the workgroup; a vector-row of n
+// vectors is ceil(n / 32) steps, and an empty vector-row is one step without vectors (its zeros
+// still have to be written).  Two cursors run over the same sequence: the head issues the loads of
+// a step, the tail, kSlabRing - 1 steps behind it, consumes them.  The head records the rows it
+// drew in a small per-wave queue in LDS from which the tail reads them back.  Either cursor asks
+// for the offsets of its following vector-row one row ahead, so that the LDS round trip and the
+// scalar loads are off the critical path.
 struct SlabCursor {
-  int pos;                       // position of the current vector-row in the row block
-  int row, kc, end;              // current step: vectors [kc, min(kc + 32, end)) of vector-row `row`
+  int row, kc, end;  // current step: vectors [kc, min(kc + 32, end)) of vector-row `row`
   bool valid;
   int next_row, next_kc, next_end;
   bool next_valid;
+  int count;  // rows requested so far (index into the per-wave queue)
 };
 
-__device__ __forceinline__ void cursor_prefetch(SlabCursor &c, int pos, int row_hi,
-                                                const int32_t *__restrict__ row_offsets,
-                                                const int32_t *__restrict__ row_indices) {
-  c.next_valid = pos < row_hi;
+struct SlabRows {  // what the cursors need to find rows
+  int *counter;    // LDS: next undrawn position of the row block
+  int *queue;      // LDS: this wave's queue of drawn positions (kSlabQueue entries)
+  int row_lo, row_hi, lane;
+  const int32_t *__restrict__ row_offsets;
+  const int32_t *__restrict__ row_indices;
+};
+static constexpr int kSlabQueue = 16;
+
+template <bool HEAD>
+__device__ __forceinline__ void cursor_prefetch(SlabCursor &c, const SlabRows &rows) {
+  int pos = 0;
+  int *slot = rows.queue + (c.count & (kSlabQueue - 1));
+  if (HEAD) {
+    if (rows.lane == 0) {
+      pos = atomicAdd(rows.counter, 1) + rows.row_lo;
+      *slot = pos;
+    }
+  } else {
+    if (rows.lane == 0) pos = *slot;
+  }
+  pos = __builtin_amdgcn_readfirstlane(pos);
+  ++c.count;
+  c.next_valid = pos < rows.row_hi;
   c.next_row = c.next_kc = c.next_end = 0;
   if (c.next_valid) {
-    c.next_row = row_indices ? row_indices[pos] : pos;
-    c.next_kc = row_offsets[c.next_row];
-    c.next_end = row_offsets[c.next_row + 1];
+    c.next_row = rows.row_indices ? rows.row_indices[pos] : pos;
+    c.next_kc = rows.row_offsets[c.next_row];
+    c.next_end = rows.row_offsets[c.next_row + 1];
   }
 }
 
-__device__ __forceinline__ void cursor_take_next(SlabCursor &c, int row_hi, const int32_t *__restrict__ row_offsets,
-                                                 const int32_t *__restrict__ row_indices) {
-  c.pos += kSlabWaves;
+template <bool HEAD>
+__device__ __forceinline__ void cursor_take_next(SlabCursor &c, const SlabRows &rows) {
   c.row = c.next_row;
   c.kc = c.next_kc;
   c.end = c.next_end;
   c.valid = c.next_valid;
-  if (c.valid) cursor_prefetch(c, c.pos + kSlabWaves, row_hi, row_offsets, row_indices);
+  if (c.valid) cursor_prefetch<HEAD>(c, rows);
 }
 
-__device__ __forceinline__ void cursor_advance(SlabCursor &c, int row_hi, const int32_t *__restrict__ row_offsets,
-                                               const int32_t *__restrict__ row_indices) {
+template <bool HEAD>
+__device__ __forceinline__ void cursor_advance(SlabCursor &c, const SlabRows &rows) {
   c.kc += 32;
-  if (c.kc >= c.end) cursor_take_next(c, row_hi, row_offsets, row_indices);
+  if (c.kc >= c.end) cursor_take_next<HEAD>(c, rows);
 }
 
 template <int V>
@@ -340,13 +361,27 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
                                                                  const int32_t *__restrict__ row_indices) {
   extern __shared__ __align__(16) unsigned char lds[];
   const uint32_t id = blockIdx.x;
-  // Blocks that share a slab differ by multiples of 8 in their id: they land on one XCD and
-  // fetch the slab from the same L2.
-  const uint32_t slab_lo = id & 7u, qd = id >> 3;
-  const uint32_t rb = qd % p.row_blocks;
-  const uint32_t slab_id = (qd / p.row_blocks) * 8u + slab_lo;
-  if (slab_id >= p.n_slabs) return;
-  const uint32_t tile = slab_id % p.n_tiles, batch = slab_id / p.n_tiles;
+  // The hardware deals consecutive block ids round-robin to the 8 XCDs, each with its own L2, so
+  // blocks whose ids are equal modulo 8 share an L2.  With at least 8 batch elements, all blocks of
+  // one batch element (every column tile and row block) are given the same residue: the value
+  // vectors, read once per column tile, and the slab, read once per row block, then come from
+  // that L2 after the first touch.  With fewer batch elements the residue is taken from the slab.
+  const uint32_t xcd = id & 7u, qd = id >> 3;
+  uint32_t rb, tile, batch;
+  if (p.group_by_batch) {
+    const uint32_t per_batch = p.n_tiles * p.row_blocks;
+    const uint32_t rem = qd % per_batch;
+    batch = (qd / per_batch) * 8u + xcd;
+    tile = rem / p.row_blocks;
+    rb = rem % p.row_blocks;
+    if (batch >= (uint32_t)p.batch) return;
+  } else {
+    rb = qd % p.row_blocks;
+    const uint32_t slab_id = (qd / p.row_blocks) * 8u + xcd;
+    if (slab_id >= p.n_slabs) return;
+    tile = slab_id % p.n_tiles;
+    batch = slab_id / p.n_tiles;
+  }
 
   const int tid = threadIdx.x, lane = tid & 63, m = lane & 15, g = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // tell the compiler it is wave-uniform
@@ -355,6 +390,7 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
   const uint16_t *bmat = p.B + (int64_t)batch * p.stride_B;
   const uint32_t b_bytes = (uint32_t)p.K * (uint32_t)p.N * 2u;
   const __amdgpu_buffer_rsrc_t srd_b = make_srd(bmat, b_bytes);
+  uint32_t touch_sink = 0;  // keeps the destination register of the warming loads reserved
 
   // ---- stage the slab: unit u = 16 bytes = columns n0 + 8*(u % 8) .. +7 of row u / 8; the
   // 32-byte segment (u % 8) / 2 of row c lands at segment ((u % 8) / 2) ^ ((c >> 1) & 3).
@@ -377,9 +413,27 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
       if (u < units) *reinterpret_cast<uintx4 *>(lds + dst) = d[i];
     }
   }
+  // ---- warm the L2 with this block's value vectors.  Under a saturating stream of C stores an
+  // HBM read takes several microseconds, far more than the register ring of the main loop covers,
+  // so every 128-byte line of the block's (contiguous) value range is touched once now, behind the
+  // loads of the slab; nothing ever waits for these loads, and the main loop then finds the
+  // lines in the L2 or on their way to it.  One 4-byte load per lane touches 64 lines per instruction.
+  if (row_indices == nullptr) {
+    const int row_lo_p = (int)(rb * p.rows_per_block);
+    const int row_hi_p = min(p.m_vec, row_lo_p + (int)p.rows_per_block);
+    const uint32_t lo = (uint32_t)row_offsets[row_lo_p] * (V * 2u), hi = (uint32_t)row_offsets[row_hi_p] * (V * 2u);
+    const __amdgpu_buffer_rsrc_t srd_touch = make_srd(vals, hi);
+    uint32_t sink = 0;
+    for (uint32_t off = (lo & ~127u) + (uint32_t)tid * 128u; off < hi; off += kSlabThreads * 128u)
+      asm volatile("buffer_load_dword %0, %1, %2, 0 offen" : "+v"(sink) : "v"(off), "s"(srd_touch) : "memory");
+    touch_sink = sink;
+  }
+
   const uint32_t zero_row = (uint32_t)p.K;
   if (tid < 8) *reinterpret_cast<uintx4 *>(lds + zero_row * kSlabRowBytes + tid * 16) = uintx4{0u, 0u, 0u, 0u};
   const uint32_t tiles_off = (zero_row + 1u) * kSlabRowBytes;
+  int *counter = reinterpret_cast<int *>(lds + tiles_off + kSlabWaves * wave_lds_bytes(V));
+  if (tid == 0) *counter = 0;
   __syncthreads();
 
   // ---- per-lane constants
@@ -418,19 +472,30 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
   // ---- this wave's stream of steps
   const int row_lo = (int)(rb * p.rows_per_block);
   const int row_hi = min(p.m_vec, row_lo + (int)p.rows_per_block);
+  SlabRows rows;
+  rows.counter = counter;
+  rows.queue = counter + 1 + wave * kSlabQueue;
+  rows.row_lo = row_lo;
+  rows.row_hi = row_hi;
+  rows.lane = lane;
+  rows.row_offsets = row_offsets;
+  rows.row_indices = row_indices;
   SlabCursor head;  // issues loads
-  head.pos = row_lo + wave - kSlabWaves;
-  cursor_prefetch(head, row_lo + wave, row_hi, row_offsets, row_indices);
-  cursor_take_next(head, row_hi, row_offsets, row_indices);
+  head.count = 0;
+  cursor_prefetch<true>(head, rows);
+  cursor_take_next<true>(head, rows);
   if (!head.valid) return;
-  SlabCursor tail = head;  // consumes them
+  SlabCursor tail;  // consumes them
+  tail.count = 0;
+  cursor_prefetch<false>(tail, rows);
+  cursor_take_next<false>(tail, rows);
 
   SlabLoads<V> ld[kSlabRing];
 #pragma unroll
   for (int i = 0; i < kSlabRing - 1; ++i) {
     if (head.valid) {
       slab_issue<V>(ld[i], head.kc, head.end, lane, slot0, srd_cols, vals);
-      cursor_advance(head, row_hi, row_offsets, row_indices);
+      cursor_advance<true>(head, rows);
     }
   }
   // the value tile of the first step
@@ -445,11 +510,11 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
       const int cur = u, nxt = (u + 1) % R, fill = (u + R - 1) % R;
       if (head.valid) {
         slab_issue<V>(ld[fill], head.kc, head.end, lane, slot0, srd_cols, vals);
-        cursor_advance(head, row_hi, row_offsets, row_indices);
+        cursor_advance<true>(head, rows);
       }
       const int row = tail.row;
       const int left = tail.end - tail.kc;  // vectors of this vector-row from this step on
-      cursor_advance(tail, row_hi, row_offsets, row_indices);
+      cursor_advance<false>(tail, rows);
 
       // A operand: this step's value tile
       Half8Bits a;
@@ -507,7 +572,10 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
           }
         }
       }
-      if (!tail.valid) return;
+      if (!tail.valid) {
+        asm volatile("" ::"v"(touch_sink));  // the warming loads may still be writing this register
+        return;
+      }
     }
   }
 }
@@ -549,7 +617,7 @@ int set_kernel_override(int which) {
   return old;
 }
 
-static constexpr int kSlabMaxK = 1136;  // slab + zero row + 8 x (value tile + staging tile) must fit in 160 KB of LDS
+static constexpr int kSlabMaxK = 1128;  // slab + zero row + 8 x (value tile + staging tile) must fit in 160 KB of LDS
 
 template <int V, typename OutT>
 static hipError_t launch_slab(const SpmmArgs &a, hipStream_t stream) {
@@ -563,7 +631,7 @@ static hipError_t launch_slab(const SpmmArgs &a, hipStream_t stream) {
   if (rows < 32u) rows = 32u;
   p.rows_per_block = rows;
   p.row_blocks = ((uint32_t)a.m_vec + rows - 1u) / rows;
-  const size_t lds = (size_t)(a.K + 1) * kSlabRowBytes + kSlabWaves * wave_lds_bytes(V);
+  const size_t lds = (size_t)(a.K + 1) * kSlabRowBytes + kSlabWaves * wave_lds_bytes(V) + 4 * (1 + kSlabWaves * kSlabQueue);
   auto kern = spmm_slab_kernel<V, OutT>;
   static size_t lds_allowed = 64 * 1024;  // per instantiation
   if (lds > lds_allowed) {
@@ -572,7 +640,9 @@ static hipError_t launch_slab(const SpmmArgs &a, hipStream_t stream) {
     if (e != hipSuccess) return e;
     lds_allowed = 160 * 1024;
   }
-  const uint32_t grid = ((p.n_slabs + 7u) / 8u) * 8u * p.row_blocks;
+  p.group_by_batch = a.batch >= 8 ? 1u : 0u;
+  const uint32_t grid = p.group_by_batch ? (((uint32_t)a.batch + 7u) / 8u) * 8u * p.n_tiles * p.row_blocks
+                                         : ((p.n_slabs + 7u) / 8u) * 8u * p.row_blocks;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kSlabThreads), lds, stream, p, a.row_offsets, a.row_indices);
   return hipGetLastError();
 }

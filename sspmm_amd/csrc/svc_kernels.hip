@@ -29,6 +29,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
+
 #include "svc_kernels.h"
 
 namespace sspmm {
@@ -233,6 +235,201 @@ __global__ __launch_bounds__(THREADS) void svc_merge_cpython_kernel(const SvcArg
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// Fast replay: keys stay in registers, the table holds 32-bit entries.
+//
+// The kernel above moves the whole key list through memory in every phase.  This one keeps each
+// key in a register of a fixed "home" thread (the a-th key ever appended lives in register
+// a / THREADS of thread a % THREADS) together with its current insertion index, and never
+// rewrites the list:
+//   * a table entry is (insertion index << key_bits | key) in 32 bits, so a phase is claimed with
+//     32-bit LDS atomic mins; key_bits = bits of K - 1, which leaves 32 - key_bits bits for the
+//     insertion index (enough for 19 660 keys whenever K <= 131 072; other shapes take the
+//     kernel above);
+//   * after the inserts of a phase the occupancy of the table is reduced to one 64-bit mask and
+//     one running count per 64 slots; a key's next insertion index -- its rank among the occupied
+//     slots -- is count[slot / 64] + popcount(mask[slot / 64] below slot % 64), two small LDS reads
+//     instead of a compaction of the table;
+//   * all atomics (and lookups) of a thread's keys are issued back to back, so a round of a phase
+//     costs one LDS round trip, not one per key.
+// A group's list only exists as an append log, written once per member row so that new keys reach
+// their home thread: in LDS, or in the workspace for groups above 4914 keys.
+static constexpr uint32_t kEmpty32 = 0xffffffffu;
+
+struct FastTable {
+  uint32_t *slots;      // LDS
+  unsigned long long *mask;  // LDS: occupancy of slots 64w .. 64w+63
+  uint32_t *count;      // LDS: occupied slots below 64w
+  uint32_t key_bits, key_mask;
+};
+
+__device__ __forceinline__ int find_slot32(const FastTable &t, uint32_t mask, uint32_t key) {
+  uint32_t i, perturb, lin;
+  probe_start(key, mask, i, perturb, lin);
+  for (;;) {
+    const uint32_t x = t.slots[i + lin];
+    if (x == kEmpty32) return -1;
+    if ((x & t.key_mask) == key) return (int)(i + lin);
+    probe_next(mask, i, perturb, lin);
+  }
+}
+
+__device__ __forceinline__ uint32_t rank_of_slot(const FastTable &t, uint32_t slot) {
+  const unsigned long long m = t.mask[slot >> 6];
+  return t.count[slot >> 6] + (uint32_t)__popcll(m & ((1ull << (slot & 63u)) - 1ull));
+}
+
+// First-come-first-served placement of one key, as in place() above, on 32-bit entries.
+__device__ __forceinline__ void place32(const FastTable &t, uint32_t mask, uint32_t key, uint32_t order) {
+  uint32_t mine = (order << t.key_bits) | key;
+  uint32_t i, perturb, lin;
+  probe_start(key, mask, i, perturb, lin);
+  for (;;) {
+    const uint32_t s0 = i + lin;
+    const uint32_t old = atomicMin(&t.slots[s0], mine);
+    if (old == kEmpty32 || ((old ^ mine) & t.key_mask) == 0) return;  // placed, or a repeated key (invalid row)
+    if (old > mine) {
+      // a later entry sat here: carry it on from this slot of its own probe sequence
+      mine = old;
+      probe_start(old & t.key_mask, mask, i, perturb, lin);
+      while (i + lin != s0) probe_next(mask, i, perturb, lin);
+    }
+    probe_next(mask, i, perturb, lin);
+  }
+}
+
+template <int THREADS, int KPL, bool LIST_IN_LDS>
+__global__ __launch_bounds__(THREADS) void svc_merge_fast_kernel(const SvcArgs a, int class_lo, int class_hi,
+                                                                 uint32_t key_bits, uint32_t max_slots) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int grp = blockIdx.x;
+  const int r0 = grp * a.V, r1 = min(a.M, r0 + a.V);
+  const int e0 = a.row_ptr[r0], e1 = a.row_ptr[r1];
+  const int bound = min(e1 - e0, a.K);
+  if (!in_class(bound, class_lo, class_hi)) return;  // uniform over the group
+  constexpr int WAVES = THREADS / 64;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+  int *scratch = reinterpret_cast<int *>(smem);  // 32 ints
+  FastTable t;
+  t.slots = reinterpret_cast<uint32_t *>(smem + 128);
+  const uint32_t max_words = max_slots >= 64u ? max_slots / 64u : 1u;
+  t.mask = reinterpret_cast<unsigned long long *>(smem + 128 + (size_t)max_slots * 4);
+  t.count = reinterpret_cast<uint32_t *>(smem + 128 + (size_t)max_slots * 4 + (size_t)max_words * 8);
+  t.key_bits = key_bits;
+  t.key_mask = (1u << key_bits) - 1u;
+  int *list = LIST_IN_LDS ? reinterpret_cast<int *>(smem + 128 + (size_t)max_slots * 4 + (size_t)max_words * 12)
+                          : a.pos + e0;  // the position array is free until the very end
+  const int cap = THREADS * KPL < bound ? THREADS * KPL : bound;
+
+  uint32_t key[KPL], ord[KPL];
+#pragma unroll
+  for (int r = 0; r < KPL; ++r) key[r] = ord[r] = 0;
+  int n = 0;
+  uint32_t slots = 0;
+
+  for (int row = r0; row < r1; ++row) {
+    const int b = a.row_ptr[row], e = a.row_ptr[row + 1];
+    // ---- acc + row: log the row's columns that are not in acc yet, in row order
+    int appended = 0;
+    for (int base = b; base < e; base += THREADS) {
+      const int idx = base + tid;
+      bool is_new = false;
+      uint32_t k = 0;
+      if (idx < e) {
+        k = (uint32_t)a.col_ind[idx];
+        is_new = (slots == 0) || find_slot32(t, slots - 1u, k) < 0;
+      }
+      int total;
+      const int rank = block_exclusive_scan<THREADS>(is_new ? 1 : 0, &total, scratch);
+      if (is_new && n + appended + rank < cap) list[n + appended + rank] = (int)k;
+      appended += total;
+    }
+    const int n_new = min(n + appended, cap);  // the cap only bites for invalid input (repeated columns)
+    if (!LIST_IN_LDS) __threadfence_block();
+    __syncthreads();
+    // ---- new keys move to their home threads; their insertion index is their append number
+#pragma unroll
+    for (int r = 0; r < KPL; ++r) {
+      const int ai = tid + r * THREADS;
+      if (ai >= n && ai < n_new) {
+        // a log in global memory was written by other waves of this group: read it past the L1
+        key[r] = LIST_IN_LDS ? (uint32_t)list[ai]
+                             : (uint32_t)__hip_atomic_load(list + ai, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ord[r] = (uint32_t)ai;
+      }
+    }
+    n = n_new;
+
+    // ---- list(set(...)): phases of growing table size
+    slots = 8;
+    for (;;) {
+      const uint32_t thr = resize_threshold(slots);
+      const uint32_t cnt = min((uint32_t)n, thr);
+      const uint32_t mask = slots - 1u;
+      for (uint32_t sidx = tid; sidx < slots; sidx += THREADS) t.slots[sidx] = kEmpty32;
+      __syncthreads();
+      uint32_t part = 0;  // bit r: register r takes part in this phase
+#pragma unroll
+      for (int r = 0; r < KPL; ++r) part |= ((tid + r * THREADS < n) && ord[r] < cnt) ? (1u << r) : 0u;
+#pragma unroll
+      for (int r = 0; r < KPL; ++r)
+        if ((part >> r) & 1u) place32(t, mask, key[r], ord[r]);
+      __syncthreads();
+      // occupancy: one mask and one count per 64 slots
+      const uint32_t words = slots >= 64u ? slots / 64u : 1u;
+      for (uint32_t w = wave; w < words; w += WAVES) {
+        const uint32_t sidx = w * 64u + lane;
+        const bool occ = sidx < slots && t.slots[sidx] != kEmpty32;
+        const unsigned long long m = __ballot(occ);
+        if (lane == 0) {
+          t.mask[w] = m;
+          t.count[w] = (uint32_t)__popcll(m);
+        }
+      }
+      __syncthreads();
+      if (wave == 0) {  // exclusive running count over the words
+        uint32_t carry = 0;
+        for (uint32_t w0 = 0; w0 < words; w0 += 64) {
+          const uint32_t w = w0 + lane;
+          const uint32_t c = w < words ? t.count[w] : 0u;
+          uint32_t incl = c;
+#pragma unroll
+          for (int d = 1; d < 64; d <<= 1) {
+            const uint32_t y = __shfl_up(incl, d, 64);
+            if (lane >= d) incl += y;
+          }
+          if (w < words) t.count[w] = carry + incl - c;
+          carry += __shfl(incl, 63, 64);
+        }
+      }
+      __syncthreads();
+      // a key's next insertion index is its rank in slot order
+#pragma unroll
+      for (int r = 0; r < KPL; ++r) {
+        if ((part >> r) & 1u) {
+          const int sl = find_slot32(t, mask, key[r]);
+          ord[r] = rank_of_slot(t, (uint32_t)sl);
+        }
+      }
+      if ((uint32_t)n < thr) break;
+      slots = resized_slots(thr);
+      __syncthreads();  // the lookups above are done before the table is cleared again
+    }
+  }
+
+  if (tid == 0) a.vec_row_ptr[grp + 1] = n;
+#pragma unroll
+  for (int r = 0; r < KPL; ++r)
+    if (tid + r * THREADS < n) a.tmp_cols[e0 + ord[r]] = (int)key[r];
+  if (!LIST_IN_LDS) __syncthreads();  // the append log lives in the position array
+  if (n > 0)
+    for (int idx = e0 + tid; idx < e1; idx += THREADS) {
+      const int sl = find_slot32(t, slots - 1u, (uint32_t)a.col_ind[idx]);
+      a.pos[idx] = sl >= 0 ? (int)rank_of_slot(t, (uint32_t)sl) : 0;  // sl < 0 only for invalid (capped) input
+    }
+}
+
 // Ascending order: a K-bit occupancy bitmap per group plus a per-word running popcount.
 template <int THREADS>
 __global__ __launch_bounds__(THREADS) void svc_merge_sorted_kernel(const SvcArgs a) {
@@ -333,7 +530,7 @@ size_t svc_workspace_layout(int64_t nnz, size_t *off_pos, size_t *off_tables) {
   return cols + pos + tables;
 }
 
-static constexpr int kSmallKeys = 306, kMediumKeys = 1228, kLargeKeys = 4914;
+static constexpr int kSmallKeys = 306, kMediumKeys = 1228, kLargeKeys = 4914, kXLargeKeys = 19660;
 
 template <int THREADS>
 static hipError_t launch_lds_class(const SvcArgs &base, int m_vec, int lo, int hi, int slots, hipStream_t stream) {
@@ -350,18 +547,85 @@ static hipError_t launch_lds_class(const SvcArgs &base, int m_vec, int lo, int h
   return hipGetLastError();
 }
 
+template <int THREADS, int KPL, bool LIST_IN_LDS>
+static hipError_t launch_fast_class(const SvcArgs &a, int m_vec, int lo, int hi, uint32_t slots, uint32_t key_bits,
+                                    hipStream_t stream) {
+  const uint32_t words = slots >= 64u ? slots / 64u : 1u;
+  const size_t lds = 128 + (size_t)slots * 4 + (size_t)words * 12 + (LIST_IN_LDS ? (size_t)hi * 4 : 0);
+  auto kern = svc_merge_fast_kernel<THREADS, KPL, LIST_IN_LDS>;
+  if (lds > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return e;
+  }
+  hipLaunchKernelGGL(kern, dim3(m_vec), dim3(THREADS), lds, stream, a, lo, hi, key_bits, slots);
+  return hipGetLastError();
+}
+
+// The size classes are independent kernels over disjoint groups: they run side by side on three
+// helper streams (default priority, created once per device) forked from and joined back into
+// the caller's stream with events, so the phase costs what its slowest class costs.
+struct SideStreams {
+  bool ready = false;
+  hipStream_t s[3];
+  hipEvent_t fork, join[3];
+};
+static SideStreams g_side[16];
+static std::mutex g_side_mutex;
+
+static SideStreams *side_streams() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return nullptr;
+  std::lock_guard<std::mutex> lock(g_side_mutex);
+  SideStreams &ss = g_side[dev];
+  if (!ss.ready) {
+    for (int i = 0; i < 3; ++i) {
+      if (hipStreamCreateWithFlags(&ss.s[i], hipStreamNonBlocking) != hipSuccess) return nullptr;
+      if (hipEventCreateWithFlags(&ss.join[i], hipEventDisableTiming) != hipSuccess) return nullptr;
+    }
+    if (hipEventCreateWithFlags(&ss.fork, hipEventDisableTiming) != hipSuccess) return nullptr;
+    ss.ready = true;
+  }
+  return &ss;
+}
+
 hipError_t launch_svc_count(const SvcArgs &a, int order, hipStream_t stream) {
   const int m_vec = (a.M + a.V - 1) / a.V;
   hipError_t e;
   if (order == 0) {
-    // Four passes over the groups, each taking the groups of its size class; a group's class is
-    // decided from min(non-zeros of the group, K), an upper bound of its distinct columns.
-    if ((e = launch_lds_class<64>(a, m_vec, -1, kSmallKeys, 512, stream)) != hipSuccess) return e;
-    if ((e = launch_lds_class<256>(a, m_vec, kSmallKeys, kMediumKeys, 2048, stream)) != hipSuccess) return e;
-    if ((e = launch_lds_class<1024>(a, m_vec, kMediumKeys, kLargeKeys, 8192, stream)) != hipSuccess) return e;
-    hipLaunchKernelGGL((svc_merge_cpython_kernel<1024, false>), dim3(m_vec), dim3(1024), 128, stream, a, kLargeKeys,
-                       0x7fffffff, 0);
+    // One pass over the groups per size class, each taking the groups of its class; a group's class
+    // is decided from min(non-zeros of the group, K), an upper bound of its distinct columns.
+    uint32_t key_bits = 1;
+    while (key_bits < 31 && (1u << key_bits) < (uint32_t)a.K) ++key_bits;
+    SideStreams *ss = side_streams();
+    hipStream_t st[4] = {stream, stream, stream, stream};
+    if (ss) {
+      if ((e = hipEventRecord(ss->fork, stream)) != hipSuccess) return e;
+      for (int i = 0; i < 3; ++i) {
+        if ((e = hipStreamWaitEvent(ss->s[i], ss->fork, 0)) != hipSuccess) return e;
+        st[i + 1] = ss->s[i];
+      }
+    }
+    if ((e = launch_lds_class<64>(a, m_vec, -1, kSmallKeys, 512, st[0])) != hipSuccess) return e;
+    if ((e = launch_lds_class<256>(a, m_vec, kSmallKeys, kMediumKeys, 2048, st[1])) != hipSuccess) return e;
+    if ((e = launch_lds_class<1024>(a, m_vec, kMediumKeys, kLargeKeys, 8192, st[2])) != hipSuccess) return e;
+    int top = kLargeKeys;
+    if (key_bits <= 17) {
+      // 32-bit table entries in LDS: 15 bits of insertion index are enough up to 19 660 keys
+      if ((e = launch_fast_class<1024, 20, false>(a, m_vec, kLargeKeys, kXLargeKeys, 32768, key_bits, st[3])) !=
+          hipSuccess)
+        return e;
+      top = kXLargeKeys;
+    }
+    hipLaunchKernelGGL((svc_merge_cpython_kernel<1024, false>), dim3(m_vec), dim3(1024), 128, st[3], a, top, 0x7fffffff,
+                       0);
     if ((e = hipGetLastError()) != hipSuccess) return e;
+    if (ss) {
+      for (int i = 0; i < 3; ++i) {
+        if ((e = hipEventRecord(ss->join[i], ss->s[i])) != hipSuccess) return e;
+        if ((e = hipStreamWaitEvent(stream, ss->join[i], 0)) != hipSuccess) return e;
+      }
+    }
   } else {
     const int words = (a.K + 31) / 32;
     const size_t lds = 128 + (size_t)words * 8;

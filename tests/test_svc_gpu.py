@@ -134,3 +134,22 @@ def test_svc_then_spmm_equals_csr_matmul(oracle, built_library):
         A[i, csr.col_ind[csr.row_ptr[i]:csr.row_ptr[i + 1]]] = csr.values[csr.row_ptr[i]:csr.row_ptr[i + 1]]
     want = A @ B.astype(np.float64)
     assert np.abs(out.cpu().numpy() - want).max() <= 2e-5 * np.abs(want).max()
+
+
+def test_wide_matrices_and_giant_groups_take_the_64_bit_tables(oracle, built_library):
+    """K above 2^17 (column indices too wide for 32-bit table entries) and a group above 19 660 keys
+    run the kernels with 64-bit entries, the giant group with its table in the workspace."""
+    rng = np.random.default_rng(42)
+    K = 300000
+    lens = np.zeros(24, np.int64)
+    lens[:8] = 3000          # 24 000 distinct columns in one group
+    lens[8:16] = [0, 5, 700, 1, 0, 90, 2000, 3]
+    lens[16:] = 40
+    ptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cols = np.concatenate([np.sort(rng.choice(K, n, replace=False)) for n in lens]).astype(np.int32)
+    csr = synth.Csr(24, K, ptr, cols, rng.standard_normal(cols.size).astype(np.float16))
+    _compare_with_oracle(oracle, csr, 8)
+    # same shape of groups with narrow columns: the giant group is the only one on 64-bit entries
+    K2 = 100000
+    cols2 = np.concatenate([np.sort(rng.choice(K2, n, replace=False)) for n in lens]).astype(np.int32)
+    _compare_with_oracle(oracle, synth.Csr(24, K2, ptr, cols2, csr.values), 8)

@@ -35,6 +35,9 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--batch", type=int, default=128, help="independent value/B/C sets per step")
     ap.add_argument("--quick", action="store_true", help="skip the extra configurations and CPU legs")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy (its hardware-counter readings calibrate FETCH_SIZE / "
+                         "WRITE_SIZE when the run is profiled)")
     ap.add_argument("--kernel", choices=["auto", "generic", "gather", "slab"], default="auto",
                     help="force one SpMM kernel (tuning); the default lets the library choose")
     return ap.parse_args()
@@ -114,6 +117,14 @@ def main():
     L = _lib.lib()
     torch.cuda.set_device(0)
     L.sspmm_select_kernel({"auto": 0, "generic": 1, "gather": 2, "slab": 3}[args.kernel])
+
+    if args.calibrate_copy:
+        src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     M, K, V, sparsity, N = 2048, 512, 8, 0.9, 256
     main_res, (vs, vals, B, C) = spmm_case(L, torch, synth, M, K, V, sparsity, N, args.batch, True, 0.02, 2,

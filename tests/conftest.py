@@ -16,7 +16,8 @@ def pytest_configure(config):
 def built_library():
     """Path of libsspmm_amd.so; compiles it first only when no built library is there."""
     from sspmm_amd import _lib
-    if not os.path.exists(_lib.library_path()):
+    harness = os.path.join(ROOT, "sspmm_amd", "bin", "sspmm_test")
+    if not (os.path.exists(_lib.library_path()) and os.path.exists(harness)):
         _lib.build_library(force=False)
     return _lib.library_path()
 

@@ -26,6 +26,10 @@ import numpy as np
 
 HBM_PEAK_GBPS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
+# HBM bytes per launch of the headline workload at the default batch of 128, from hardware counters
+# (FETCH_SIZE and WRITE_SIZE, each scaled by its reading for a 256 MiB device copy): see
+# profiles/spmm_slab_v8_f32_cfg2_batch128_hbm_traffic.txt.  Other batch sizes report null.
+MEASURED_TRAFFIC_BYTES = {128: 76.9e6 + 268.4e6}
 
 
 def parse_args():
@@ -231,7 +235,8 @@ def main():
         "config": {"workload": main_res["workload"] + " (one launch, pattern shared by the batch)",
                    "hbm_gbps": main_res["hbm_gbps"]},
         "roofline": {"bound": "hbm", "achieved": main_res["hbm_gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": main_res["hbm_frac"], "traffic": None,
+                     "frac": main_res["hbm_frac"],
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.batch) if args.kernel == "auto" else None,
                      "kernel": "spmm_gather_kernel<8,float>", "alg_bytes_per_launch": main_res["alg_bytes"]},
         "cpu_baseline": cpu,
         "parity_max_rel_err": parity,

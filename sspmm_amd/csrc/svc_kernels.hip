@@ -236,34 +236,24 @@ __global__ __launch_bounds__(THREADS) void svc_merge_cpython_kernel(const SvcArg
 }
 
 // ------------------------------------------------------------------------------------------
-// Fast replay: keys stay in registers, the table holds 32-bit entries.
+// The same replay on 32-bit table entries.
 //
-// The kernel above moves the whole key list through memory in every phase.  This one keeps each
-// key in a register of a fixed "home" thread (the a-th key ever appended lives in register
-// a / THREADS of thread a % THREADS) together with its current insertion index, and never
-// rewrites the list:
-//   * a table entry is (insertion index << key_bits | key) in 32 bits, so a phase is claimed with
-//     32-bit LDS atomic mins; key_bits = bits of K - 1, which leaves 32 - key_bits bits for the
-//     insertion index (enough for 19 660 keys whenever K <= 131 072; other shapes take the
-//     kernel above);
-//   * after the inserts of a phase the occupancy of the table is reduced to one 64-bit mask and
-//     one running count per 64 slots; a key's next insertion index -- its rank among the occupied
-//     slots -- is count[slot / 64] + popcount(mask[slot / 64] below slot % 64), two small LDS reads
-//     instead of a compaction of the table;
-//   * all atomics (and lookups) of a thread's keys are issued back to back, so a round of a phase
-//     costs one LDS round trip, not one per key.
-// A group's list only exists as an append log, written once per member row so that new keys reach
-// their home thread: in LDS, or in the workspace for groups above 4914 keys.
+// When the column indices fit in 17 bits (K <= 131 072) a table entry is
+// (insertion index << key_bits | key) in 32 bits, key_bits = bits of K - 1, which leaves at least 15
+// bits of insertion index: enough for 19 660 keys, the largest set CPython keeps in a 32 768-slot
+// table.  Halving the entries brings groups of up to 19 660 keys into LDS (a 128 KB table; their
+// key list stays in the workspace) and makes the atomics 32-bit.  The compaction of a phase is done
+// one 64-slot word per wave iteration: a ballot gives the occupancy mask, a first pass leaves the
+// population of every word, wave 0 turns them into running counts, and a second pass writes
+// list[count[word] + rank in word] = key, so nothing is scanned per thread.
 static constexpr uint32_t kEmpty32 = 0xffffffffu;
 
-struct FastTable {
-  uint32_t *slots;      // LDS
-  unsigned long long *mask;  // LDS: occupancy of slots 64w .. 64w+63
-  uint32_t *count;      // LDS: occupied slots below 64w
+struct Table32 {
+  uint32_t *slots;  // LDS
   uint32_t key_bits, key_mask;
 };
 
-__device__ __forceinline__ int find_slot32(const FastTable &t, uint32_t mask, uint32_t key) {
+__device__ __forceinline__ int find_slot32(const Table32 &t, uint32_t mask, uint32_t key) {
   uint32_t i, perturb, lin;
   probe_start(key, mask, i, perturb, lin);
   for (;;) {
@@ -274,13 +264,8 @@ __device__ __forceinline__ int find_slot32(const FastTable &t, uint32_t mask, ui
   }
 }
 
-__device__ __forceinline__ uint32_t rank_of_slot(const FastTable &t, uint32_t slot) {
-  const unsigned long long m = t.mask[slot >> 6];
-  return t.count[slot >> 6] + (uint32_t)__popcll(m & ((1ull << (slot & 63u)) - 1ull));
-}
-
 // First-come-first-served placement of one key, as in place() above, on 32-bit entries.
-__device__ __forceinline__ void place32(const FastTable &t, uint32_t mask, uint32_t key, uint32_t order) {
+__device__ __forceinline__ void place32(const Table32 &t, uint32_t mask, uint32_t key, uint32_t order) {
   uint32_t mine = (order << t.key_bits) | key;
   uint32_t i, perturb, lin;
   probe_start(key, mask, i, perturb, lin);
@@ -298,7 +283,95 @@ __device__ __forceinline__ void place32(const FastTable &t, uint32_t mask, uint3
   }
 }
 
-template <int THREADS, int KPL, bool LIST_IN_LDS>
+// The key list lives in LDS, or in the workspace where other waves of the group wrote it: those
+// accesses go past the L1.
+template <bool IN_LDS>
+__device__ __forceinline__ int list_load(const int *list, int idx) {
+  return IN_LDS ? list[idx] : __hip_atomic_load(list + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <bool IN_LDS>
+__device__ __forceinline__ void list_store(int *list, int idx, int v) {
+  if (IN_LDS) list[idx] = v;
+  else __hip_atomic_store(list + idx, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <int THREADS, bool LIST_IN_LDS>
+__device__ __forceinline__ uint32_t rebuild_set32(const Table32 &t, uint32_t *wcount, int *list, int &n, int *scratch) {
+  constexpr int WAVES = THREADS / 64;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  (void)scratch;
+  uint32_t slots = 8;
+  for (;;) {
+    const uint32_t thr = resize_threshold(slots);
+    const int cnt = min(n, (int)thr);
+    const uint32_t mask = slots - 1u;
+    for (uint32_t s = tid; s < slots; s += THREADS) t.slots[s] = kEmpty32;
+    __syncthreads();
+    // A thread inserts its keys in list order (idx = tid, tid + THREADS, ...), so the whole group works
+    // through the list in chunks of THREADS keys and a later key rarely arrives before an earlier
+    // one.  The keys are fetched eight at a time ahead of the inserts: one round trip per batch.
+    for (int base = tid; base < cnt; base += 8 * THREADS) {
+      int k8[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int idx = base + j * THREADS;
+        k8[j] = idx < cnt ? list_load<LIST_IN_LDS>(list, idx) : 0;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int idx = base + j * THREADS;
+        if (idx < cnt) place32(t, mask, (uint32_t)k8[j], (uint32_t)idx);
+      }
+    }
+    __syncthreads();
+    const bool final = n < (int)thr;
+    const uint32_t words = slots >= 64u ? slots / 64u : 1u;
+    for (uint32_t w = wave; w < words; w += WAVES) {
+      const uint32_t s = w * 64u + lane;
+      const bool occ = s < slots && t.slots[s] != kEmpty32;
+      const unsigned long long m = __ballot(occ);
+      if (lane == 0) wcount[w] = (uint32_t)__popcll(m);
+    }
+    __syncthreads();
+    if (wave == 0) {  // running counts over the words
+      uint32_t carry = 0;
+      for (uint32_t w0 = 0; w0 < words; w0 += 64) {
+        const uint32_t w = w0 + lane;
+        const uint32_t c = w < words ? wcount[w] : 0u;
+        uint32_t incl = c;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+          const uint32_t y = __shfl_up(incl, d, 64);
+          if (lane >= d) incl += y;
+        }
+        if (w < words) wcount[w] = carry + incl - c;
+        carry += __shfl(incl, 63, 64);
+      }
+      if (lane == 0) wcount[words] = carry;  // number of keys in the table
+    }
+    __syncthreads();
+    for (uint32_t w = wave; w < words; w += WAVES) {
+      const uint32_t s = w * 64u + lane;
+      const uint32_t x = s < slots ? t.slots[s] : kEmpty32;
+      const bool occ = x != kEmpty32;
+      const unsigned long long m = __ballot(occ);
+      const uint32_t rank = wcount[w] + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+      if (occ) {
+        list_store<LIST_IN_LDS>(list, (int)rank, (int)(x & t.key_mask));
+        if (final) t.slots[s] = (rank << t.key_bits) | (x & t.key_mask);
+      }
+    }
+    const int kept = (int)wcount[words];
+    __syncthreads();
+    if (final) {
+      n = kept;
+      return slots;
+    }
+    slots = resized_slots(thr);
+  }
+}
+
+template <int THREADS, bool LIST_IN_LDS>
 __global__ __launch_bounds__(THREADS) void svc_merge_fast_kernel(const SvcArgs a, int class_lo, int class_hi,
                                                                  uint32_t key_bits, uint32_t max_slots) {
   extern __shared__ __align__(16) unsigned char smem[];
@@ -307,30 +380,24 @@ __global__ __launch_bounds__(THREADS) void svc_merge_fast_kernel(const SvcArgs a
   const int e0 = a.row_ptr[r0], e1 = a.row_ptr[r1];
   const int bound = min(e1 - e0, a.K);
   if (!in_class(bound, class_lo, class_hi)) return;  // uniform over the group
-  constexpr int WAVES = THREADS / 64;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x;
 
   int *scratch = reinterpret_cast<int *>(smem);  // 32 ints
-  FastTable t;
+  Table32 t;
   t.slots = reinterpret_cast<uint32_t *>(smem + 128);
-  const uint32_t max_words = max_slots >= 64u ? max_slots / 64u : 1u;
-  t.mask = reinterpret_cast<unsigned long long *>(smem + 128 + (size_t)max_slots * 4);
-  t.count = reinterpret_cast<uint32_t *>(smem + 128 + (size_t)max_slots * 4 + (size_t)max_words * 8);
   t.key_bits = key_bits;
   t.key_mask = (1u << key_bits) - 1u;
-  int *list = LIST_IN_LDS ? reinterpret_cast<int *>(smem + 128 + (size_t)max_slots * 4 + (size_t)max_words * 12)
-                          : a.pos + e0;  // the position array is free until the very end
-  const int cap = THREADS * KPL < bound ? THREADS * KPL : bound;
+  const uint32_t max_words = max_slots >= 64u ? max_slots / 64u : 1u;
+  uint32_t *wcount = reinterpret_cast<uint32_t *>(smem + 128 + (size_t)max_slots * 4);  // max_words + 1 entries
+  int *list = LIST_IN_LDS ? reinterpret_cast<int *>(smem + 128 + (size_t)max_slots * 4 + (size_t)(max_words + 1) * 4)
+                          : a.tmp_cols + e0;
+  const int cap = LIST_IN_LDS ? min(class_hi, bound) : bound;
 
-  uint32_t key[KPL], ord[KPL];
-#pragma unroll
-  for (int r = 0; r < KPL; ++r) key[r] = ord[r] = 0;
   int n = 0;
   uint32_t slots = 0;
-
   for (int row = r0; row < r1; ++row) {
     const int b = a.row_ptr[row], e = a.row_ptr[row + 1];
-    // ---- acc + row: log the row's columns that are not in acc yet, in row order
+    // acc + row: append the row's columns that are not in acc yet, in row order
     int appended = 0;
     for (int base = b; base < e; base += THREADS) {
       const int idx = base + tid;
@@ -342,91 +409,21 @@ __global__ __launch_bounds__(THREADS) void svc_merge_fast_kernel(const SvcArgs a
       }
       int total;
       const int rank = block_exclusive_scan<THREADS>(is_new ? 1 : 0, &total, scratch);
-      if (is_new && n + appended + rank < cap) list[n + appended + rank] = (int)k;
+      if (is_new && n + appended + rank < cap) list_store<LIST_IN_LDS>(list, n + appended + rank, (int)k);
       appended += total;
     }
-    const int n_new = min(n + appended, cap);  // the cap only bites for invalid input (repeated columns)
-    if (!LIST_IN_LDS) __threadfence_block();
+    n = min(n + appended, cap);  // the cap only bites for invalid input (repeated columns)
     __syncthreads();
-    // ---- new keys move to their home threads; their insertion index is their append number
-#pragma unroll
-    for (int r = 0; r < KPL; ++r) {
-      const int ai = tid + r * THREADS;
-      if (ai >= n && ai < n_new) {
-        // a log in global memory was written by other waves of this group: read it past the L1
-        key[r] = LIST_IN_LDS ? (uint32_t)list[ai]
-                             : (uint32_t)__hip_atomic_load(list + ai, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        ord[r] = (uint32_t)ai;
-      }
-    }
-    n = n_new;
-
-    // ---- list(set(...)): phases of growing table size
-    slots = 8;
-    for (;;) {
-      const uint32_t thr = resize_threshold(slots);
-      const uint32_t cnt = min((uint32_t)n, thr);
-      const uint32_t mask = slots - 1u;
-      for (uint32_t sidx = tid; sidx < slots; sidx += THREADS) t.slots[sidx] = kEmpty32;
-      __syncthreads();
-      uint32_t part = 0;  // bit r: register r takes part in this phase
-#pragma unroll
-      for (int r = 0; r < KPL; ++r) part |= ((tid + r * THREADS < n) && ord[r] < cnt) ? (1u << r) : 0u;
-#pragma unroll
-      for (int r = 0; r < KPL; ++r)
-        if ((part >> r) & 1u) place32(t, mask, key[r], ord[r]);
-      __syncthreads();
-      // occupancy: one mask and one count per 64 slots
-      const uint32_t words = slots >= 64u ? slots / 64u : 1u;
-      for (uint32_t w = wave; w < words; w += WAVES) {
-        const uint32_t sidx = w * 64u + lane;
-        const bool occ = sidx < slots && t.slots[sidx] != kEmpty32;
-        const unsigned long long m = __ballot(occ);
-        if (lane == 0) {
-          t.mask[w] = m;
-          t.count[w] = (uint32_t)__popcll(m);
-        }
-      }
-      __syncthreads();
-      if (wave == 0) {  // exclusive running count over the words
-        uint32_t carry = 0;
-        for (uint32_t w0 = 0; w0 < words; w0 += 64) {
-          const uint32_t w = w0 + lane;
-          const uint32_t c = w < words ? t.count[w] : 0u;
-          uint32_t incl = c;
-#pragma unroll
-          for (int d = 1; d < 64; d <<= 1) {
-            const uint32_t y = __shfl_up(incl, d, 64);
-            if (lane >= d) incl += y;
-          }
-          if (w < words) t.count[w] = carry + incl - c;
-          carry += __shfl(incl, 63, 64);
-        }
-      }
-      __syncthreads();
-      // a key's next insertion index is its rank in slot order
-#pragma unroll
-      for (int r = 0; r < KPL; ++r) {
-        if ((part >> r) & 1u) {
-          const int sl = find_slot32(t, mask, key[r]);
-          ord[r] = rank_of_slot(t, (uint32_t)sl);
-        }
-      }
-      if ((uint32_t)n < thr) break;
-      slots = resized_slots(thr);
-      __syncthreads();  // the lookups above are done before the table is cleared again
-    }
+    slots = rebuild_set32<THREADS, LIST_IN_LDS>(t, wcount, list, n, scratch);
   }
 
   if (tid == 0) a.vec_row_ptr[grp + 1] = n;
-#pragma unroll
-  for (int r = 0; r < KPL; ++r)
-    if (tid + r * THREADS < n) a.tmp_cols[e0 + ord[r]] = (int)key[r];
-  if (!LIST_IN_LDS) __syncthreads();  // the append log lives in the position array
+  if (LIST_IN_LDS)
+    for (int p = tid; p < n; p += THREADS) a.tmp_cols[e0 + p] = list[p];
   if (n > 0)
     for (int idx = e0 + tid; idx < e1; idx += THREADS) {
       const int sl = find_slot32(t, slots - 1u, (uint32_t)a.col_ind[idx]);
-      a.pos[idx] = sl >= 0 ? (int)rank_of_slot(t, (uint32_t)sl) : 0;  // sl < 0 only for invalid (capped) input
+      a.pos[idx] = sl >= 0 ? (int)(t.slots[sl] >> key_bits) : 0;  // sl < 0 only for invalid (capped) input
     }
 }
 
@@ -547,12 +544,12 @@ static hipError_t launch_lds_class(const SvcArgs &base, int m_vec, int lo, int h
   return hipGetLastError();
 }
 
-template <int THREADS, int KPL, bool LIST_IN_LDS>
+template <int THREADS, bool LIST_IN_LDS>
 static hipError_t launch_fast_class(const SvcArgs &a, int m_vec, int lo, int hi, uint32_t slots, uint32_t key_bits,
                                     hipStream_t stream) {
   const uint32_t words = slots >= 64u ? slots / 64u : 1u;
-  const size_t lds = 128 + (size_t)slots * 4 + (size_t)words * 12 + (LIST_IN_LDS ? (size_t)hi * 4 : 0);
-  auto kern = svc_merge_fast_kernel<THREADS, KPL, LIST_IN_LDS>;
+  const size_t lds = 128 + (size_t)slots * 4 + (size_t)(words + 1) * 4 + (LIST_IN_LDS ? (size_t)hi * 4 : 0);
+  auto kern = svc_merge_fast_kernel<THREADS, LIST_IN_LDS>;
   if (lds > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -606,16 +603,21 @@ hipError_t launch_svc_count(const SvcArgs &a, int order, hipStream_t stream) {
         st[i + 1] = ss->s[i];
       }
     }
-    if ((e = launch_lds_class<64>(a, m_vec, -1, kSmallKeys, 512, st[0])) != hipSuccess) return e;
-    if ((e = launch_lds_class<256>(a, m_vec, kSmallKeys, kMediumKeys, 2048, st[1])) != hipSuccess) return e;
-    if ((e = launch_lds_class<1024>(a, m_vec, kMediumKeys, kLargeKeys, 8192, st[2])) != hipSuccess) return e;
     int top = kLargeKeys;
     if (key_bits <= 17) {
-      // 32-bit table entries in LDS: 15 bits of insertion index are enough up to 19 660 keys
-      if ((e = launch_fast_class<1024, 20, false>(a, m_vec, kLargeKeys, kXLargeKeys, 32768, key_bits, st[3])) !=
-          hipSuccess)
+      // 32-bit table entries: 15 bits of insertion index are enough up to 19 660 keys
+      if ((e = launch_fast_class<64, true>(a, m_vec, -1, kSmallKeys, 512, key_bits, st[0])) != hipSuccess) return e;
+      if ((e = launch_fast_class<256, true>(a, m_vec, kSmallKeys, kMediumKeys, 2048, key_bits, st[1])) != hipSuccess)
+        return e;
+      if ((e = launch_fast_class<1024, true>(a, m_vec, kMediumKeys, kLargeKeys, 8192, key_bits, st[2])) != hipSuccess)
+        return e;
+      if ((e = launch_fast_class<1024, false>(a, m_vec, kLargeKeys, kXLargeKeys, 32768, key_bits, st[3])) != hipSuccess)
         return e;
       top = kXLargeKeys;
+    } else {
+      if ((e = launch_lds_class<64>(a, m_vec, -1, kSmallKeys, 512, st[0])) != hipSuccess) return e;
+      if ((e = launch_lds_class<256>(a, m_vec, kSmallKeys, kMediumKeys, 2048, st[1])) != hipSuccess) return e;
+      if ((e = launch_lds_class<1024>(a, m_vec, kMediumKeys, kLargeKeys, 8192, st[2])) != hipSuccess) return e;
     }
     hipLaunchKernelGGL((svc_merge_cpython_kernel<1024, false>), dim3(m_vec), dim3(1024), 128, st[3], a, top, 0x7fffffff,
                        0);

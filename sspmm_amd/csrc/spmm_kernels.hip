@@ -228,12 +228,9 @@ static constexpr int kSlabWaves = 8;
 static constexpr int kSlabThreads = kSlabWaves * 64;
 static constexpr int kSlabRowBytes = 128;       // 64 columns of fp16
 // Per-wave LDS: the value tile of a step (32 vectors x V halfs; the V = 8 transpose read touches 16
-// bytes past its 512) and a staging tile of 8 rows x 128 bytes (+16 bytes of padding per row)
-// through which finished tiles of C are turned into row-contiguous 16-byte stores.
+// bytes past its 512).
 static constexpr int val_tile_bytes(int V) { return V == 8 ? 528 : 1024; }
-static constexpr int kStageStride = 144;
-static constexpr int kStageBytes = 8 * kStageStride;
-static constexpr int wave_lds_bytes(int V) { return val_tile_bytes(V) + kStageBytes; }
+static constexpr int wave_lds_bytes(int V) { return val_tile_bytes(V); }
 
 static constexpr int kSlabRing = 8;  // steps whose loads are in flight or waiting in registers
 
@@ -342,16 +339,119 @@ __device__ __forceinline__ void slab_issue(SlabLoads<V> &r, int kc, int end, int
   r.vraw = SlabVals<V>::load(srd_vals, (uint32_t)kc * (V * 2u) + (uint32_t)lane * kLaneBytes);
 }
 
-template <typename OutT>
-struct StageElem;  // writes one accumulator element into the staging tile in the output type
-template <>
-struct StageElem<float> {
-  static __device__ __forceinline__ void put(unsigned char *p, float a) { *reinterpret_cast<float *>(p) = a; }
+// The store of one 16-byte piece of C per lane.  A wave's vector-memory counter counts loads and
+// stores together and guarantees order only within each kind, so a compiler that sees a store in
+// flight must drain the whole counter wherever the wave waits for a load; that would serialise
+// every step of the main loop behind its own loads.  The store is therefore issued from inline
+// assembly, which keeps it out of the compiler's count: the waits it computes for the loads of the
+// ring are then "at most n operations outstanding" with n the number of younger loads.  Loads
+// return in order among themselves, so while an awaited load is outstanding so are its n younger
+// loads, and the wait cannot pass early whatever the stores do; stores in flight only make it
+// pass later.  The trailing s_nop covers the cycles in which the store still reads its data registers.
+__device__ __forceinline__ void slab_store_line(uintx4 line, __amdgpu_buffer_rsrc_t srd, uint32_t voff, uint32_t soff) {
+  asm volatile("buffer_store_dwordx4 %0, %1, %2, %3 offen\n\ts_nop 1" ::"v"(line), "v"(voff), "s"(srd), "s"(soff));
+}
+
+// Writing a finished V x 64 tile of C.  The MFMAs run with the slab as their first operand, so
+// accumulator q of lane (m, g) holds C[row m][n0 + 16q + 4g .. + 3]: four consecutive columns of
+// one row.  Lanes are then regrouped in registers so that each lane owns 16 contiguous bytes and a
+// store instruction writes whole 128-byte lines:
+//   * fp32: the 16 bytes are the lane's own four columns.  With V = 8 only lanes m < 8 hold rows;
+//     lanes m >= 8 take tile q + 1 of row m - 8 (a DPP shift by 8 inside the 16-lane row), so one
+//     instruction writes 8 rows x (64 + 64) bytes.  With V = 16 the same exchange runs in both
+//     directions and two instructions write rows 0..7 and 8..15.
+//   * fp16: a lane's four columns are 8 bytes; v_permlane16_swap pairs lane groups g and g + 1 of
+//     two tiles so that a lane owns eight consecutive columns, then the DPP exchange as above
+//     gathers all four tiles of a row into one instruction.
+template <int V, typename OutT>
+struct SlabStore;
+
+__device__ __forceinline__ uint32_t dpp_from_m_minus_8(uint32_t keep, uint32_t src) {  // lanes m >= 8 take src of lane m - 8
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)keep, (int)src, 0x118, 0xf, 0xc, false);
+}
+__device__ __forceinline__ uint32_t dpp_from_m_plus_8(uint32_t keep, uint32_t src) {  // lanes m < 8 take src of lane m + 8
+  return (uint32_t)__builtin_amdgcn_update_dpp((int)keep, (int)src, 0x108, 0xf, 0x3, false);
+}
+
+template <int V>
+struct SlabStore<V, float> {
+  static constexpr int kInstr = V / 4;  // 2 tile pairs x (V / 8) row halves
+  uint32_t voff[V / 8];                 // byte offset of the lane's 16 bytes for tile pair 0, per row half
+  int col[V / 8];                       // its first column
+  __device__ __forceinline__ void init(int lane, int n0, int N) {
+    const int m = lane & 15, g = lane >> 4;
+#pragma unroll
+    for (int h = 0; h < V / 8; ++h) {
+      const int row = 8 * h + (m & 7);
+      const int tile = h == 0 ? (m >> 3) : 1 - (m >> 3);
+      col[h] = n0 + 16 * tile + 4 * g;
+      voff[h] = ((uint32_t)row * (uint32_t)N + (uint32_t)col[h]) * 4u;
+    }
+  }
+  __device__ __forceinline__ void store(const floatx4 (&acc)[4], __amdgpu_buffer_rsrc_t srd, uint32_t crow, int N) const {
+#pragma unroll
+    for (int qp = 0; qp < 2; ++qp) {
+#pragma unroll
+      for (int h = 0; h < V / 8; ++h) {
+        uintx4 line;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          // (copied to scalars first: a bit cast applied directly to a vector element reads element 0)
+          const float fx = acc[2 * qp][r], fy = acc[2 * qp + 1][r];
+          const uint32_t x = __builtin_bit_cast(uint32_t, fx), y = __builtin_bit_cast(uint32_t, fy);
+          line[r] = h == 0 ? dpp_from_m_minus_8(x, y) : dpp_from_m_plus_8(x, y);
+        }
+        if (col[h] + 32 * qp < N) slab_store_line(line, srd, voff[h] + 128u * qp, crow);
+      }
+    }
+  }
 };
-template <>
-struct StageElem<_Float16> {
-  static __device__ __forceinline__ void put(unsigned char *p, float a) {
-    *reinterpret_cast<_Float16 *>(p) = (_Float16)a;  // round to nearest even
+
+template <int V>
+struct SlabStore<V, _Float16> {
+  uint32_t voff[V / 8];
+  int col[V / 8];
+  __device__ __forceinline__ void init(int lane, int n0, int N) {
+    const int m = lane & 15, g = lane >> 4;
+#pragma unroll
+    for (int h = 0; h < V / 8; ++h) {
+      const int row = 8 * h + (m & 7);
+      const int pair = h == 0 ? (m >> 3) : 1 - (m >> 3);
+      col[h] = n0 + 32 * pair + 16 * (g & 1) + 8 * (g >> 1);
+      voff[h] = ((uint32_t)row * (uint32_t)N + (uint32_t)col[h]) * 2u;
+    }
+  }
+  __device__ __forceinline__ void store(const floatx4 (&acc)[4], __amdgpu_buffer_rsrc_t srd, uint32_t crow, int N) const {
+    // pr[pair][0..3]: after the swaps, lane (m, g) holds columns 8 * (g >> 1) .. + 7 of tile
+    // 2 * pair + (g & 1), row m
+    uint32_t pr[2][4];
+#pragma unroll
+    for (int pair = 0; pair < 2; ++pair) {
+      uint32_t pk[2][2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+          typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+          const half2v hv = {(_Float16)acc[2 * pair + t][2 * w], (_Float16)acc[2 * pair + t][2 * w + 1]};  // round to nearest even
+          pk[t][w] = __builtin_bit_cast(uint32_t, hv);
+        }
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        // odd rows of the first operand <-> even rows of the second
+        const auto sw = __builtin_amdgcn_permlane16_swap(pk[0][w], pk[1][w], false, false);
+        pr[pair][w] = sw[0];      // lane group g: columns 4 * (g & ~1) .. + 3 of tile 2 * pair + (g & 1)
+        pr[pair][2 + w] = sw[1];  // and the four columns after them
+      }
+    }
+#pragma unroll
+    for (int h = 0; h < V / 8; ++h) {
+      uintx4 line;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        line[r] = h == 0 ? dpp_from_m_minus_8(pr[0][r], pr[1][r]) : dpp_from_m_plus_8(pr[0][r], pr[1][r]);
+      if (col[h] < N) slab_store_line(line, srd, voff[h], crow);
+    }
   }
 };
 
@@ -438,28 +538,14 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
 
   // ---- per-lane constants
   unsigned char *val_tile = lds + tiles_off + wave * wave_lds_bytes(V);
-  unsigned char *stage = val_tile + val_tile_bytes(V);
   constexpr uint32_t kLaneBytes = V * 2u * 32u / 64u;
   unsigned char *val_dst = val_tile + lane * kLaneBytes;
   // value tile rows are V*2 bytes; transpose read h picks rows 8g + 4h + m/4
   const uint32_t a_off = (uint32_t)(8 * g + (m >> 2)) * (V * 2u) + (uint32_t)(m & 3) * 8u;
   const uint32_t slot0 = (uint32_t)(8 * g + (m >> 2));
   const uint32_t b_lane_off = (uint32_t)(m & 3) * 8u;
-  // Accumulator q of lane (m, g) holds rows 4g .. 4g+3 of column n0 + 16q + m.  A finished tile goes
-  // to C in passes of 8 rows x 128 bytes: the lanes owning those rows write their elements into the
-  // staging tile, then every lane reads 16 contiguous bytes of one row and stores them, so a store
-  // instruction writes eight full 128-byte lines.
-  constexpr int kColsPerPass = 128 / (int)sizeof(OutT);  // 32 fp32 or 64 fp16 columns
-  constexpr int kTilesPerPass = kColsPerPass / 16;        // accumulators per pass
-  constexpr int kPasses = 64 / kColsPerPass;
-  unsigned char *stage_w = stage + (4 * (g & 1)) * kStageStride + m * (int)sizeof(OutT);
-  const unsigned char *stage_r = stage + (lane >> 3) * kStageStride + (lane & 7) * 16;
-  const uint32_t c_voff = ((uint32_t)(lane >> 3) * (uint32_t)p.N + (uint32_t)n0) * (uint32_t)sizeof(OutT) +
-                          (uint32_t)(lane & 7) * 16u;
-  bool pass_ok[kPasses];
-#pragma unroll
-  for (int ps = 0; ps < kPasses; ++ps)
-    pass_ok[ps] = n0 + ps * kColsPerPass + (lane & 7) * (16 / (int)sizeof(OutT)) < p.N;
+  SlabStore<V, OutT> out;
+  out.init(lane, n0, p.N);
   // One buffer descriptor spans this batch element's C (the launcher checks it is below 4 GiB).
   const uint32_t c_vrow_bytes = (uint32_t)V * (uint32_t)p.N * (uint32_t)sizeof(OutT);
   const __amdgpu_buffer_rsrc_t srd_c = make_srd(reinterpret_cast<OutT *>(p.C) + (int64_t)batch * p.stride_C,
@@ -493,10 +579,11 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
   SlabLoads<V> ld[kSlabRing];
 #pragma unroll
   for (int i = 0; i < kSlabRing - 1; ++i) {
-    if (head.valid) {
-      slab_issue<V>(ld[i], head.kc, head.end, lane, slot0, srd_cols, vals);
-      cursor_advance<true>(head, rows);
-    }
+    // Loads are issued whether or not the head still has a step (an exhausted head has kc = end = 0:
+    // the value load is out of bounds and returns zeros), so that the number of loads in flight
+    // behind any ring slot is a compile-time constant and the waits below can be exact.
+    slab_issue<V>(ld[i], head.kc, head.end, lane, slot0, srd_cols, vals);
+    if (head.valid) cursor_advance<true>(head, rows);
   }
   // the value tile of the first step
   *reinterpret_cast<typename SlabVals<V>::type *>(val_dst) = ld[0].vraw;
@@ -508,10 +595,8 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
     for (int u = 0; u < kSlabRing; ++u) {
       constexpr int R = kSlabRing;
       const int cur = u, nxt = (u + 1) % R, fill = (u + R - 1) % R;
-      if (head.valid) {
-        slab_issue<V>(ld[fill], head.kc, head.end, lane, slot0, srd_cols, vals);
-        cursor_advance<true>(head, rows);
-      }
+      slab_issue<V>(ld[fill], head.kc, head.end, lane, slot0, srd_cols, vals);
+      if (head.valid) cursor_advance<true>(head, rows);
       const int row = tail.row;
       const int left = tail.end - tail.kc;  // vectors of this vector-row from this step on
       cursor_advance<false>(tail, rows);
@@ -545,32 +630,14 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
       if (first) {
         const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int q = 0; q < 4; ++q) acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a.h, b[q].h, zero, 0, 0, 0);
+        for (int q = 0; q < 4; ++q) acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[q].h, a.h, zero, 0, 0, 0);
       } else {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a.h, b[q].h, acc[q], 0, 0, 0);
+        for (int q = 0; q < 4; ++q) acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[q].h, a.h, acc[q], 0, 0, 0);
       }
       first = left <= 32;
       if (first) {  // last step of the vector-row: write its V x 64 tile of C
-        const uint32_t crow = (uint32_t)row * c_vrow_bytes;
-#pragma unroll
-        for (int vh = 0; vh < V / 8; ++vh) {
-#pragma unroll
-          for (int ps = 0; ps < kPasses; ++ps) {
-            if ((g >> 1) == vh) {
-#pragma unroll
-              for (int qi = 0; qi < kTilesPerPass; ++qi)
-#pragma unroll
-                for (int rr = 0; rr < 4; ++rr)
-                  StageElem<OutT>::put(stage_w + rr * kStageStride + qi * 16 * (int)sizeof(OutT),
-                                       acc[ps * kTilesPerPass + qi][rr]);
-            }
-            const uintx4 line = *reinterpret_cast<const uintx4 *>(stage_r);
-            if (pass_ok[ps])
-              __builtin_amdgcn_raw_buffer_store_b128(line, srd_c, c_voff + ps * 128,
-                                                     crow + (uint32_t)vh * 8u * (uint32_t)p.N * (uint32_t)sizeof(OutT), 0);
-          }
-        }
+        out.store(acc, srd_c, (uint32_t)row * c_vrow_bytes, p.N);
       }
       if (!tail.valid) {
         asm volatile("" ::"v"(touch_sink));  // the warming loads may still be writing this register
@@ -617,7 +684,7 @@ int set_kernel_override(int which) {
   return old;
 }
 
-static constexpr int kSlabMaxK = 1128;  // slab + zero row + 8 x (value tile + staging tile) must fit in 160 KB of LDS
+static constexpr int kSlabMaxK = 1200;  // slab + zero row + 8 value tiles + row queues must fit in 160 KB of LDS
 
 template <int V, typename OutT>
 static hipError_t launch_slab(const SpmmArgs &a, hipStream_t stream) {

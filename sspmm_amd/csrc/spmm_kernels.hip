@@ -221,9 +221,9 @@ __global__ __launch_bounds__(64) void spmm_gather_kernel(const SpmmArgs p) {
 // and 4 MFMAs, with no byte shuffling in registers.  A 16-lane group of a slab read touches four
 // different rows of B at the same column offset; the 32-byte segments of slab row c are stored
 // XOR-swizzled by (c >> 1) & 3 so that those rows spread over the LDS banks.
-// Waves draw vector-rows from a counter in LDS, so ragged rows balance inside the workgroup, and
-// the loads of a step are issued two steps ahead (across vector-row boundaries).  Row K of the
-// slab is all zeros: unused k slots of a partial step point there.
+// The vector-rows of a row block are dealt to the waves round-robin, and the loads of a step are
+// issued kSlabRing - 1 steps ahead (across vector-row boundaries).  Row K of the slab is all
+// zeros: unused k slots of a partial step point there.
 static constexpr int kSlabWaves = 8;
 static constexpr int kSlabThreads = kSlabWaves * 64;
 static constexpr int kSlabRowBytes = 128;       // 64 columns of fp16
@@ -265,67 +265,46 @@ struct SlabLoads {
   typename SlabVals<V>::type vraw;
 };
 
-// Walks one wave's sequence of steps.  Waves draw the vector-rows of their row block from a counter
-// in LDS, so ragged rows and uneven memory latency balance inside the workgroup; a vector-row of n
-// vectors is ceil(n / 32) steps, and an empty vector-row is one step without vectors (its zeros
-// still have to be written).  Two cursors run over the same sequence: the head issues the loads of
-// a step, the tail, kSlabRing - 1 steps behind it, consumes them.  The head records the rows it
-// drew in a small per-wave queue in LDS from which the tail reads them back.  Either cursor asks
-// for the offsets of its following vector-row one row ahead, so that the LDS round trip and the
-// scalar loads are off the critical path.
+// Walks one wave's sequence of steps.  The (vector-row, first vector, end vector) triples of the
+// row block are copied into a table in LDS when the workgroup starts; wave w takes the positions
+// w, w + 8, w + 16, ... of the block, so finding the next vector-row is one broadcast LDS read and
+// no scalar-memory or atomic round trip sits in the main loop.  A vector-row of n vectors is
+// ceil(n / 32) steps, and an empty vector-row is one step without vectors (its zeros still have
+// to be written).  Two cursors run over the same sequence: the head issues the loads of a step,
+// the tail, kSlabRing - 1 steps behind it, consumes them.  Either cursor reads the table entry of
+// its following vector-row one row ahead, so that the LDS latency is off the critical path.
+typedef int intx4 __attribute__((ext_vector_type(4)));
 struct SlabCursor {
   int row, kc, end;  // current step: vectors [kc, min(kc + 32, end)) of vector-row `row`
   bool valid;
-  int next_row, next_kc, next_end;
+  intx4 next;        // table entry of the following vector-row (still in vector registers)
   bool next_valid;
-  int count;  // rows requested so far (index into the per-wave queue)
+  int count;         // rows requested so far
 };
 
-struct SlabRows {  // what the cursors need to find rows
-  int *counter;    // LDS: next undrawn position of the row block
-  int *queue;      // LDS: this wave's queue of drawn positions (kSlabQueue entries)
-  int row_lo, row_hi, lane;
-  const int32_t *__restrict__ row_offsets;
-  const int32_t *__restrict__ row_indices;
+struct SlabRows {      // what the cursors need to find rows
+  const intx4 *table;  // LDS: n_rows entries (row, first vector, end vector, -) and an all-zero entry behind them
+  int n_rows, wave;
 };
-static constexpr int kSlabQueue = 16;
 
-template <bool HEAD>
 __device__ __forceinline__ void cursor_prefetch(SlabCursor &c, const SlabRows &rows) {
-  int pos = 0;
-  int *slot = rows.queue + (c.count & (kSlabQueue - 1));
-  if (HEAD) {
-    if (rows.lane == 0) {
-      pos = atomicAdd(rows.counter, 1) + rows.row_lo;
-      *slot = pos;
-    }
-  } else {
-    if (rows.lane == 0) pos = *slot;
-  }
-  pos = __builtin_amdgcn_readfirstlane(pos);
+  const int idx = rows.wave + kSlabWaves * c.count;
   ++c.count;
-  c.next_valid = pos < rows.row_hi;
-  c.next_row = c.next_kc = c.next_end = 0;
-  if (c.next_valid) {
-    c.next_row = rows.row_indices ? rows.row_indices[pos] : pos;
-    c.next_kc = rows.row_offsets[c.next_row];
-    c.next_end = rows.row_offsets[c.next_row + 1];
-  }
+  c.next_valid = idx < rows.n_rows;
+  c.next = rows.table[min(idx, rows.n_rows)];
 }
 
-template <bool HEAD>
 __device__ __forceinline__ void cursor_take_next(SlabCursor &c, const SlabRows &rows) {
-  c.row = c.next_row;
-  c.kc = c.next_kc;
-  c.end = c.next_end;
+  c.row = __builtin_amdgcn_readfirstlane(c.next[0]);
+  c.kc = __builtin_amdgcn_readfirstlane(c.next[1]);
+  c.end = __builtin_amdgcn_readfirstlane(c.next[2]);
   c.valid = c.next_valid;
-  if (c.valid) cursor_prefetch<HEAD>(c, rows);
+  cursor_prefetch(c, rows);
 }
 
-template <bool HEAD>
 __device__ __forceinline__ void cursor_advance(SlabCursor &c, const SlabRows &rows) {
   c.kc += 32;
-  if (c.kc >= c.end) cursor_take_next<HEAD>(c, rows);
+  if (c.kc >= c.end) cursor_take_next(c, rows);
 }
 
 template <int V>
@@ -349,7 +328,7 @@ __device__ __forceinline__ void slab_issue(SlabLoads<V> &r, int kc, int end, int
 // loads, and the wait cannot pass early whatever the stores do; stores in flight only make it
 // pass later.  The trailing s_nop covers the cycles in which the store still reads its data registers.
 __device__ __forceinline__ void slab_store_line(uintx4 line, __amdgpu_buffer_rsrc_t srd, uint32_t voff, uint32_t soff) {
-  asm volatile("buffer_store_dwordx4 %0, %1, %2, %3 offen\n\ts_nop 1" ::"v"(line), "v"(voff), "s"(srd), "s"(soff));
+  asm volatile("buffer_store_dwordx4 %0, %1, %2, %3 offen nt\n\ts_nop 1" ::"v"(line), "v"(voff), "s"(srd), "s"(soff));
 }
 
 // Writing a finished V x 64 tile of C.  The MFMAs run with the slab as their first operand, so
@@ -532,8 +511,20 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
   const uint32_t zero_row = (uint32_t)p.K;
   if (tid < 8) *reinterpret_cast<uintx4 *>(lds + zero_row * kSlabRowBytes + tid * 16) = uintx4{0u, 0u, 0u, 0u};
   const uint32_t tiles_off = (zero_row + 1u) * kSlabRowBytes;
-  int *counter = reinterpret_cast<int *>(lds + tiles_off + kSlabWaves * wave_lds_bytes(V));
-  if (tid == 0) *counter = 0;
+  // ---- the row table of this block
+  const int row_lo = (int)(rb * p.rows_per_block);
+  const int row_hi = min(p.m_vec, row_lo + (int)p.rows_per_block);
+  const int n_rows = row_hi - row_lo;
+  intx4 *table = reinterpret_cast<intx4 *>(lds + tiles_off + kSlabWaves * wave_lds_bytes(V));
+  for (int i = tid; i <= n_rows; i += kSlabThreads) {
+    intx4 e = {0, 0, 0, 0};
+    if (i < n_rows) {
+      e[0] = row_indices ? row_indices[row_lo + i] : row_lo + i;
+      e[1] = row_offsets[e[0]];
+      e[2] = row_offsets[e[0] + 1];
+    }
+    table[i] = e;
+  }
   __syncthreads();
 
   // ---- per-lane constants
@@ -550,31 +541,23 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
   const uint32_t c_vrow_bytes = (uint32_t)V * (uint32_t)p.N * (uint32_t)sizeof(OutT);
   const __amdgpu_buffer_rsrc_t srd_c = make_srd(reinterpret_cast<OutT *>(p.C) + (int64_t)batch * p.stride_C,
                                                 (uint32_t)p.m_vec * c_vrow_bytes);
-  // Row bookkeeping is read through the restrict-qualified kernel arguments so that it goes
-  // through the scalar cache and does not share the vector-memory counter with the stores of C.
   const uint32_t nvec = (uint32_t)row_offsets[p.m_vec];
   const __amdgpu_buffer_rsrc_t srd_cols = make_srd(p.col_idx, nvec * 4u);
 
   // ---- this wave's stream of steps
-  const int row_lo = (int)(rb * p.rows_per_block);
-  const int row_hi = min(p.m_vec, row_lo + (int)p.rows_per_block);
   SlabRows rows;
-  rows.counter = counter;
-  rows.queue = counter + 1 + wave * kSlabQueue;
-  rows.row_lo = row_lo;
-  rows.row_hi = row_hi;
-  rows.lane = lane;
-  rows.row_offsets = row_offsets;
-  rows.row_indices = row_indices;
+  rows.table = table;
+  rows.n_rows = n_rows;
+  rows.wave = wave;
   SlabCursor head;  // issues loads
   head.count = 0;
-  cursor_prefetch<true>(head, rows);
-  cursor_take_next<true>(head, rows);
+  cursor_prefetch(head, rows);
+  cursor_take_next(head, rows);
   if (!head.valid) return;
   SlabCursor tail;  // consumes them
   tail.count = 0;
-  cursor_prefetch<false>(tail, rows);
-  cursor_take_next<false>(tail, rows);
+  cursor_prefetch(tail, rows);
+  cursor_take_next(tail, rows);
 
   SlabLoads<V> ld[kSlabRing];
 #pragma unroll
@@ -583,7 +566,7 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
     // the value load is out of bounds and returns zeros), so that the number of loads in flight
     // behind any ring slot is a compile-time constant and the waits below can be exact.
     slab_issue<V>(ld[i], head.kc, head.end, lane, slot0, srd_cols, vals);
-    if (head.valid) cursor_advance<true>(head, rows);
+    if (head.valid) cursor_advance(head, rows);
   }
   // the value tile of the first step
   *reinterpret_cast<typename SlabVals<V>::type *>(val_dst) = ld[0].vraw;
@@ -596,10 +579,10 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
       constexpr int R = kSlabRing;
       const int cur = u, nxt = (u + 1) % R, fill = (u + R - 1) % R;
       slab_issue<V>(ld[fill], head.kc, head.end, lane, slot0, srd_cols, vals);
-      if (head.valid) cursor_advance<true>(head, rows);
+      if (head.valid) cursor_advance(head, rows);
       const int row = tail.row;
       const int left = tail.end - tail.kc;  // vectors of this vector-row from this step on
-      cursor_advance<false>(tail, rows);
+      cursor_advance(tail, rows);
 
       // A operand: this step's value tile
       Half8Bits a;
@@ -684,7 +667,8 @@ int set_kernel_override(int which) {
   return old;
 }
 
-static constexpr int kSlabMaxK = 1200;  // slab + zero row + 8 value tiles + row queues must fit in 160 KB of LDS
+static constexpr uint32_t kSlabMaxRows = 255;  // vector-rows per workgroup (row table of 256 entries)
+static constexpr int kSlabMaxK = 1180;  // slab + zero row + 8 value tiles + row table must fit in 160 KB of LDS
 
 template <int V, typename OutT>
 static hipError_t launch_slab(const SpmmArgs &a, hipStream_t stream) {
@@ -692,13 +676,18 @@ static hipError_t launch_slab(const SpmmArgs &a, hipStream_t stream) {
   p.n_tiles = (uint32_t)((a.N + 63) / 64);
   p.n_slabs = p.n_tiles * (uint32_t)a.batch;
   // Aim at ~4 workgroups per CU, but keep at least 32 vector-rows per workgroup so that the copy
-  // of the slab into LDS stays a small part of the workgroup's traffic.
+  // of the slab into LDS stays a small part of the workgroup's traffic, and at most kSlabMaxRows
+  // (the row table in LDS).
   const uint32_t rb_target = p.n_slabs >= 1024u ? 1u : 1024u / p.n_slabs;
   uint32_t rows = ((uint32_t)a.m_vec + rb_target - 1u) / rb_target;
   if (rows < 32u) rows = 32u;
+  if (rows > kSlabMaxRows) {
+    const uint32_t blocks = ((uint32_t)a.m_vec + kSlabMaxRows - 1u) / kSlabMaxRows;
+    rows = ((uint32_t)a.m_vec + blocks - 1u) / blocks;
+  }
   p.rows_per_block = rows;
   p.row_blocks = ((uint32_t)a.m_vec + rows - 1u) / rows;
-  const size_t lds = (size_t)(a.K + 1) * kSlabRowBytes + kSlabWaves * wave_lds_bytes(V) + 4 * (1 + kSlabWaves * kSlabQueue);
+  const size_t lds = (size_t)(a.K + 1) * kSlabRowBytes + kSlabWaves * wave_lds_bytes(V) + 16 * (rows + 1);
   auto kern = spmm_slab_kernel<V, OutT>;
   static size_t lds_allowed = 64 * 1024;  // per instantiation
   if (lds > lds_allowed) {

@@ -471,6 +471,17 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
   const __amdgpu_buffer_rsrc_t srd_b = make_srd(bmat, b_bytes);
   uint32_t touch_sink = 0;  // keeps the destination register of the warming loads reserved
 
+  // ---- the row table of this block: thread i fetches entry i (kSlabMaxRows < kSlabThreads).  The
+  // loads go out first so that they do not queue behind the slab and the warming loads.
+  const int row_lo = (int)(rb * p.rows_per_block);
+  const int row_hi = min(p.m_vec, row_lo + (int)p.rows_per_block);
+  const int n_rows = row_hi - row_lo;
+  intx4 table_entry = {0, 0, 0, 0};
+  if (tid < n_rows) {
+    table_entry[0] = row_indices ? row_indices[row_lo + tid] : row_lo + tid;
+    table_entry[1] = row_offsets[table_entry[0]];
+    table_entry[2] = row_offsets[table_entry[0] + 1];
+  }
   // ---- stage the slab: unit u = 16 bytes = columns n0 + 8*(u % 8) .. +7 of row u / 8; the
   // 32-byte segment (u % 8) / 2 of row c lands at segment ((u % 8) / 2) ^ ((c >> 1) & 3).
   const uint32_t units = (uint32_t)p.K * 8u;
@@ -498,9 +509,7 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
   // loads of the slab; nothing ever waits for these loads, and the main loop then finds the
   // lines in the L2 or on their way to it.  One 4-byte load per lane touches 64 lines per instruction.
   if (row_indices == nullptr) {
-    const int row_lo_p = (int)(rb * p.rows_per_block);
-    const int row_hi_p = min(p.m_vec, row_lo_p + (int)p.rows_per_block);
-    const uint32_t lo = (uint32_t)row_offsets[row_lo_p] * (V * 2u), hi = (uint32_t)row_offsets[row_hi_p] * (V * 2u);
+    const uint32_t lo = (uint32_t)row_offsets[row_lo] * (V * 2u), hi = (uint32_t)row_offsets[row_hi] * (V * 2u);
     const __amdgpu_buffer_rsrc_t srd_touch = make_srd(vals, hi);
     uint32_t sink = 0;
     for (uint32_t off = (lo & ~127u) + (uint32_t)tid * 128u; off < hi; off += kSlabThreads * 128u)
@@ -511,20 +520,8 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
   const uint32_t zero_row = (uint32_t)p.K;
   if (tid < 8) *reinterpret_cast<uintx4 *>(lds + zero_row * kSlabRowBytes + tid * 16) = uintx4{0u, 0u, 0u, 0u};
   const uint32_t tiles_off = (zero_row + 1u) * kSlabRowBytes;
-  // ---- the row table of this block
-  const int row_lo = (int)(rb * p.rows_per_block);
-  const int row_hi = min(p.m_vec, row_lo + (int)p.rows_per_block);
-  const int n_rows = row_hi - row_lo;
   intx4 *table = reinterpret_cast<intx4 *>(lds + tiles_off + kSlabWaves * wave_lds_bytes(V));
-  for (int i = tid; i <= n_rows; i += kSlabThreads) {
-    intx4 e = {0, 0, 0, 0};
-    if (i < n_rows) {
-      e[0] = row_indices ? row_indices[row_lo + i] : row_lo + i;
-      e[1] = row_offsets[e[0]];
-      e[2] = row_offsets[e[0] + 1];
-    }
-    table[i] = e;
-  }
+  if (tid <= n_rows) table[tid] = table_entry;
   __syncthreads();
 
   // ---- per-lane constants

@@ -206,11 +206,17 @@ __global__ __launch_bounds__(64) void spmm_gather_kernel(const SpmmArgs p) {
 // Slab kernel: B resident in LDS, operands formed by LDS transpose reads.
 //
 // When K is small enough that a 64-column slab of B (K rows x 128 bytes) fits in the 160 KB of
-// LDS, a workgroup of 8 waves copies the slab into LDS once with coalesced 16-byte loads and
-// then walks a block of vector-rows against it, so HBM/L2 only see each slab once per row
-// block, the value vectors, the column indices and the stores of C.
+// LDS, a workgroup copies the slab into LDS with coalesced 16-byte loads and then walks a block of
+// vector-rows against it, so HBM/L2 only see each slab once per row block, the value vectors, the
+// column indices and the stores of C.
 //
-// ds_read_b64_tr_b16 is what makes this cheap.  Within 16 lanes, lane n receives element n of the
+// The kernel is persistent: one workgroup of 16 waves per CU walks a list of work items
+// (slab, row block).  Where two slabs fit in LDS the next item's slab and row table are fetched
+// into registers while the current item is computed and are written to the other LDS buffer when
+// the item is done, so the copy of B never stalls the CU after its first item; larger K runs the
+// same loop with one buffer.  Items that follow each other on the same slab reuse it.
+//
+// ds_read_b64_tr_b16 is what makes the inner loop cheap.  Within 16 lanes, lane n receives element n of the
 // four 32-byte runs addressed by lanes 0-3, 4-7, 8-11, 12-15: four rows that are contiguous in the
 // column direction come back as "four k of one column", which is the MFMA operand layout.  Per
 // step of 32 vectors a wave therefore issues
@@ -222,9 +228,9 @@ __global__ __launch_bounds__(64) void spmm_gather_kernel(const SpmmArgs p) {
 // different rows of B at the same column offset; the 32-byte segments of slab row c are stored
 // XOR-swizzled by (c >> 1) & 3 so that those rows spread over the LDS banks.
 // The vector-rows of a row block are dealt to the waves round-robin, and the loads of a step are
-// issued kSlabRing - 1 steps ahead (across vector-row boundaries).  Row K of the slab is all
+// issued a few steps ahead (across vector-row boundaries).  Row K of the slab is all
 // zeros: unused k slots of a partial step point there.
-static constexpr int kSlabWaves = 8;
+static constexpr int kSlabWaves = 16;
 static constexpr int kSlabThreads = kSlabWaves * 64;
 static constexpr int kSlabRowBytes = 128;       // 64 columns of fp16
 // Per-wave LDS: the value tile of a step (32 vectors x V halfs; the V = 8 transpose read touches 16
@@ -232,7 +238,9 @@ static constexpr int kSlabRowBytes = 128;       // 64 columns of fp16
 static constexpr int val_tile_bytes(int V) { return V == 8 ? 528 : 1024; }
 static constexpr int wave_lds_bytes(int V) { return val_tile_bytes(V); }
 
-static constexpr int kSlabRing = 8;  // steps whose loads are in flight or waiting in registers
+// steps whose loads are in flight or waiting in registers (bounded by the 128 registers a lane has
+// with 16 waves per CU)
+static constexpr int slab_ring(int V) { return V == 8 ? 6 : 5; }
 
 typedef short shortx4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) shortx4 lds_shortx4;
@@ -260,9 +268,11 @@ struct SlabVals<16> {
 };
 
 template <int V>
-struct SlabLoads {
-  uint32_t col[2];  // column index of k slots 8g + m/4 and 8g + 4 + m/4
+struct SlabLoads {    // what the head records for a step; the step consumes it slab_ring(V) - 1 steps later
+  uint32_t col[2];    // column index of k slots 8g + m/4 and 8g + 4 + m/4
   typename SlabVals<V>::type vraw;
+  int row, left;      // (wave-uniform) vector-row and its vectors from this step on
+  bool valid;         // (wave-uniform) false once the wave has run out of steps
 };
 
 // Walks one wave's sequence of steps.  The (vector-row, first vector, end vector) triples of the
@@ -270,9 +280,10 @@ struct SlabLoads {
 // w, w + 8, w + 16, ... of the block, so finding the next vector-row is one broadcast LDS read and
 // no scalar-memory or atomic round trip sits in the main loop.  A vector-row of n vectors is
 // ceil(n / 32) steps, and an empty vector-row is one step without vectors (its zeros still have
-// to be written).  Two cursors run over the same sequence: the head issues the loads of a step,
-// the tail, kSlabRing - 1 steps behind it, consumes them.  Either cursor reads the table entry of
-// its following vector-row one row ahead, so that the LDS latency is off the critical path.
+// to be written).  The cursor runs slab_ring(V) - 1 steps ahead of the arithmetic: it issues the
+// loads of a step and records the step's vector-row and length in the ring slot that receives
+// them.  It reads the table entry of its following vector-row one row ahead, so that the LDS
+// latency is off the critical path.
 typedef int intx4 __attribute__((ext_vector_type(4)));
 struct SlabCursor {
   int row, kc, end;  // current step: vectors [kc, min(kc + 32, end)) of vector-row `row`
@@ -308,8 +319,11 @@ __device__ __forceinline__ void cursor_advance(SlabCursor &c, const SlabRows &ro
 }
 
 template <int V>
-__device__ __forceinline__ void slab_issue(SlabLoads<V> &r, int kc, int end, int lane, uint32_t slot0,
+__device__ __forceinline__ void slab_issue(SlabLoads<V> &r, int row, int kc, int end, bool valid, int lane, uint32_t slot0,
                                            __amdgpu_buffer_rsrc_t srd_cols, const uint16_t *vals) {
+  r.row = row;
+  r.left = end - kc;
+  r.valid = valid;
   r.col[0] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(srd_cols, (kc + (int)slot0) * 4, 0, 0);
   r.col[1] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(srd_cols, (kc + (int)slot0) * 4 + 16, 0, 0);
   // The value descriptor ends with the vector-row: vectors past it read as zero.
@@ -434,167 +448,67 @@ struct SlabStore<V, _Float16> {
   }
 };
 
+// Per-lane constants of the inner loop and the operands of the current work item.
 template <int V, typename OutT>
-__global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs p,
-                                                                 const int32_t *__restrict__ row_offsets,
-                                                                 const int32_t *__restrict__ row_indices) {
-  extern __shared__ __align__(16) unsigned char lds[];
-  const uint32_t id = blockIdx.x;
-  // The hardware deals consecutive block ids round-robin to the 8 XCDs, each with its own L2, so
-  // blocks whose ids are equal modulo 8 share an L2.  With at least 8 batch elements, all blocks of
-  // one batch element (every column tile and row block) are given the same residue: the value
-  // vectors, read once per column tile, and the slab, read once per row block, then come from
-  // that L2 after the first touch.  With fewer batch elements the residue is taken from the slab.
-  const uint32_t xcd = id & 7u, qd = id >> 3;
-  uint32_t rb, tile, batch;
-  if (p.group_by_batch) {
-    const uint32_t per_batch = p.n_tiles * p.row_blocks;
-    const uint32_t rem = qd % per_batch;
-    batch = (qd / per_batch) * 8u + xcd;
-    tile = rem / p.row_blocks;
-    rb = rem % p.row_blocks;
-    if (batch >= (uint32_t)p.batch) return;
-  } else {
-    rb = qd % p.row_blocks;
-    const uint32_t slab_id = (qd / p.row_blocks) * 8u + xcd;
-    if (slab_id >= p.n_slabs) return;
-    tile = slab_id % p.n_tiles;
-    batch = slab_id / p.n_tiles;
-  }
+struct SlabCtx {
+  int lane;
+  uint32_t slot0, a_off, b_lane_off, zero_row;
+  unsigned char *val_tile, *val_dst;
+  __amdgpu_buffer_rsrc_t srd_cols;
+  int N;
+  uint32_t c_vrow_bytes;
+};
 
-  const int tid = threadIdx.x, lane = tid & 63, m = lane & 15, g = lane >> 4;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // tell the compiler it is wave-uniform
-  const int n0 = (int)tile * 64;
-  const uint16_t *vals = p.values + (int64_t)batch * p.stride_values;
-  const uint16_t *bmat = p.B + (int64_t)batch * p.stride_B;
-  const uint32_t b_bytes = (uint32_t)p.K * (uint32_t)p.N * 2u;
-  const __amdgpu_buffer_rsrc_t srd_b = make_srd(bmat, b_bytes);
-  uint32_t touch_sink = 0;  // keeps the destination register of the warming loads reserved
-
-  // ---- the row table of this block: thread i fetches entry i (kSlabMaxRows < kSlabThreads).  The
-  // loads go out first so that they do not queue behind the slab and the warming loads.
-  const int row_lo = (int)(rb * p.rows_per_block);
-  const int row_hi = min(p.m_vec, row_lo + (int)p.rows_per_block);
-  const int n_rows = row_hi - row_lo;
-  intx4 table_entry = {0, 0, 0, 0};
-  if (tid < n_rows) {
-    table_entry[0] = row_indices ? row_indices[row_lo + tid] : row_lo + tid;
-    table_entry[1] = row_offsets[table_entry[0]];
-    table_entry[2] = row_offsets[table_entry[0] + 1];
-  }
-  // ---- stage the slab: unit u = 16 bytes = columns n0 + 8*(u % 8) .. +7 of row u / 8; the
-  // 32-byte segment (u % 8) / 2 of row c lands at segment ((u % 8) / 2) ^ ((c >> 1) & 3).
-  const uint32_t units = (uint32_t)p.K * 8u;
-  const uint32_t n2 = (uint32_t)p.N * 2u;
-  for (uint32_t u0 = 0; u0 < units; u0 += kSlabThreads * 8) {
-    uintx4 d[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const uint32_t u = u0 + i * kSlabThreads + tid;
-      const uint32_t col = (uint32_t)n0 + (u & 7u) * 8u;
-      const uint32_t off = (u < units && col < (uint32_t)p.N) ? __umul24(u >> 3, n2) + col * 2u : b_bytes;
-      d[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_b, off, 0, 0));
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const uint32_t u = u0 + i * kSlabThreads + tid;
-      const uint32_t c = u >> 3;
-      const uint32_t dst = c * kSlabRowBytes + (((u & 7u) * 16u) ^ (((c >> 1) & 3u) << 5));
-      if (u < units) *reinterpret_cast<uintx4 *>(lds + dst) = d[i];
-    }
-  }
-  // ---- warm the L2 with this block's value vectors.  Under a saturating stream of C stores an
-  // HBM read takes several microseconds, far more than the register ring of the main loop covers,
-  // so every 128-byte line of the block's (contiguous) value range is touched once now, behind the
-  // loads of the slab; nothing ever waits for these loads, and the main loop then finds the
-  // lines in the L2 or on their way to it.  One 4-byte load per lane touches 64 lines per instruction.
-  if (row_indices == nullptr) {
-    const uint32_t lo = (uint32_t)row_offsets[row_lo] * (V * 2u), hi = (uint32_t)row_offsets[row_hi] * (V * 2u);
-    const __amdgpu_buffer_rsrc_t srd_touch = make_srd(vals, hi);
-    uint32_t sink = 0;
-    for (uint32_t off = (lo & ~127u) + (uint32_t)tid * 128u; off < hi; off += kSlabThreads * 128u)
-      asm volatile("buffer_load_dword %0, %1, %2, 0 offen" : "+v"(sink) : "v"(off), "s"(srd_touch) : "memory");
-    touch_sink = sink;
-  }
-
-  const uint32_t zero_row = (uint32_t)p.K;
-  if (tid < 8) *reinterpret_cast<uintx4 *>(lds + zero_row * kSlabRowBytes + tid * 16) = uintx4{0u, 0u, 0u, 0u};
-  const uint32_t tiles_off = (zero_row + 1u) * kSlabRowBytes;
-  intx4 *table = reinterpret_cast<intx4 *>(lds + tiles_off + kSlabWaves * wave_lds_bytes(V));
-  if (tid <= n_rows) table[tid] = table_entry;
-  __syncthreads();
-
-  // ---- per-lane constants
-  unsigned char *val_tile = lds + tiles_off + wave * wave_lds_bytes(V);
-  constexpr uint32_t kLaneBytes = V * 2u * 32u / 64u;
-  unsigned char *val_dst = val_tile + lane * kLaneBytes;
-  // value tile rows are V*2 bytes; transpose read h picks rows 8g + 4h + m/4
-  const uint32_t a_off = (uint32_t)(8 * g + (m >> 2)) * (V * 2u) + (uint32_t)(m & 3) * 8u;
-  const uint32_t slot0 = (uint32_t)(8 * g + (m >> 2));
-  const uint32_t b_lane_off = (uint32_t)(m & 3) * 8u;
-  SlabStore<V, OutT> out;
-  out.init(lane, n0, p.N);
-  // One buffer descriptor spans this batch element's C (the launcher checks it is below 4 GiB).
-  const uint32_t c_vrow_bytes = (uint32_t)V * (uint32_t)p.N * (uint32_t)sizeof(OutT);
-  const __amdgpu_buffer_rsrc_t srd_c = make_srd(reinterpret_cast<OutT *>(p.C) + (int64_t)batch * p.stride_C,
-                                                (uint32_t)p.m_vec * c_vrow_bytes);
-  const uint32_t nvec = (uint32_t)row_offsets[p.m_vec];
-  const __amdgpu_buffer_rsrc_t srd_cols = make_srd(p.col_idx, nvec * 4u);
-
-  // ---- this wave's stream of steps
-  SlabRows rows;
-  rows.table = table;
-  rows.n_rows = n_rows;
-  rows.wave = wave;
+// One wave's share of a work item: the vector-rows wave, wave + 16, ... of the item's row table
+// against the slab at byte offset slab_base of LDS.
+template <int V, typename OutT>
+__device__ __forceinline__ void slab_process_item(const SlabCtx<V, OutT> &x, unsigned char *lds, uint32_t slab_base,
+                                                  const SlabRows &rows, const uint16_t *vals,
+                                                  __amdgpu_buffer_rsrc_t srd_c, const SlabStore<V, OutT> &out) {
   SlabCursor head;  // issues loads
   head.count = 0;
   cursor_prefetch(head, rows);
   cursor_take_next(head, rows);
   if (!head.valid) return;
-  SlabCursor tail;  // consumes them
-  tail.count = 0;
-  cursor_prefetch(tail, rows);
-  cursor_take_next(tail, rows);
 
-  SlabLoads<V> ld[kSlabRing];
+  constexpr int R = slab_ring(V);
+  SlabLoads<V> ld[R];
 #pragma unroll
-  for (int i = 0; i < kSlabRing - 1; ++i) {
+  for (int i = 0; i < R - 1; ++i) {
     // Loads are issued whether or not the head still has a step (an exhausted head has kc = end = 0:
     // the value load is out of bounds and returns zeros), so that the number of loads in flight
     // behind any ring slot is a compile-time constant and the waits below can be exact.
-    slab_issue<V>(ld[i], head.kc, head.end, lane, slot0, srd_cols, vals);
+    slab_issue<V>(ld[i], head.row, head.kc, head.end, head.valid, x.lane, x.slot0, x.srd_cols, vals);
     if (head.valid) cursor_advance(head, rows);
   }
   // the value tile of the first step
-  *reinterpret_cast<typename SlabVals<V>::type *>(val_dst) = ld[0].vraw;
+  *reinterpret_cast<typename SlabVals<V>::type *>(x.val_dst) = ld[0].vraw;
 
+  const uint32_t lane_base = x.b_lane_off + slab_base;  // slab_base is a multiple of 128
   floatx4 acc[4];
-  bool first = true;  // first step of a vector-row: accumulate onto zero
+#pragma unroll
+  for (int q = 0; q < 4; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
   for (;;) {
 #pragma unroll
-    for (int u = 0; u < kSlabRing; ++u) {
-      constexpr int R = kSlabRing;
+    for (int u = 0; u < R; ++u) {
       const int cur = u, nxt = (u + 1) % R, fill = (u + R - 1) % R;
-      slab_issue<V>(ld[fill], head.kc, head.end, lane, slot0, srd_cols, vals);
+      slab_issue<V>(ld[fill], head.row, head.kc, head.end, head.valid, x.lane, x.slot0, x.srd_cols, vals);
       if (head.valid) cursor_advance(head, rows);
-      const int row = tail.row;
-      const int left = tail.end - tail.kc;  // vectors of this vector-row from this step on
-      cursor_advance(tail, rows);
+      const int left = ld[cur].left;
 
       // A operand: this step's value tile
       Half8Bits a;
       {
-        const uintx2 lo = lds_read_tr(val_tile, a_off);
-        const uintx2 hi = lds_read_tr(val_tile, a_off + 4u * (V * 2u));
+        const uintx2 lo = lds_read_tr(x.val_tile, x.a_off);
+        const uintx2 hi = lds_read_tr(x.val_tile, x.a_off + 4u * (V * 2u));
         a.u[0] = lo[0]; a.u[1] = lo[1]; a.u[2] = hi[0]; a.u[3] = hi[1];
       }
       // B operands: two column indices per lane; unused k slots of a partial step read the zero row
       uint32_t addr[2];
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        const uint32_t c = ((int)slot0 + 4 * h < left) ? ld[cur].col[h] : zero_row;
-        const uint32_t t = c << 4;
-        addr[h] = (t << 3) | ((t & 0x60u) | b_lane_off);
+        const uint32_t c = ((int)x.slot0 + 4 * h < left) ? ld[cur].col[h] : x.zero_row;
+        addr[h] = ((c << 7) + lane_base) | ((c << 4) & 0x60u);
       }
       Half8Bits b[4];
 #pragma unroll
@@ -605,25 +519,217 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
       }
       // the next step's value tile goes to LDS behind the reads above (LDS operations of a wave
       // execute in order)
-      if (tail.valid) *reinterpret_cast<typename SlabVals<V>::type *>(val_dst) = ld[nxt].vraw;
+      if (ld[nxt].valid) *reinterpret_cast<typename SlabVals<V>::type *>(x.val_dst) = ld[nxt].vraw;
 
-      if (first) {
-        const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int q = 0; q < 4; ++q) acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[q].h, a.h, zero, 0, 0, 0);
-      } else {
+      for (int q = 0; q < 4; ++q) acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[q].h, a.h, acc[q], 0, 0, 0);
+      if (left <= 32) {  // last step of the vector-row: write its V x 64 tile of C and start over from zero
+        out.store(acc, srd_c, (uint32_t)ld[cur].row * x.c_vrow_bytes, x.N);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[q].h, a.h, acc[q], 0, 0, 0);
+        for (int q = 0; q < 4; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
       }
-      first = left <= 32;
-      if (first) {  // last step of the vector-row: write its V x 64 tile of C
-        out.store(acc, srd_c, (uint32_t)row * c_vrow_bytes, p.N);
-      }
-      if (!tail.valid) {
-        asm volatile("" ::"v"(touch_sink));  // the warming loads may still be writing this register
-        return;
+      if (!ld[nxt].valid) return;
+    }
+  }
+}
+
+// A work item of the slab kernel.
+struct SlabItem {
+  uint32_t batch, tile, rb;
+};
+
+// Item `it` of XCD `xcd`: slabs are dealt to the XCDs so that workgroups sharing an L2 share
+// operands.  With at least 8 batch elements a batch element (all its column tiles and row blocks)
+// stays on one XCD: its value vectors, read once per column tile, then come from that L2 after
+// the first touch.  With fewer batch elements the slabs are dealt round-robin.
+__device__ __forceinline__ SlabItem slab_item(const SpmmArgs &p, uint32_t xcd, uint32_t it) {
+  SlabItem r;
+  const uint32_t q = it / p.row_blocks;
+  r.rb = it % p.row_blocks;
+  if (p.group_by_batch) {
+    r.batch = (q / p.n_tiles) * 8u + xcd;
+    r.tile = q % p.n_tiles;
+  } else {
+    const uint32_t slab_id = q * 8u + xcd;
+    r.tile = slab_id % p.n_tiles;
+    r.batch = slab_id / p.n_tiles;
+  }
+  return r;
+}
+
+// The slab of an item on its way from global memory to LDS.  Unit u = 16 bytes = columns
+// n0 + 8 * (u % 8) .. + 7 of row u / 8; the 32-byte segment (u % 8) / 2 of row c lands at segment
+// ((u % 8) / 2) ^ ((c >> 1) & 3).
+static constexpr int kSlabFetchUnits = 4;  // 16-byte units per thread held in registers (double-buffered mode)
+struct SlabFetch {
+  uintx4 d[kSlabFetchUnits];
+  intx4 entry;
+};
+
+__device__ __forceinline__ uint32_t slab_unit_src(const SpmmArgs &p, uint32_t u, uint32_t units, uint32_t n0, uint32_t b_bytes) {
+  const uint32_t col = n0 + (u & 7u) * 8u;
+  return (u < units && col < (uint32_t)p.N) ? __umul24(u >> 3, (uint32_t)p.N * 2u) + col * 2u : b_bytes;  // b_bytes: out of bounds, reads zeros
+}
+__device__ __forceinline__ uint32_t slab_unit_dst(uint32_t u) {
+  const uint32_t c = u >> 3;
+  return c * kSlabRowBytes + (((u & 7u) * 16u) ^ (((c >> 1) & 3u) << 5));
+}
+
+__device__ __forceinline__ intx4 slab_table_fetch(const SpmmArgs &p, const int32_t *__restrict__ row_offsets,
+                                                  const int32_t *__restrict__ row_indices, uint32_t rb, int tid) {
+  const int row_lo = (int)(rb * p.rows_per_block);
+  const int n_rows = min(p.m_vec, row_lo + (int)p.rows_per_block) - row_lo;
+  intx4 e = {0, 0, 0, 0};
+  if (tid < n_rows) {
+    e[0] = row_indices ? row_indices[row_lo + tid] : row_lo + tid;
+    e[1] = row_offsets[e[0]];
+    e[2] = row_offsets[e[0] + 1];
+  }
+  return e;
+}
+
+template <int V, typename OutT, bool DOUBLE>
+__global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs p,
+                                                                 const int32_t *__restrict__ row_offsets,
+                                                                 const int32_t *__restrict__ row_indices) {
+  extern __shared__ __align__(16) unsigned char lds[];
+  // The hardware deals consecutive workgroup ids round-robin to the 8 XCDs, each with its own L2.
+  const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3, wgs_per_xcd = gridDim.x >> 3;
+  const uint32_t slabs_x = p.group_by_batch ? (((uint32_t)p.batch + 7u - xcd) / 8u) * p.n_tiles : (p.n_slabs + 7u - xcd) / 8u;
+  const uint32_t items_x = slabs_x * p.row_blocks;
+  uint32_t it = (uint32_t)(((uint64_t)slot * items_x) / wgs_per_xcd);
+  const uint32_t it_end = (uint32_t)(((uint64_t)(slot + 1u) * items_x) / wgs_per_xcd);
+  if (it >= it_end) return;
+
+  const int tid = threadIdx.x, lane = tid & 63, m = lane & 15, g = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // tell the compiler it is wave-uniform
+  const uint32_t b_bytes = (uint32_t)p.K * (uint32_t)p.N * 2u;
+  const uint32_t units = (uint32_t)p.K * 8u;
+
+  // ---- LDS: slab 0, [slab 1], value tiles, row table 0, row table 1
+  const uint32_t zero_row = (uint32_t)p.K;
+  const uint32_t slab_bytes = (zero_row + 1u) * kSlabRowBytes;
+  const uint32_t tiles_off = slab_bytes * (DOUBLE ? 2u : 1u);
+  const uint32_t table_off = tiles_off + kSlabWaves * wave_lds_bytes(V);
+  const uint32_t table_bytes = (p.rows_per_block + 1u) * 16u;
+  if (tid < 8) {
+    *reinterpret_cast<uintx4 *>(lds + zero_row * kSlabRowBytes + tid * 16) = uintx4{0u, 0u, 0u, 0u};
+    if (DOUBLE) *reinterpret_cast<uintx4 *>(lds + slab_bytes + zero_row * kSlabRowBytes + tid * 16) = uintx4{0u, 0u, 0u, 0u};
+  }
+
+  SlabCtx<V, OutT> x;
+  x.lane = lane;
+  x.val_tile = lds + tiles_off + wave * wave_lds_bytes(V);
+  constexpr uint32_t kLaneBytes = V * 2u * 32u / 64u;
+  x.val_dst = x.val_tile + lane * kLaneBytes;
+  // value tile rows are V*2 bytes; transpose read h picks rows 8g + 4h + m/4
+  x.a_off = (uint32_t)(8 * g + (m >> 2)) * (V * 2u) + (uint32_t)(m & 3) * 8u;
+  x.slot0 = (uint32_t)(8 * g + (m >> 2));
+  x.b_lane_off = (uint32_t)(m & 3) * 8u;
+  x.zero_row = zero_row;
+  x.N = p.N;
+  x.c_vrow_bytes = (uint32_t)V * (uint32_t)p.N * (uint32_t)sizeof(OutT);
+  const uint32_t nvec = (uint32_t)row_offsets[p.m_vec];
+  x.srd_cols = make_srd(p.col_idx, nvec * 4u);
+
+  // ---- first item: fetch and commit its slab and table
+  SlabItem cur = slab_item(p, xcd, it);
+  {
+    const __amdgpu_buffer_rsrc_t srd_b = make_srd(p.B + (int64_t)cur.batch * p.stride_B, b_bytes);
+    const intx4 e = slab_table_fetch(p, row_offsets, row_indices, cur.rb, tid);
+    for (uint32_t u0 = 0; u0 < units; u0 += kSlabThreads * 4) {
+      uintx4 d[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        d[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(
+                                              srd_b, slab_unit_src(p, u0 + i * kSlabThreads + tid, units, cur.tile * 64u, b_bytes), 0, 0));
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t u = u0 + i * kSlabThreads + tid;
+        if (u < units) *reinterpret_cast<uintx4 *>(lds + slab_unit_dst(u)) = d[i];
       }
     }
+    if ((uint32_t)tid <= p.rows_per_block) *reinterpret_cast<intx4 *>(lds + table_off + tid * 16) = e;
+  }
+  __syncthreads();
+
+  uint32_t slab_sel = 0, table_sel = 0;
+  for (;;) {
+    const bool has_next = it + 1u < it_end;
+    const SlabItem nxt = has_next ? slab_item(p, xcd, it + 1u) : cur;
+    const bool new_slab = nxt.batch != cur.batch || nxt.tile != cur.tile;
+    SlabFetch f;
+    // (a copy of the thread index the compiler cannot see through: the address arithmetic of the
+    // fetch would otherwise be hoisted out of the item loop and held in registers across it)
+    int ftid = tid;
+    asm volatile("" : "+v"(ftid));
+    if (DOUBLE && has_next) {
+      // the next item's table and slab start their way to registers now and are written to LDS
+      // when this item's rows are done
+      f.entry = slab_table_fetch(p, row_offsets, row_indices, nxt.rb, ftid);
+      if (new_slab) {
+        const __amdgpu_buffer_rsrc_t srd_b = make_srd(p.B + (int64_t)nxt.batch * p.stride_B, b_bytes);
+#pragma unroll
+        for (int i = 0; i < kSlabFetchUnits; ++i)
+          f.d[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(
+                                                  srd_b, slab_unit_src(p, i * kSlabThreads + ftid, units, nxt.tile * 64u, b_bytes), 0, 0));
+      }
+    }
+
+    {
+      const int row_lo = (int)(cur.rb * p.rows_per_block);
+      SlabRows rows;
+      rows.table = reinterpret_cast<const intx4 *>(lds + table_off + table_sel * table_bytes);
+      rows.n_rows = min(p.m_vec, row_lo + (int)p.rows_per_block) - row_lo;
+      rows.wave = wave;
+      SlabStore<V, OutT> out;
+      out.init(lane, (int)cur.tile * 64, p.N);
+      // One buffer descriptor spans this batch element's C (the launcher checks it is below 4 GiB).
+      const __amdgpu_buffer_rsrc_t srd_c = make_srd(reinterpret_cast<OutT *>(p.C) + (int64_t)cur.batch * p.stride_C,
+                                                    (uint32_t)p.m_vec * x.c_vrow_bytes);
+      slab_process_item<V, OutT>(x, lds, slab_sel * slab_bytes, rows, p.values + (int64_t)cur.batch * p.stride_values,
+                                 srd_c, out);
+    }
+    if (!has_next) break;
+
+    int ctid = tid;
+    asm volatile("" : "+v"(ctid));
+    if (DOUBLE) {
+      // The other buffers were last read during the previous item, which every wave has left.
+      if (new_slab) {
+        slab_sel ^= 1u;
+#pragma unroll
+        for (int i = 0; i < kSlabFetchUnits; ++i) {
+          const uint32_t u = i * kSlabThreads + ctid;
+          if (u < units) *reinterpret_cast<uintx4 *>(lds + slab_sel * slab_bytes + slab_unit_dst(u)) = f.d[i];
+        }
+      }
+      table_sel ^= 1u;
+      if ((uint32_t)ctid <= p.rows_per_block) *reinterpret_cast<intx4 *>(lds + table_off + table_sel * table_bytes + ctid * 16) = f.entry;
+      __syncthreads();
+    } else {
+      __syncthreads();  // every wave is done with the slab and the table
+      const intx4 e = slab_table_fetch(p, row_offsets, row_indices, nxt.rb, ctid);
+      if (new_slab) {
+        const __amdgpu_buffer_rsrc_t srd_b = make_srd(p.B + (int64_t)nxt.batch * p.stride_B, b_bytes);
+        for (uint32_t u0 = 0; u0 < units; u0 += kSlabThreads * 4) {
+          uintx4 d[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            d[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(
+                                                  srd_b, slab_unit_src(p, u0 + i * kSlabThreads + ctid, units, nxt.tile * 64u, b_bytes), 0, 0));
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const uint32_t u = u0 + i * kSlabThreads + ctid;
+            if (u < units) *reinterpret_cast<uintx4 *>(lds + slab_unit_dst(u)) = d[i];
+          }
+        }
+      }
+      if ((uint32_t)ctid <= p.rows_per_block) *reinterpret_cast<intx4 *>(lds + table_off + ctid * 16) = e;
+      __syncthreads();
+    }
+    cur = nxt;
+    ++it;
   }
 }
 
@@ -664,40 +770,64 @@ int set_kernel_override(int which) {
   return old;
 }
 
-static constexpr uint32_t kSlabMaxRows = 255;  // vector-rows per workgroup (row table of 256 entries)
-static constexpr int kSlabMaxK = 1180;  // slab + zero row + 8 value tiles + row table must fit in 160 KB of LDS
+static constexpr uint32_t kSlabLds = 160u * 1024u;
+static constexpr uint32_t kSlabMaxRows = 512;  // vector-rows per work item (one row table entry per thread, tables of 8 KB)
+static constexpr uint32_t kSlabMinRows = 32;   // keeps the copy of the slab a small part of an item's traffic
+
+// LDS bytes of a workgroup: slabs (+ zero rows), value tiles, two row tables.
+static uint32_t slab_lds_bytes(int K, int V, uint32_t rows, bool dbl) {
+  return (uint32_t)(K + 1) * kSlabRowBytes * (dbl ? 2u : 1u) + kSlabWaves * wave_lds_bytes(V) + 2u * 16u * (rows + 1u);
+}
+// Largest K the slab kernel takes (one slab, smallest row tables).
+static bool slab_fits(int K, int V) { return slab_lds_bytes(K, V, kSlabMinRows, false) <= kSlabLds; }
+
+static uint32_t device_cus() {
+  static uint32_t cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 8)
+      n = 256;
+    cus = (uint32_t)n;
+  }
+  return cus;
+}
+
+template <int V, typename OutT, bool DOUBLE>
+static hipError_t launch_slab_kernel(const SpmmArgs &p, uint32_t grid, uint32_t lds, hipStream_t stream) {
+  auto kern = spmm_slab_kernel<V, OutT, DOUBLE>;
+  static bool raised = false;  // per instantiation
+  if (!raised) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSlabLds);
+    if (e != hipSuccess) return e;
+    raised = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kSlabThreads), lds, stream, p, p.row_offsets, p.row_indices);
+  return hipGetLastError();
+}
 
 template <int V, typename OutT>
 static hipError_t launch_slab(const SpmmArgs &a, hipStream_t stream) {
   SpmmArgs p = a;
   p.n_tiles = (uint32_t)((a.N + 63) / 64);
   p.n_slabs = p.n_tiles * (uint32_t)a.batch;
-  // Aim at ~4 workgroups per CU, but keep at least 32 vector-rows per workgroup so that the copy
-  // of the slab into LDS stays a small part of the workgroup's traffic, and at most kSlabMaxRows
-  // (the row table in LDS).
-  const uint32_t rb_target = p.n_slabs >= 1024u ? 1u : 1024u / p.n_slabs;
-  uint32_t rows = ((uint32_t)a.m_vec + rb_target - 1u) / rb_target;
-  if (rows < 32u) rows = 32u;
-  if (rows > kSlabMaxRows) {
-    const uint32_t blocks = ((uint32_t)a.m_vec + kSlabMaxRows - 1u) / kSlabMaxRows;
-    rows = ((uint32_t)a.m_vec + blocks - 1u) / blocks;
-  }
+  p.group_by_batch = a.batch >= 8 ? 1u : 0u;
+  const uint32_t wgs_per_xcd = device_cus() / 8u;
+  // Aim at two or more items per workgroup (so that fetching a slab overlaps computing on the
+  // previous one), within kSlabMinRows .. kSlabMaxRows vector-rows per item.
+  const uint32_t slabs_per_xcd = p.group_by_batch ? (((uint32_t)a.batch + 7u) / 8u) * p.n_tiles : (p.n_slabs + 7u) / 8u;
+  uint32_t row_blocks = (2u * wgs_per_xcd + slabs_per_xcd - 1u) / slabs_per_xcd;
+  const uint32_t max_blocks = ((uint32_t)a.m_vec + kSlabMinRows - 1u) / kSlabMinRows;
+  const uint32_t min_blocks = ((uint32_t)a.m_vec + kSlabMaxRows - 1u) / kSlabMaxRows;
+  if (row_blocks > max_blocks) row_blocks = max_blocks;
+  if (row_blocks < min_blocks) row_blocks = min_blocks;
+  uint32_t rows = ((uint32_t)a.m_vec + row_blocks - 1u) / row_blocks;
+  bool dbl = (uint32_t)a.K * 8u <= (uint32_t)kSlabFetchUnits * kSlabThreads && slab_lds_bytes(a.K, V, rows, true) <= kSlabLds;
+  while (!dbl && slab_lds_bytes(a.K, V, rows, false) > kSlabLds && rows > kSlabMinRows) rows = (rows + 1u) / 2u;  // smaller tables for a tall slab
   p.rows_per_block = rows;
   p.row_blocks = ((uint32_t)a.m_vec + rows - 1u) / rows;
-  const size_t lds = (size_t)(a.K + 1) * kSlabRowBytes + kSlabWaves * wave_lds_bytes(V) + 16 * (rows + 1);
-  auto kern = spmm_slab_kernel<V, OutT>;
-  static size_t lds_allowed = 64 * 1024;  // per instantiation
-  if (lds > lds_allowed) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (e != hipSuccess) return e;
-    lds_allowed = 160 * 1024;
-  }
-  p.group_by_batch = a.batch >= 8 ? 1u : 0u;
-  const uint32_t grid = p.group_by_batch ? (((uint32_t)a.batch + 7u) / 8u) * 8u * p.n_tiles * p.row_blocks
-                                         : ((p.n_slabs + 7u) / 8u) * 8u * p.row_blocks;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(kSlabThreads), lds, stream, p, a.row_offsets, a.row_indices);
-  return hipGetLastError();
+  const uint32_t lds = slab_lds_bytes(a.K, V, rows, dbl);
+  const uint32_t grid = 8u * wgs_per_xcd;
+  return dbl ? launch_slab_kernel<V, OutT, true>(p, grid, lds, stream) : launch_slab_kernel<V, OutT, false>(p, grid, lds, stream);
 }
 
 template <int V, typename OutT>
@@ -734,7 +864,7 @@ hipError_t launch_spmm(const SpmmArgs &a, int V, bool out_f16, hipStream_t strea
     const uint64_t slabs = (uint64_t)((a.N + 63) / 64) * (uint64_t)a.batch;
     const uint64_t blocks = slabs * (uint64_t)((a.m_vec + 31) / 32);
     // The slab kernel addresses one batch element's C through a 32-bit buffer descriptor.
-    const bool slab_ok = a.K <= kSlabMaxK && (uint64_t)a.m_vec * (V == 8 ? 8u : 16u) * (uint64_t)a.N * out_size < 0xffffffffull;
+    const bool slab_ok = slab_fits(a.K, V) && (uint64_t)a.m_vec * (V == 8 ? 8u : 16u) * (uint64_t)a.N * out_size < 0xffffffffull;
     which = (slab_ok && a.m_vec >= 64 && blocks >= 1024) ? 3 : 2;
     if (g_kernel_override == 2) which = 2;
     if (g_kernel_override == 3 && slab_ok) which = 3;

@@ -245,6 +245,15 @@ static constexpr int slab_ring(int V) { return V == 8 ? 6 : 5; }
 typedef short shortx4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) shortx4 lds_shortx4;
 
+// The same read at an absolute LDS byte address (saves adding the base of the dynamic LDS array,
+// which the compiler does not fold, to every address).
+__device__ __forceinline__ uintx2 lds_read_tr_abs(uint32_t lds_addr) {
+  const shortx4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4 *)(uintptr_t)lds_addr);
+  return __builtin_bit_cast(uintx2, v);
+}
+__device__ __forceinline__ uint32_t lds_address(const unsigned char *p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const unsigned char *)p;
+}
 __device__ __forceinline__ uintx2 lds_read_tr(const unsigned char *lds_base, uint32_t byte_off) {
   const shortx4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4 *)(lds_base + byte_off));
   return __builtin_bit_cast(uintx2, v);
@@ -272,7 +281,7 @@ struct SlabLoads {    // what the head records for a step; the step consumes it 
   uint32_t col[2];    // column index of k slots 8g + m/4 and 8g + 4 + m/4
   typename SlabVals<V>::type vraw;
   int row, left;      // (wave-uniform) vector-row and its vectors from this step on
-  bool valid;         // (wave-uniform) false once the wave has run out of steps
+  int valid;          // (wave-uniform) 0 once the wave has run out of steps
 };
 
 // Walks one wave's sequence of steps.  The (vector-row, first vector, end vector) triples of the
@@ -287,9 +296,9 @@ struct SlabLoads {    // what the head records for a step; the step consumes it 
 typedef int intx4 __attribute__((ext_vector_type(4)));
 struct SlabCursor {
   int row, kc, end;  // current step: vectors [kc, min(kc + 32, end)) of vector-row `row`
-  bool valid;
+  int valid;  // flags are ints: wave-uniform 0 / 1 that stay in scalar registers
   intx4 next;        // table entry of the following vector-row (still in vector registers)
-  bool next_valid;
+  int next_valid;
   int count;         // rows requested so far
 };
 
@@ -301,7 +310,7 @@ struct SlabRows {      // what the cursors need to find rows
 __device__ __forceinline__ void cursor_prefetch(SlabCursor &c, const SlabRows &rows) {
   const int idx = rows.wave + kSlabWaves * c.count;
   ++c.count;
-  c.next_valid = idx < rows.n_rows;
+  c.next_valid = idx < rows.n_rows ? 1 : 0;
   c.next = rows.table[min(idx, rows.n_rows)];
 }
 
@@ -319,7 +328,7 @@ __device__ __forceinline__ void cursor_advance(SlabCursor &c, const SlabRows &ro
 }
 
 template <int V>
-__device__ __forceinline__ void slab_issue(SlabLoads<V> &r, int row, int kc, int end, bool valid, int lane, uint32_t slot0,
+__device__ __forceinline__ void slab_issue(SlabLoads<V> &r, int row, int kc, int end, int valid, int lane, uint32_t slot0,
                                            __amdgpu_buffer_rsrc_t srd_cols, const uint16_t *vals) {
   r.row = row;
   r.left = end - kc;
@@ -484,10 +493,16 @@ __device__ __forceinline__ void slab_process_item(const SlabCtx<V, OutT> &x, uns
   // the value tile of the first step
   *reinterpret_cast<typename SlabVals<V>::type *>(x.val_dst) = ld[0].vraw;
 
-  const uint32_t lane_base = x.b_lane_off + slab_base;  // slab_base is a multiple of 128
+  const uint32_t lane_base = x.b_lane_off + slab_base + lds_address(lds);  // slab_base is a multiple of 128, and so is the LDS base
+  // Accumulators are cleared by an MFMA of two zero operands: four instructions on the otherwise
+  // idle matrix pipe instead of sixteen register moves on the vector ALU, which the loop saturates.
+  Half8Bits zero_op;
+  zero_op.u[0] = zero_op.u[1] = zero_op.u[2] = zero_op.u[3] = 0u;
+  asm volatile("" : "+v"(zero_op.u[0]), "+v"(zero_op.u[1]), "+v"(zero_op.u[2]), "+v"(zero_op.u[3]));  // keep it in registers
+  const floatx4 zero_c = {0.f, 0.f, 0.f, 0.f};
   floatx4 acc[4];
 #pragma unroll
-  for (int q = 0; q < 4; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int q = 0; q < 4; ++q) acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(zero_op.h, zero_op.h, zero_c, 0, 0, 0);
   for (;;) {
 #pragma unroll
     for (int u = 0; u < R; ++u) {
@@ -513,8 +528,8 @@ __device__ __forceinline__ void slab_process_item(const SlabCtx<V, OutT> &x, uns
       Half8Bits b[4];
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const uintx2 lo = lds_read_tr(lds, addr[0] ^ ((uint32_t)q << 5));
-        const uintx2 hi = lds_read_tr(lds, addr[1] ^ ((uint32_t)q << 5));
+        const uintx2 lo = lds_read_tr_abs(addr[0] ^ ((uint32_t)q << 5));
+        const uintx2 hi = lds_read_tr_abs(addr[1] ^ ((uint32_t)q << 5));
         b[q].u[0] = lo[0]; b[q].u[1] = lo[1]; b[q].u[2] = hi[0]; b[q].u[3] = hi[1];
       }
       // the next step's value tile goes to LDS behind the reads above (LDS operations of a wave
@@ -526,7 +541,7 @@ __device__ __forceinline__ void slab_process_item(const SlabCtx<V, OutT> &x, uns
       if (left <= 32) {  // last step of the vector-row: write its V x 64 tile of C and start over from zero
         out.store(acc, srd_c, (uint32_t)ld[cur].row * x.c_vrow_bytes, x.N);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
+        for (int q = 0; q < 4; ++q) acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(zero_op.h, zero_op.h, zero_c, 0, 0, 0);
       }
       if (!ld[nxt].valid) return;
     }
@@ -592,7 +607,7 @@ template <int V, typename OutT, bool DOUBLE>
 __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs p,
                                                                  const int32_t *__restrict__ row_offsets,
                                                                  const int32_t *__restrict__ row_indices) {
-  extern __shared__ __align__(16) unsigned char lds[];
+  extern __shared__ __align__(128) unsigned char lds[];
   // The hardware deals consecutive workgroup ids round-robin to the 8 XCDs, each with its own L2.
   const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3, wgs_per_xcd = gridDim.x >> 3;
   const uint32_t slabs_x = p.group_by_batch ? (((uint32_t)p.batch + 7u - xcd) / 8u) * p.n_tiles : (p.n_slabs + 7u - xcd) / 8u;

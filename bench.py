@@ -131,9 +131,11 @@ def main():
         del src, dst
 
     M, K, V, sparsity, N = 2048, 512, 8, 0.9, 256
+    kernel_names = {1: "spmm_generic_kernel<8,float>", 2: "spmm_gather_kernel<8,float>", 3: "spmm_slab_kernel<8,float,true>"}
     main_res, (vs, vals, B, C) = spmm_case(L, torch, synth, M, K, V, sparsity, N, args.batch, True, 0.02, 2,
                                            args.steps, args.warmup, dense=not args.quick)
     torch.cuda.synchronize()
+    main_kernel = kernel_names.get(L.sspmm_last_kernel(), "unknown")
 
     # parity of batch element 0 against the CPU oracle, and the CPU baseline on the same element
     cpu = None
@@ -237,7 +239,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": main_res["hbm_gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": main_res["hbm_frac"],
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.batch) if args.kernel == "auto" else None,
-                     "kernel": "spmm_gather_kernel<8,float>", "alg_bytes_per_launch": main_res["alg_bytes"]},
+                     "kernel": main_kernel, "alg_bytes_per_launch": main_res["alg_bytes"]},
         "cpu_baseline": cpu,
         "parity_max_rel_err": parity,
         "dense_gemm": {k: main_res[k] for k in main_res if k.startswith("dense") or k.startswith("speedup")},

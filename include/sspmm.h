@@ -37,6 +37,10 @@ int sspmm_version(void);
  */
 int sspmm_select_kernel(int which);
 
+/* Companion of sspmm_select_kernel (no counterpart in the reference either): the kernel the latest
+ * SpMM call of this process ran, numbered as above; 0 before any call.  Not thread-safe. */
+int sspmm_last_kernel(void);
+
 /* Static text for a return code of this library. */
 const char *sspmm_error_string(int code);
 

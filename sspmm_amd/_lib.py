@@ -17,6 +17,7 @@ SIGNATURES = {
     "sspmm_version": (_int, []),
     "sspmm_error_string": (ctypes.c_char_p, [_int]),
     "sspmm_select_kernel": (_int, [_int]),
+    "sspmm_last_kernel": (_int, []),
     "sspmm_f16_f32": (_int, [_int] * 4 + [_vp] * 7),
     "sspmm_f16_f16": (_int, [_int] * 4 + [_vp] * 7),
     "sspmm_batched_f16_f16": (_int, [_int] * 5 + [_vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),

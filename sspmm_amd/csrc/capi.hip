@@ -52,6 +52,8 @@ int sspmm_select_kernel(int which) {
   return sspmm::set_kernel_override(which);
 }
 
+int sspmm_last_kernel(void) { return sspmm::last_kernel(); }
+
 const char *sspmm_error_string(int code) {
   if (code == 0) return "success";
   if (code == kInvalid) return "invalid argument (unsupported V, negative size, null pointer or index range)";

@@ -779,6 +779,9 @@ __global__ __launch_bounds__(64) void spmm_generic_kernel(const SpmmArgs p) {
 
 static int g_kernel_override = 0;  // 0 auto, 1 generic, 2 gather, 3 slab (tests and tuning)
 
+static int g_last_kernel = 0;  // kernel of the latest launch
+int last_kernel() { return g_last_kernel; }
+
 int set_kernel_override(int which) {
   const int old = g_kernel_override;
   g_kernel_override = which;
@@ -885,6 +888,7 @@ hipError_t launch_spmm(const SpmmArgs &a, int V, bool out_f16, hipStream_t strea
     if (g_kernel_override == 3 && slab_ok) which = 3;
   }
   if (g_kernel_override == 1) which = 1;
+  g_last_kernel = which;
   if (V == 8) return out_f16 ? launch_v<8, _Float16>(a, which, stream) : launch_v<8, float>(a, which, stream);
   return out_f16 ? launch_v<16, _Float16>(a, which, stream) : launch_v<16, float>(a, which, stream);
 }

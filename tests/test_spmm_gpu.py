@@ -52,6 +52,9 @@ def test_cfg1_512x512_v8(oracle, kernel, out_dtype):
 def test_cfg2_ffn_v8(oracle, kernel, shape, sparsity):
     vs = synth.vector_sparse(shape[0], shape[1], 8, sparsity, seed=2, std=0.02)
     check(oracle, vs, synth.dense_rhs(shape[1], 256, seed=12))
+    from sspmm_amd import _lib
+    if kernel != "auto" and shape[1] == 512:  # the forced kernel is the one that ran (K = 2048 is too tall for the slab)
+        assert _lib.lib().sspmm_last_kernel() == KERNELS[kernel]
 
 
 @pytest.mark.parametrize("shape,sparsity,N", [((1024, 2304), 0.8, 256), ((2048, 1024), 0.95, 256),
@@ -204,6 +207,36 @@ def test_bspmm_matches_looped_spmm(oracle, kernel, V, out_dtype):
         assert np.array_equal(out[b], single)
         want = oracle.spmm(vs.m_vec, V, N, K, vs.row_offsets, vs.col_idx, vals[b], B[b])
         assert max_rel_err(out[b], want) <= (TIGHT_F32 if out_dtype == torch.float32 else TIGHT_F16)
+
+
+@pytest.mark.parametrize("V,batch,m_rows,K,N,sparsity", [
+    (8, 1, 3000, 96, 64, 0.7),      # one slab, many row blocks: work items that follow each other on the same slab
+    (8, 20, 400, 200, 192, 0.8),    # uneven batch elements per XCD, item lists that cross slabs (two slabs in LDS)
+    (16, 11, 150, 160, 136, 0.8),   # V = 16, a partial last column tile, batch not a multiple of 8
+    (8, 40, 128, 700, 128, 0.9),    # K too tall for two slabs: the single-buffer path with several items per workgroup
+    (16, 5, 70, 1000, 64, 0.9),     # fewer than 8 batch elements: slabs dealt round-robin to the XCDs
+])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
+def test_slab_kernel_work_item_lists(oracle, built_library, V, batch, m_rows, K, N, sparsity, out_dtype):
+    """Shapes chosen to walk the persistent slab kernel through every kind of item transition."""
+    from sspmm_amd import _lib
+    vs = synth.vector_sparse(m_rows * V, K, V, sparsity, seed=60 + batch)
+    rng = np.random.default_rng(61)
+    vals = rng.standard_normal((batch, vs.values.size)).astype(np.float16)
+    B = rng.standard_normal((batch, K, N)).astype(np.float16)
+    print("slab items V=%d batch=%d m_vec=%d K=%d N=%d %s" % (V, batch, vs.m_vec, K, N, out_dtype), flush=True)
+    _lib.lib().sspmm_select_kernel(3)
+    try:
+        out = sspmm_amd.bspmm(None, dev(vs.row_offsets), dev(vs.col_idx), dev(vals), dev(B), V, out_dtype=out_dtype)
+        torch.cuda.synchronize()
+        assert _lib.lib().sspmm_last_kernel() == 3
+    finally:
+        _lib.lib().sspmm_select_kernel(0)
+    out = out.cpu().numpy()
+    tol = TIGHT_F32 if out_dtype == torch.float32 else TIGHT_F16
+    for b in range(batch):
+        want = oracle.spmm(vs.m_vec, V, N, K, vs.row_offsets, vs.col_idx, vals[b], B[b], threads=8)
+        assert max_rel_err(out[b], want) <= tol, b
 
 
 def test_row_swizzle_matches_oracle(oracle, built_library):

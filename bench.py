@@ -229,6 +229,30 @@ def main():
             "alg_bytes": svc_bytes, "hbm_gbps": svc_bytes / svc_k_ms / 1e6,
         }
 
+        # ... and the SpMM that consumes it: the skewed pattern straight from the SVC, B 16384 x 256
+        N4 = 256
+        B4 = torch.from_numpy(synth.dense_rhs(csr.K, N4, seed=14)).cuda()
+        C4 = torch.empty(csr.M, N4, dtype=torch.float32, device="cuda")
+        m_vec4 = csr.M // 8
+
+        def spmm_cfg4():
+            rc = L.sspmm_f16_f32(m_vec4, 8, N4, csr.K, None, r.vec_row_ptr.data_ptr(), r.vec_col.data_ptr(),
+                                 r.vec_val.data_ptr(), B4.data_ptr(), C4.data_ptr(), stream)
+            assert rc == 0, rc
+
+        ms4 = time_launches(spmm_cfg4, st, wu)
+        lens = np.diff(r.vec_row_ptr.cpu().numpy())
+        touched = int(np.unique(r.vec_col.cpu().numpy()).size)
+        bytes4 = synth.spmm_algorithmic_bytes(m_vec4, 8, int(r.num_vec), csr.K, N4, 4, k_touched=touched)
+        extra["cfg4_spmm_on_svc_output"] = {
+            "workload": "A 16384x16384 Zipf rows (nnz %d) after SVC V=8, B 16384x%d, C fp32" % (nnz, N4),
+            "ms": ms4, "useful_tflops": 2.0 * nnz * N4 / ms4 / 1e9, "alg_bytes": bytes4,
+            "hbm_gbps": bytes4 / ms4 / 1e6, "hbm_frac": bytes4 / ms4 / 1e6 / HBM_PEAK_GBPS,
+            "kernel": kernel_names.get(L.sspmm_last_kernel(), "unknown"),
+            "vector_row_len_max": int(lens.max()), "vector_row_len_mean": float(lens.mean()),
+            "steps_of_longest_row": int((lens.max() + 31) // 32), "steps_total": int(((lens + 31) // 32).sum()),
+        }
+
     line = {
         "metric": "SpMM useful TFLOP/s (2*nnz*N/t), V=8 @90% sparsity, fp16 in / fp32 accumulate",
         "value": main_res["useful_tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,

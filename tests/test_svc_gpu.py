@@ -121,6 +121,23 @@ def test_cfg4_zipf_16384(oracle, built_library):
     _compare_with_oracle(oracle, csr, 16, "sorted")
 
 
+def test_cfg4_svc_then_spmm_at_full_size(oracle, built_library):
+    """cfg4 end to end at its real shape: Zipf CSR 16384^2 -> SVC (GPU) -> SpMM (GPU) against the
+    oracle's SpMM on the oracle's SVC output (a pattern with vector-rows from 0 to several thousand vectors)."""
+    csr = synth.zipf_csr(16384, 16384, seed=4)
+    N = 256
+    B = synth.dense_rhs(csr.K, N, seed=14)
+    r = sspmm_amd.svc(dev(csr.row_ptr), dev(csr.col_ind), dev(csr.values), csr.M, csr.K, 8)
+    for out_dtype, tol in ((torch.float32, 2e-5), (torch.float16, 2e-3)):
+        out = sspmm_amd.spmm(None, r.vec_row_ptr, r.vec_col, r.vec_val, dev(B), 8, out_dtype=out_dtype)
+        torch.cuda.synchronize()
+        vrp, vcol, vval = oracle.svc(csr.M, csr.K, 8, csr.row_ptr, csr.col_ind, csr.values)
+        want = oracle.spmm(csr.M // 8, 8, N, csr.K, vrp, vcol, vval, B, threads=8)
+        got = out.float().cpu().numpy()
+        scale = np.abs(want).max()
+        assert np.abs(got - want).max() / scale <= tol
+
+
 def test_svc_then_spmm_equals_csr_matmul(oracle, built_library):
     """End of the pipe: unstructured CSR -> SVC (GPU) -> SpMM (GPU) == dense(A) @ B."""
     rng = np.random.default_rng(8)

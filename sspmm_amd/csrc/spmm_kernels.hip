@@ -80,38 +80,52 @@ struct Store8<_Float16> {
   }
 };
 
-// One chunk = 32 consecutive non-zero vectors of a vector-row.
+// One chunk = 32 consecutive non-zero vectors of a vector-row.  Its loads form a chain of two
+// memory round trips (column indices, then the rows of B they name), so they are issued in two
+// stages, one step apart: while chunk s is contracted, the gathers of chunk s + 1 and the column
+// indices of chunk s + 2 are in flight.
+struct ChunkHead {   // stage 1: what does not depend on other loads
+  uintx4 c0, c1;     // column indices of k slots 8g .. 8g+7
+  uint16_t a16[8];   // a16[j] = values[(k slot 8g+j), v = m]
+  int kc;            // first vector of the chunk
+};
 struct Chunk {
   uintx4 raw[8];     // raw[j] = 8 halfs (columns n0+8m..+7) of the row of B named by k slot 8g+j
-  uint16_t a16[8];   // a16[j] = values[(k slot 8g+j), v = m]
+  uint16_t a16[8];
 };
 
 template <int V>
-__device__ __forceinline__ void load_chunk(Chunk &c, int kc, int end, int g, __amdgpu_buffer_rsrc_t srd_cols,
-                                           __amdgpu_buffer_rsrc_t srd_vals, __amdgpu_buffer_rsrc_t srd_b,
-                                           uint32_t lane_n2, uint32_t lane_col_off, uint32_t b_bytes,
-                                           uint32_t vals_lane_off) {
+__device__ __forceinline__ void load_head(ChunkHead &h, int kc, int g, __amdgpu_buffer_rsrc_t srd_cols,
+                                          __amdgpu_buffer_rsrc_t srd_vals, uint32_t vals_lane_off) {
   const int kb = kc + 8 * g;
+  h.kc = kc;
   // srd_cols / srd_vals end at this vector-row's last vector: slots past it read as zero.
-  const uintx4 c0 = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_cols, kb * 4, 0, 0));
-  const uintx4 c1 = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_cols, kb * 4 + 16, 0, 0));
+  h.c0 = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_cols, kb * 4, 0, 0));
+  h.c1 = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_cols, kb * 4 + 16, 0, 0));
   const uint32_t voff = (uint32_t)kb * (V * 2) + vals_lane_off;
 #pragma unroll
   for (int j = 0; j < 8; ++j)
-    c.a16[j] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(srd_vals, voff + j * V * 2, 0, 0);
+    h.a16[j] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(srd_vals, voff + j * V * 2, 0, 0);
+}
+
+__device__ __forceinline__ void load_body(Chunk &c, const ChunkHead &h, int end, int g, __amdgpu_buffer_rsrc_t srd_b,
+                                          uint32_t lane_n2, uint32_t lane_col_off, uint32_t b_bytes) {
+  const int kb = h.kc + 8 * g;
   uint32_t off[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
-    const uint32_t col = j < 4 ? c0[j] : c1[j - 4];
+    const uint32_t col = j < 4 ? h.c0[j] : h.c1[j - 4];
     off[j] = __umul24(col, lane_n2) + lane_col_off;
   }
-  if (kc + 32 > end) {  // wave-uniform: only the last chunk of a vector-row can be partial
+  if (h.kc + 32 > end) {  // wave-uniform: only the last chunk of a vector-row can be partial
 #pragma unroll
     for (int j = 0; j < 8; ++j) off[j] = (kb + j < end) ? off[j] : b_bytes;
   }
 #pragma unroll
-  for (int j = 0; j < 8; ++j)
+  for (int j = 0; j < 8; ++j) {
     c.raw[j] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_b, off[j], 0, 0));
+    c.a16[j] = h.a16[j];
+  }
 }
 
 __device__ __forceinline__ void mac_chunk(const Chunk &c, floatx4 (&acc)[8]) {
@@ -164,24 +178,29 @@ __global__ __launch_bounds__(64) void spmm_gather_kernel(const SpmmArgs p) {
   for (int q = 0; q < 8; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   if (beg < end) {
-    // Two chunk buffers used alternately: the gathers of the next 32 vectors are in flight while
-    // the current 32 are contracted.
+    // Heads run two chunks ahead of the arithmetic, bodies one (two buffers of each, used alternately).
+    // A head past the end of the row reads zeros and is never turned into a body.
+    ChunkHead h0, h1;
     Chunk c0, c1;
-    load_chunk<V>(c0, beg, end, g, srd_cols, srd_vals, srd_b, lane_n2, lane_col_off, b_bytes, vals_lane_off);
-    int kc = beg + 32;
+    load_head<V>(h0, beg, g, srd_cols, srd_vals, vals_lane_off);
+    load_head<V>(h1, beg + 32, g, srd_cols, srd_vals, vals_lane_off);
+    load_body(c0, h0, end, g, srd_b, lane_n2, lane_col_off, b_bytes);
+    int kc = beg + 32;  // first vector of the chunk whose body is loaded next
     for (;;) {
       if (kc >= end) {
         mac_chunk(c0, acc);
         break;
       }
-      load_chunk<V>(c1, kc, end, g, srd_cols, srd_vals, srd_b, lane_n2, lane_col_off, b_bytes, vals_lane_off);
+      load_head<V>(h0, kc + 32, g, srd_cols, srd_vals, vals_lane_off);
+      load_body(c1, h1, end, g, srd_b, lane_n2, lane_col_off, b_bytes);
       mac_chunk(c0, acc);
       kc += 32;
       if (kc >= end) {
         mac_chunk(c1, acc);
         break;
       }
-      load_chunk<V>(c0, kc, end, g, srd_cols, srd_vals, srd_b, lane_n2, lane_col_off, b_bytes, vals_lane_off);
+      load_head<V>(h1, kc + 32, g, srd_cols, srd_vals, vals_lane_off);
+      load_body(c0, h0, end, g, srd_b, lane_n2, lane_col_off, b_bytes);
       mac_chunk(c1, acc);
       kc += 32;
     }

@@ -253,6 +253,38 @@ def main():
             "steps_of_longest_row": int((lens.max() + 31) // 32), "steps_total": int(((lens + 31) // 32).sum()),
         }
 
+        # cfg5: one BERT-base shaped encoder layer (hidden 768, 12 heads, FFN 3072, 8 x 512 tokens) with
+        # six vector-sparse weights (V=16, 90 %) and dense attention in torch; the same layer with dense fp16
+        # matmuls on the densified weights beside it
+        from sspmm_amd.layers import SparseEncoderLayer, SparseLinear
+        hid, heads, ffn, V5, bsz, seq = 768, 12, 3072, 16, 8, 512
+
+        def mk(o, i, seed):
+            w = synth.vector_sparse(o, i, V5, 0.9, seed=seed, std=0.02)
+            return SparseLinear.from_cvse(i, V5, torch.from_numpy(w.row_offsets).cuda(), torch.from_numpy(w.col_idx).cuda(),
+                                          torch.from_numpy(w.values).cuda())
+
+        layer = SparseEncoderLayer(hid, heads, ffn, mk(hid, hid, 51), mk(hid, hid, 52), mk(hid, hid, 53), mk(hid, hid, 54),
+                                   mk(ffn, hid, 55), mk(hid, ffn, 56)).cuda().half()
+        x5 = (torch.randn(hid, bsz * seq, device="cuda") * 1.0).half()
+        dense_w = {n: getattr(layer, n).dense_weight() for n in ("q", "k", "v", "o", "ffn1", "ffn2")}
+        with torch.no_grad():
+            y_sp = layer(x5, bsz, seq)
+            y_de = layer(x5, bsz, seq, linear=lambda n, lin, t: dense_w[n] @ t)
+            sp_ms = time_launches(lambda: layer(x5, bsz, seq), st, wu)
+            de_ms = time_launches(lambda: layer(x5, bsz, seq, linear=lambda n, lin, t: dense_w[n] @ t), st, wu)
+            per = {}
+            for n in ("q", "o", "ffn1", "ffn2"):
+                lin = getattr(layer, n)
+                xin = torch.randn(lin.in_features, bsz * seq, device="cuda").half()
+                per[n] = {"sparse_ms": time_launches(lambda: lin(xin), st, wu),
+                          "dense_ms": time_launches(lambda: dense_w[n] @ xin, st, wu)}
+        extra["cfg5_encoder_layer_v16_s0.9_tokens4096"] = {
+            "sparse_layer_ms": sp_ms, "dense_layer_ms": de_ms, "speedup_vs_dense_layer": de_ms / sp_ms,
+            "max_rel_diff_vs_dense_layer": float((y_sp.float() - y_de.float()).abs().max() / y_de.float().abs().max()),
+            "projections": per,
+        }
+
     line = {
         "metric": "SpMM useful TFLOP/s (2*nnz*N/t), V=8 @90% sparsity, fp16 in / fp32 accumulate",
         "value": main_res["useful_tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,

@@ -40,7 +40,7 @@ def check(oracle, vs, B, out_dtype=torch.float32, row_indices=None):
     return got, want
 
 
-# BASELINE configs at their real shapes (the oracle runs each in well under a second with 8 threads)
+# the benchmark configurations at their real shapes (the oracle runs each in well under a second with 8 threads)
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
 def test_cfg1_512x512_v8(oracle, kernel, out_dtype):
     vs = synth.vector_sparse(512, 512, 8, 0.9, seed=1)

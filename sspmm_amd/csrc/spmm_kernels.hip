@@ -818,25 +818,33 @@ static uint32_t slab_lds_bytes(int K, int V, uint32_t rows, bool dbl) {
 // Largest K the slab kernel takes (one slab, smallest row tables).
 static bool slab_fits(int K, int V) { return slab_lds_bytes(K, V, kSlabMinRows, false) <= kSlabLds; }
 
-static uint32_t device_cus() {
-  static uint32_t cus = 0;
-  if (cus == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 8)
-      n = 256;
-    cus = (uint32_t)n;
+static constexpr int kMaxDevices = 64;
+static int current_device() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) dev = 0;
+  return dev;
+}
+
+static uint32_t device_cus() {  // of the current device
+  static uint32_t cus[kMaxDevices] = {};
+  const int dev = current_device();
+  if (cus[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 8) n = 256;
+    cus[dev] = (uint32_t)n;
   }
-  return cus;
+  return cus[dev];
 }
 
 template <int V, typename OutT, bool DOUBLE>
 static hipError_t launch_slab_kernel(const SpmmArgs &p, uint32_t grid, uint32_t lds, hipStream_t stream) {
   auto kern = spmm_slab_kernel<V, OutT, DOUBLE>;
-  static bool raised = false;  // per instantiation
-  if (!raised) {
+  static bool raised[kMaxDevices] = {};  // per instantiation and device
+  const int dev = current_device();
+  if (!raised[dev]) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSlabLds);
     if (e != hipSuccess) return e;
-    raised = true;
+    raised[dev] = true;
   }
   hipLaunchKernelGGL(kern, dim3(grid), dim3(kSlabThreads), lds, stream, p, p.row_offsets, p.row_indices);
   return hipGetLastError();

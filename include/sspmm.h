@@ -93,6 +93,40 @@ int sspmm_batched_f16_f32(int batch, int m_vec, int V, int N, int K, const int32
 int sspmm_sorted_row_swizzle(int m_vec, const int32_t *row_offsets, int32_t *row_indices, void *hip_stream);
 
 /* ------------------------------------------------------------------------------------------
+ * The two steps either side of the batched SpMM in the reference's sparse attention block
+ * (end2end/sspmm_e2e/spattention.py:167-179), on the same pattern arrays.
+ *
+ * Sampled dense-dense product: out_values[j*V + v] = sum_f lhs[(i*V + v)*F + f] * rhs[col_idx[j]*F + f]
+ * for every stored vector j of every vector-row i; fp16 inputs, fp32 accumulation, fp16 result.
+ * Replaces sddmm_cuda / batched_sddmm_cuda, reference end2end/sspmm_e2e/src/cuda/sddmm_kernel.cu:
+ * 1161-1226 and 1228-1295 (batch strides m*k, n*k, nnz*V at :1244-1246).
+ *   lhs [m_vec*V, F] and rhs [n_rhs, F] row-major, F a multiple of 8 up to 256, 16-byte aligned;
+ *   column indices in [0, n_rhs); n_rhs*F below 2^31.
+ * ---------------------------------------------------------------------------------------- */
+int sspmm_sddmm_f16(int m_vec, int V, int F, int n_rhs, const int32_t *row_indices, const int32_t *row_offsets,
+                    const int32_t *col_idx, const sspmm_half_t *lhs, const sspmm_half_t *rhs, sspmm_half_t *out_values,
+                    void *hip_stream);
+
+int sspmm_sddmm_batched_f16(int batch, int m_vec, int V, int F, int n_rhs, const int32_t *row_indices,
+                            const int32_t *row_offsets, const int32_t *col_idx, const sspmm_half_t *lhs,
+                            int64_t stride_lhs, const sspmm_half_t *rhs, int64_t stride_rhs, sspmm_half_t *out_values,
+                            int64_t stride_out, void *hip_stream);
+
+/*
+ * Row softmax over the stored entries: for dense row i*V + v, over the vectors j of vector-row i,
+ * out_values[j*V + v] = exp(values[j*V + v]*scaler - max) / sum, computed in fp32, fp16 result
+ * (positions that are not stored count as -infinity).  Replaces csr_softmax_cuda /
+ * batched_csr_softmax_cuda, reference end2end/sspmm_e2e/src/cuda/softmax_kernel.cu:202-290
+ * (kernel :95-165).  In place (out_values == values) is allowed; 16-byte aligned pointers.
+ */
+int sspmm_softmax_f16(int m_vec, int V, const int32_t *row_indices, const int32_t *row_offsets,
+                      const sspmm_half_t *values, float scaler, sspmm_half_t *out_values, void *hip_stream);
+
+int sspmm_softmax_batched_f16(int batch, int m_vec, int V, const int32_t *row_indices, const int32_t *row_offsets,
+                              const sspmm_half_t *values, float scaler, sspmm_half_t *out_values, int64_t stride,
+                              void *hip_stream);
+
+/* ------------------------------------------------------------------------------------------
  * Sparse Vector Compression (RowMerge): CSR -> CVSE.  Replaces the Python pass
  * CVSE.__init__, reference RowMerge/sparse_matrix_format.py:94-123 (merge at :110), and adds
  * the value packing its consumers define (SSpMM/sspmm_test.cpp:90).

@@ -40,6 +40,10 @@ def lib():
         L.oracle_spmm_f16.argtypes = [ctypes.c_int32] * 4 + [i32p, i32p, u16p, u16p, u16p, ctypes.c_int32]
         L.oracle_sorted_row_swizzle.restype = None
         L.oracle_sorted_row_swizzle.argtypes = [ctypes.c_int32, i32p, i32p]
+        L.oracle_sddmm_f16.restype = None
+        L.oracle_sddmm_f16.argtypes = [ctypes.c_int32] * 3 + [i32p, i32p, u16p, u16p, u16p]
+        L.oracle_softmax_f16.restype = None
+        L.oracle_softmax_f16.argtypes = [ctypes.c_int32] * 2 + [i32p, u16p, ctypes.c_float, u16p]
         L.oracle_h2f.restype = ctypes.c_float
         L.oracle_h2f.argtypes = [ctypes.c_uint16]
         L.oracle_f2h.restype = ctypes.c_uint16
@@ -106,6 +110,27 @@ def spmm(m_vec, V, N, K, row_offsets, col_idx, values, B, out_dtype=np.float32, 
     lib().oracle_spmm_f16(m_vec, V, N, K, _p(row_offsets, ctypes.c_int32), _p(col_idx, ctypes.c_int32),
                           _p(vals, ctypes.c_uint16), _p(Bb, ctypes.c_uint16), _p(C, ctypes.c_uint16), threads)
     return C.view(np.float16)
+
+
+def sddmm(m_vec, V, row_offsets, col_idx, lhs, rhs):
+    """Sampled dense-dense product at the vector pattern: lhs [m_vec*V, F], rhs [n, F] fp16 -> fp16 [nvec*V]."""
+    row_offsets, col_idx = _i32(row_offsets), _i32(col_idx)
+    F = lhs.shape[1]
+    a, b = _u16(lhs), _u16(rhs)
+    out = np.empty(max(col_idx.size * V, 1), dtype=np.uint16)
+    lib().oracle_sddmm_f16(m_vec, V, F, _p(row_offsets, ctypes.c_int32), _p(col_idx, ctypes.c_int32),
+                           _p(a, ctypes.c_uint16), _p(b, ctypes.c_uint16), _p(out, ctypes.c_uint16))
+    return out[:col_idx.size * V].copy().view(np.float16)
+
+
+def softmax(m_vec, V, row_offsets, values, scaler):
+    """Row softmax over the stored entries of a vector-sparse matrix: fp16 [nvec*V] -> fp16 [nvec*V]."""
+    row_offsets = _i32(row_offsets)
+    vals = _u16(values)
+    out = np.zeros(max(vals.size, 1), dtype=np.uint16)
+    lib().oracle_softmax_f16(m_vec, V, _p(row_offsets, ctypes.c_int32), _p(vals, ctypes.c_uint16),
+                             ctypes.c_float(scaler), _p(out, ctypes.c_uint16))
+    return out[:vals.size].copy().view(np.float16)
 
 
 def sorted_row_swizzle(row_offsets):

@@ -33,7 +33,22 @@
  *                           (argsort by descending vector-row length; the
  *                           reference's tie order is unspecified, ties here keep
  *                           ascending row index).  Pinned by invariants only.
+ *   oracle_sddmm_f16        the sampled product either side of the SpMM in the
+ *                           reference's sparse attention block:
+ *                           out[j*V+v] = lhs[i*V+v, :] . rhs[col_j, :] for the
+ *                           vectors j of vector-row i, fp32 accumulation over the
+ *                           feature index ascending, fp16 result
+ *                           (end2end/sspmm_e2e/src/cuda/sddmm_kernel.cu:1161-1226,
+ *                           check recipe end2end/sspmm_e2e/verify/sddmm.py:36-51).
+ *                           Pinned by: numpy fp64 matmul sampled at the pattern.
+ *   oracle_softmax_f16      csrSoftmaxKernel_, end2end/sspmm_e2e/src/cuda/
+ *                           softmax_kernel.cu:95-165: per dense row, over the
+ *                           row's stored entries, exp(x*scaler - max) / sum in
+ *                           fp32, fp16 result.  Pinned by: numpy softmax of the
+ *                           densified rows with -inf fill (the recipe of
+ *                           end2end/sspmm_e2e/verify/softmax.py:36-38).
  */
+#include <math.h>
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
@@ -333,4 +348,37 @@ void oracle_sorted_row_swizzle(int32_t rows, const int32_t *row_offsets, int32_t
   qsort(t, rows, sizeof(lenidx), cmp_lenidx_desc);
   for (int32_t i = 0; i < rows; ++i) row_indices[i] = t[i].idx;
   free(t);
+}
+
+/* ------------------------------------------------- sparse attention steps */
+
+/* lhs[M x F], rhs[n_rhs x F] fp16 row-major; out[nvec*V] fp16. */
+void oracle_sddmm_f16(int32_t m_vec, int32_t V, int32_t F, const int32_t *row_offsets, const int32_t *col_idx,
+                      const uint16_t *lhs, const uint16_t *rhs, uint16_t *out) {
+  for (int32_t i = 0; i < m_vec; ++i)
+    for (int32_t j = row_offsets[i]; j < row_offsets[i + 1]; ++j)
+      for (int32_t v = 0; v < V; ++v) {
+        const uint16_t *a = lhs + ((int64_t)i * V + v) * F, *b = rhs + (int64_t)col_idx[j] * F;
+        float acc = 0.f;
+        for (int32_t f = 0; f < F; ++f) acc += h2f(a[f]) * h2f(b[f]);
+        out[(int64_t)j * V + v] = f2h_rn(acc);
+      }
+}
+
+/* values[nvec*V] fp16 -> out[nvec*V] fp16; a vector-row without vectors writes nothing. */
+void oracle_softmax_f16(int32_t m_vec, int32_t V, const int32_t *row_offsets, const uint16_t *values, float scaler,
+                        uint16_t *out) {
+  for (int32_t i = 0; i < m_vec; ++i)
+    for (int32_t v = 0; v < V; ++v) {
+      const int32_t b = row_offsets[i], e = row_offsets[i + 1];
+      if (b == e) continue;
+      float mx = -INFINITY, sum = 0.f;
+      for (int32_t j = b; j < e; ++j) {
+        const float x = h2f(values[(int64_t)j * V + v]) * scaler;
+        mx = x > mx ? x : mx;
+      }
+      for (int32_t j = b; j < e; ++j) sum += expf(h2f(values[(int64_t)j * V + v]) * scaler - mx);
+      for (int32_t j = b; j < e; ++j)
+        out[(int64_t)j * V + v] = f2h_rn(expf(h2f(values[(int64_t)j * V + v]) * scaler - mx) / sum);
+    }
 }

@@ -23,6 +23,10 @@ SIGNATURES = {
     "sspmm_batched_f16_f16": (_int, [_int] * 5 + [_vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),
     "sspmm_batched_f16_f32": (_int, [_int] * 5 + [_vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),
     "sspmm_sorted_row_swizzle": (_int, [_int, _vp, _vp, _vp]),
+    "sspmm_sddmm_f16": (_int, [_int] * 4 + [_vp] * 7),
+    "sspmm_sddmm_batched_f16": (_int, [_int] * 5 + [_vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),
+    "sspmm_softmax_f16": (_int, [_int, _int, _vp, _vp, _vp, ctypes.c_float, _vp, _vp]),
+    "sspmm_softmax_batched_f16": (_int, [_int, _int, _int, _vp, _vp, _vp, ctypes.c_float, _vp, _i64, _vp]),
     "svc_workspace_bytes": (ctypes.c_size_t, [_int, _i64, _int]),
     "svc_count": (_int, [_int, _int, _int, _vp, _vp, _i64, _int, _vp, _vp, _vp]),
     "svc_fill": (_int, [_int, _int, _int, _vp, _vp, _vp, _i64, _int, _vp, _vp, _vp, _vp, _vp]),

@@ -1,0 +1,39 @@
+// Launch interface of the two steps that sit either side of the batched SpMM in a sparse
+// attention block: the sampled dense-dense product and the row softmax over stored entries.
+#ifndef SSPMM_AMD_ATTENTION_KERNELS_H
+#define SSPMM_AMD_ATTENTION_KERNELS_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace sspmm {
+
+struct SddmmArgs {
+  int m_vec, F, n_rhs, batch;
+  const int32_t *row_indices;  // nullable
+  const int32_t *row_offsets;
+  const int32_t *col_idx;
+  const uint16_t *lhs;  // [batch][m_vec*V][F]
+  const uint16_t *rhs;  // [batch][n_rhs][F]
+  uint16_t *out;        // [batch][nvec*V]
+  int64_t stride_lhs, stride_rhs, stride_out;  // per-batch strides in elements
+  uint32_t total_work, per_xcd;                // filled by the launcher
+};
+
+struct SoftmaxArgs {
+  int m_vec, batch;
+  const int32_t *row_indices;  // nullable
+  const int32_t *row_offsets;
+  const uint16_t *values;  // [batch][nvec*V]
+  uint16_t *out;           // [batch][nvec*V]
+  int64_t stride;          // per-batch stride in elements
+  float scaler;
+  uint32_t total_work, per_xcd;
+};
+
+// V must be 8 or 16; F a multiple of 8 up to 256; 16-byte aligned operands and strides.
+hipError_t launch_sddmm(const SddmmArgs &args, int V, hipStream_t stream);
+hipError_t launch_softmax(const SoftmaxArgs &args, int V, hipStream_t stream);
+
+}  // namespace sspmm
+#endif

@@ -1,0 +1,258 @@
+// The two steps either side of the batched SpMM in a sparse attention block, in the same
+// vector-sparse format, for gfx950 (wave64, MFMA 16x16x32 f16).
+//
+//   sddmm:   out[j*V + v] = lhs[i*V + v, :] . rhs[col_j, :]   for the vectors j of vector-row i
+//            (reference end2end/sspmm_e2e/src/cuda/sddmm_kernel.cu:1161-1295: `sddmm`, `bsddmm`);
+//   softmax: per dense row, over its stored entries, exp(x*scaler - max) / sum
+//            (reference end2end/sspmm_e2e/src/cuda/softmax_kernel.cu:95-290: `csr_softmax`, `bcsr_softmax`).
+//
+// Both are bound by memory traffic: the sddmm by the gathers of rows of rhs (F*2 bytes per stored
+// vector) and the writes of the values, the softmax by one read and one write of the values.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "attention_kernels.h"
+
+namespace sspmm {
+
+namespace {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef uint32_t uintx4 __attribute__((ext_vector_type(4)));
+typedef uint32_t uintx2 __attribute__((ext_vector_type(2)));
+
+static constexpr uint32_t kSrdWord3 = 0x00020000u;  // 32-bit raw (untyped) buffer, gfx9 family
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_srd(const void *base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, (int)kSrdWord3);
+}
+
+// Linear block ids are dealt round-robin to the 8 XCDs by the hardware; each XCD gets one
+// contiguous range of the work list so that neighbouring work shares an L2.
+__device__ __forceinline__ uint32_t xcd_work_index(uint32_t per_xcd) {
+  const uint32_t id = blockIdx.x;
+  return (id & 7u) * per_xcd + (id >> 3);
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------------------------ sddmm
+// One wave per (vector-row, batch element).  The V rows of lhs are the MFMA's first operand and
+// stay in registers (lane (m, g) holds features 32c + 8g .. + 7 of row m, c = 0 .. NC-1); per
+// group of 16 stored vectors, lane (m, g) loads the same features of the row of rhs named by
+// vector m, 16 contiguous bytes per load with no shuffling, NC MFMAs contract the features, and
+// the lane ends up with rows 4g .. 4g+3 of vector m: eight contiguous bytes of the output.
+// The column indices run two groups ahead of the arithmetic and the rows of rhs one group.
+template <int V, int NC>
+__global__ __launch_bounds__(64) void sddmm_kernel(const SddmmArgs p) {
+  const uint32_t w = xcd_work_index(p.per_xcd);
+  if (w >= p.total_work) return;
+  const uint32_t r = w % (uint32_t)p.m_vec;
+  const uint32_t batch = w / (uint32_t)p.m_vec;
+  const int row = p.row_indices ? p.row_indices[r] : (int)r;
+  const int beg = p.row_offsets[row], end = p.row_offsets[row + 1];
+  if (beg == end) return;
+
+  const int lane = threadIdx.x, m = lane & 15, g = lane >> 4;
+  const uint32_t F = (uint32_t)p.F;
+  const uint16_t *lhs = p.lhs + (int64_t)batch * p.stride_lhs + (int64_t)row * V * F;
+  const __amdgpu_buffer_rsrc_t srd_lhs = make_srd(lhs, (uint32_t)V * F * 2u);
+  const uint32_t rhs_bytes = (uint32_t)p.n_rhs * F * 2u;
+  const __amdgpu_buffer_rsrc_t srd_rhs = make_srd(p.rhs + (int64_t)batch * p.stride_rhs, rhs_bytes);
+  const __amdgpu_buffer_rsrc_t srd_cols = make_srd(p.col_idx, (uint32_t)end * 4u);  // past the row: reads 0
+  uint16_t *out = p.out + (int64_t)batch * p.stride_out;
+
+  // feature offsets of this lane's 16-byte pieces; pieces past F (or rows past V) read zeros
+  uint32_t foff[NC];
+  half8 a[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const uint32_t f0 = 32u * c + 8u * g;
+    foff[c] = f0 < F ? f0 * 2u : 0xffffffffu;
+    const uint32_t off = (m < V && f0 < F) ? ((uint32_t)m * F + f0) * 2u : 0xfffffff0u;
+    a[c] = __builtin_bit_cast(half8, __builtin_amdgcn_raw_buffer_load_b128(srd_lhs, off, 0, 0));
+  }
+
+  auto load_cols = [&](int kc) { return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(srd_cols, (kc + m) * 4, 0, 0); };
+  auto load_rows = [&](half8(&b)[NC], uint32_t col) {
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      const uint32_t off = foff[c] == 0xffffffffu ? 0xfffffff0u : __umul24(col, F * 2u) + foff[c];
+      b[c] = __builtin_bit_cast(half8, __builtin_amdgcn_raw_buffer_load_b128(srd_rhs, off, 0, 0));
+    }
+  };
+  auto finish = [&](const half8(&b)[NC], int kc) {
+    floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < NC; ++c) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[c], b[c], acc, 0, 0, 0);
+    if (kc + m < end && 4 * g < V) {
+      const half4 h = {(_Float16)acc[0], (_Float16)acc[1], (_Float16)acc[2], (_Float16)acc[3]};  // round to nearest even
+      *reinterpret_cast<half4 *>(out + ((int64_t)(kc + m) * V + 4 * g)) = h;
+    }
+  };
+
+  half8 b0[NC], b1[NC];
+  uint32_t c_next = load_cols(beg + 16);
+  load_rows(b0, load_cols(beg));
+  int kc = beg;
+  for (;;) {
+    // b0 holds group kc; c_next the columns of group kc + 16
+    if (kc + 16 >= end) {
+      finish(b0, kc);
+      break;
+    }
+    uint32_t c_after = load_cols(kc + 32);
+    load_rows(b1, c_next);
+    finish(b0, kc);
+    kc += 16;
+    if (kc + 16 >= end) {
+      finish(b1, kc);
+      break;
+    }
+    c_next = load_cols(kc + 32);
+    load_rows(b0, c_after);
+    finish(b1, kc);
+    kc += 16;
+  }
+}
+
+template <int V, int NC>
+static hipError_t launch_sddmm_nc(const SddmmArgs &a, hipStream_t stream) {
+  SddmmArgs p = a;
+  p.total_work = (uint32_t)a.m_vec * (uint32_t)a.batch;
+  p.per_xcd = (p.total_work + 7u) / 8u;
+  if (p.total_work == 0) return hipSuccess;
+  hipLaunchKernelGGL((sddmm_kernel<V, NC>), dim3(p.per_xcd * 8u), dim3(64), 0, stream, p);
+  return hipGetLastError();
+}
+
+template <int V>
+static hipError_t launch_sddmm_v(const SddmmArgs &a, hipStream_t stream) {
+  const int nc = (a.F + 31) / 32;
+  if (nc <= 1) return launch_sddmm_nc<V, 1>(a, stream);
+  if (nc <= 2) return launch_sddmm_nc<V, 2>(a, stream);
+  if (nc <= 4) return launch_sddmm_nc<V, 4>(a, stream);
+  return launch_sddmm_nc<V, 8>(a, stream);
+}
+
+hipError_t launch_sddmm(const SddmmArgs &a, int V, hipStream_t stream) {
+  return V == 8 ? launch_sddmm_v<8>(a, stream) : launch_sddmm_v<16>(a, stream);
+}
+
+// ---------------------------------------------------------------------------------- softmax
+namespace {
+
+__device__ __forceinline__ float wave_max(float x) {
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) x = fmaxf(x, __shfl_xor(x, d, 64));
+  return x;
+}
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) x += __shfl_xor(x, d, 64);
+  return x;
+}
+
+template <int V>
+struct VecLoad;  // the V halfs of one stored vector
+template <>
+struct VecLoad<8> {
+  static __device__ __forceinline__ void load(const uint16_t *p, _Float16 (&x)[8]) {
+    const half8 h = *reinterpret_cast<const half8 *>(p);
+#pragma unroll
+    for (int v = 0; v < 8; ++v) x[v] = h[v];
+  }
+  static __device__ __forceinline__ void store(uint16_t *p, const _Float16 (&x)[8]) {
+    half8 h;
+#pragma unroll
+    for (int v = 0; v < 8; ++v) h[v] = x[v];
+    *reinterpret_cast<half8 *>(p) = h;
+  }
+};
+template <>
+struct VecLoad<16> {
+  static __device__ __forceinline__ void load(const uint16_t *p, _Float16 (&x)[16]) {
+    const half8 lo = *reinterpret_cast<const half8 *>(p), hi = *reinterpret_cast<const half8 *>(p + 8);
+#pragma unroll
+    for (int v = 0; v < 8; ++v) {
+      x[v] = lo[v];
+      x[8 + v] = hi[v];
+    }
+  }
+  static __device__ __forceinline__ void store(uint16_t *p, const _Float16 (&x)[16]) {
+    half8 lo, hi;
+#pragma unroll
+    for (int v = 0; v < 8; ++v) {
+      lo[v] = x[v];
+      hi[v] = x[8 + v];
+    }
+    *reinterpret_cast<half8 *>(p) = lo;
+    *reinterpret_cast<half8 *>(p + 8) = hi;
+  }
+};
+
+}  // namespace
+
+// One wave per (vector-row, batch element); lane l takes the stored vectors l, l + 64, ... of the
+// row, V dense rows at a time.  Three passes over the row's values (maximum, sum of exponentials,
+// result): the first comes from HBM, the other two hit the caches.
+template <int V>
+__global__ __launch_bounds__(64) void softmax_kernel(const SoftmaxArgs p) {
+  const uint32_t w = xcd_work_index(p.per_xcd);
+  if (w >= p.total_work) return;
+  const uint32_t r = w % (uint32_t)p.m_vec;
+  const uint32_t batch = w / (uint32_t)p.m_vec;
+  const int row = p.row_indices ? p.row_indices[r] : (int)r;
+  const int beg = p.row_offsets[row], end = p.row_offsets[row + 1];
+  if (beg == end) return;
+  const int lane = threadIdx.x;
+  const uint16_t *in = p.values + (int64_t)batch * p.stride;
+  uint16_t *out = p.out + (int64_t)batch * p.stride;
+  const float s = p.scaler;
+
+  float mx[V], sum[V];
+#pragma unroll
+  for (int v = 0; v < V; ++v) {
+    mx[v] = -INFINITY;
+    sum[v] = 0.f;
+  }
+  for (int j = beg + lane; j < end; j += 64) {
+    _Float16 x[V];
+    VecLoad<V>::load(in + (int64_t)j * V, x);
+#pragma unroll
+    for (int v = 0; v < V; ++v) mx[v] = fmaxf(mx[v], (float)x[v] * s);
+  }
+#pragma unroll
+  for (int v = 0; v < V; ++v) mx[v] = wave_max(mx[v]);
+  for (int j = beg + lane; j < end; j += 64) {
+    _Float16 x[V];
+    VecLoad<V>::load(in + (int64_t)j * V, x);
+#pragma unroll
+    for (int v = 0; v < V; ++v) sum[v] += __expf((float)x[v] * s - mx[v]);
+  }
+#pragma unroll
+  for (int v = 0; v < V; ++v) sum[v] = 1.0f / wave_sum(sum[v]);
+  for (int j = beg + lane; j < end; j += 64) {
+    _Float16 x[V], y[V];
+    VecLoad<V>::load(in + (int64_t)j * V, x);
+#pragma unroll
+    for (int v = 0; v < V; ++v) y[v] = (_Float16)(__expf((float)x[v] * s - mx[v]) * sum[v]);
+    VecLoad<V>::store(out + (int64_t)j * V, y);
+  }
+}
+
+hipError_t launch_softmax(const SoftmaxArgs &a, int V, hipStream_t stream) {
+  SoftmaxArgs p = a;
+  p.total_work = (uint32_t)a.m_vec * (uint32_t)a.batch;
+  p.per_xcd = (p.total_work + 7u) / 8u;
+  if (p.total_work == 0) return hipSuccess;
+  if (V == 8)
+    hipLaunchKernelGGL(softmax_kernel<8>, dim3(p.per_xcd * 8u), dim3(64), 0, stream, p);
+  else
+    hipLaunchKernelGGL(softmax_kernel<16>, dim3(p.per_xcd * 8u), dim3(64), 0, stream, p);
+  return hipGetLastError();
+}
+
+}  // namespace sspmm

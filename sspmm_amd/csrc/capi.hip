@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 
 #include "../../include/sspmm.h"
+#include "attention_kernels.h"
 #include "spmm_kernels.h"
 #include "svc_kernels.h"
 
@@ -93,6 +94,72 @@ int sspmm_sorted_row_swizzle(int m_vec, const int32_t *row_offsets, int32_t *row
   if (m_vec == 0) return 0;
   if (!row_offsets || !row_indices) return kInvalid;
   return (int)sspmm::launch_sorted_row_swizzle(m_vec, row_offsets, row_indices, static_cast<hipStream_t>(hip_stream));
+}
+
+int sspmm_sddmm_batched_f16(int batch, int m_vec, int V, int F, int n_rhs, const int32_t *row_indices,
+                            const int32_t *row_offsets, const int32_t *col_idx, const sspmm_half_t *lhs,
+                            int64_t stride_lhs, const sspmm_half_t *rhs, int64_t stride_rhs, sspmm_half_t *out_values,
+                            int64_t stride_out, void *hip_stream) {
+  if (V != 8 && V != 16) return kInvalid;
+  if (batch < 0 || m_vec < 0 || F < 0 || n_rhs < 0) return kInvalid;
+  if (F % 8 != 0 || F > 256) return kInvalid;
+  if (batch == 0 || m_vec == 0) return 0;
+  if (!row_offsets) return kInvalid;
+  if ((int64_t)n_rhs * F >= (1ll << 31) || (int64_t)m_vec * batch >= (1ll << 31) - 8) return kInvalid;
+  if (reinterpret_cast<uintptr_t>(lhs) % 16 || reinterpret_cast<uintptr_t>(rhs) % 16 ||
+      reinterpret_cast<uintptr_t>(out_values) % 8 || stride_lhs % 8 || stride_rhs % 8 || stride_out % 4)
+    return kInvalid;
+  if (batch > 1 && (stride_lhs < 0 || stride_rhs < 0 || stride_out < 0)) return kInvalid;
+  sspmm::SddmmArgs a{};
+  a.m_vec = m_vec;
+  a.F = F;
+  a.n_rhs = n_rhs;
+  a.batch = batch;
+  a.row_indices = row_indices;
+  a.row_offsets = row_offsets;
+  a.col_idx = col_idx;
+  a.lhs = lhs;
+  a.rhs = rhs;
+  a.out = out_values;
+  a.stride_lhs = stride_lhs;
+  a.stride_rhs = stride_rhs;
+  a.stride_out = stride_out;
+  return (int)sspmm::launch_sddmm(a, V, static_cast<hipStream_t>(hip_stream));
+}
+
+int sspmm_sddmm_f16(int m_vec, int V, int F, int n_rhs, const int32_t *row_indices, const int32_t *row_offsets,
+                    const int32_t *col_idx, const sspmm_half_t *lhs, const sspmm_half_t *rhs, sspmm_half_t *out_values,
+                    void *hip_stream) {
+  return sspmm_sddmm_batched_f16(1, m_vec, V, F, n_rhs, row_indices, row_offsets, col_idx, lhs, 0, rhs, 0, out_values, 0,
+                                 hip_stream);
+}
+
+int sspmm_softmax_batched_f16(int batch, int m_vec, int V, const int32_t *row_indices, const int32_t *row_offsets,
+                              const sspmm_half_t *values, float scaler, sspmm_half_t *out_values, int64_t stride,
+                              void *hip_stream) {
+  if (V != 8 && V != 16) return kInvalid;
+  if (batch < 0 || m_vec < 0) return kInvalid;
+  if (batch == 0 || m_vec == 0) return 0;
+  if (!row_offsets) return kInvalid;
+  if ((int64_t)m_vec * batch >= (1ll << 31) - 8) return kInvalid;
+  if (reinterpret_cast<uintptr_t>(values) % 16 || reinterpret_cast<uintptr_t>(out_values) % 16 || stride % 8 ||
+      (batch > 1 && stride < 0))
+    return kInvalid;
+  sspmm::SoftmaxArgs a{};
+  a.m_vec = m_vec;
+  a.batch = batch;
+  a.row_indices = row_indices;
+  a.row_offsets = row_offsets;
+  a.values = values;
+  a.out = out_values;
+  a.stride = stride;
+  a.scaler = scaler;
+  return (int)sspmm::launch_softmax(a, V, static_cast<hipStream_t>(hip_stream));
+}
+
+int sspmm_softmax_f16(int m_vec, int V, const int32_t *row_indices, const int32_t *row_offsets,
+                      const sspmm_half_t *values, float scaler, sspmm_half_t *out_values, void *hip_stream) {
+  return sspmm_softmax_batched_f16(1, m_vec, V, row_indices, row_offsets, values, scaler, out_values, 0, hip_stream);
 }
 
 size_t svc_workspace_bytes(int M, int64_t nnz, int V) {

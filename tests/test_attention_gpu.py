@@ -1,0 +1,126 @@
+"""GPU parity of the sampled product, the sparse softmax and the attention block that chains them
+with the batched SpMM, through the C ABI, against the CPU oracle and dense torch arithmetic."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import sspmm_amd
+from sspmm_amd import synth
+from gpu_util import dev, max_rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def _pattern(m_rows, K, V, sparsity, seed):
+    return synth.vector_sparse(m_rows * V, K, V, sparsity, seed=seed)
+
+
+@pytest.mark.parametrize("V", [8, 16])
+@pytest.mark.parametrize("F", [8, 40, 64, 128, 200, 256])
+def test_sddmm_matches_oracle(oracle, built_library, V, F):
+    vs = _pattern(20, 300, V, 0.8, seed=100 + F)
+    rng = np.random.default_rng(F)
+    lhs = rng.standard_normal((vs.m_vec * V, F)).astype(np.float16)
+    rhs = rng.standard_normal((300, F)).astype(np.float16)
+    print("sddmm V=%d F=%d nvec=%d" % (V, F, vs.col_idx.size), flush=True)
+    got = sspmm_amd.sddmm(None, dev(vs.row_offsets), dev(vs.col_idx), dev(lhs), dev(rhs), V)
+    torch.cuda.synchronize()
+    want = oracle.sddmm(vs.m_vec, V, vs.row_offsets, vs.col_idx, lhs, rhs)
+    assert got.shape == (vs.col_idx.size * V,)
+    assert max_rel_err(got.cpu().numpy(), want) <= 2e-3
+    # exact on small integers (every product and partial sum is representable)
+    lhs_i = rng.integers(-3, 4, lhs.shape).astype(np.float16)
+    rhs_i = rng.integers(-3, 4, rhs.shape).astype(np.float16)
+    got = sspmm_amd.sddmm(None, dev(vs.row_offsets), dev(vs.col_idx), dev(lhs_i), dev(rhs_i), V).cpu().numpy()
+    assert np.array_equal(got, oracle.sddmm(vs.m_vec, V, vs.row_offsets, vs.col_idx, lhs_i, rhs_i))
+
+
+@pytest.mark.parametrize("per_row", [0, 1, 15, 16, 17, 31, 32, 33, 100])
+def test_sddmm_row_length_tails_and_permutation(oracle, built_library, per_row):
+    V, K, F, m_vec = 8, 128, 64, 6
+    rng = np.random.default_rng(per_row)
+    cols = np.concatenate([rng.permutation(K)[:per_row] for _ in range(m_vec)] or [[]]).astype(np.int32)
+    off = (np.arange(m_vec + 1) * per_row).astype(np.int32)
+    lhs = rng.standard_normal((m_vec * V, F)).astype(np.float16)
+    rhs = rng.standard_normal((K, F)).astype(np.float16)
+    want = oracle.sddmm(m_vec, V, off, cols, lhs, rhs)
+    perm = dev(rng.permutation(m_vec).astype(np.int32))
+    for ri in (None, perm):
+        got = sspmm_amd.sddmm(ri, dev(off), dev(cols) if cols.size else torch.empty(0, dtype=torch.int32, device="cuda"),
+                              dev(lhs), dev(rhs), V)
+        torch.cuda.synchronize()
+        assert got.numel() == cols.size * V
+        if cols.size:
+            assert max_rel_err(got.cpu().numpy(), want) <= 2e-3
+
+
+@pytest.mark.parametrize("V", [8, 16])
+def test_softmax_matches_oracle_and_rows_sum_to_one(oracle, built_library, V):
+    rng = np.random.default_rng(7)
+    lens = np.array([0, 1, 5, 64, 65, 200, 0, 1000, 3])
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    vals = (rng.standard_normal(off[-1] * V) * 4).astype(np.float16)
+    scaler = 1.0 / math.sqrt(64)
+    got = sspmm_amd.csr_softmax(None, dev(off), dev(vals), scaler, V)
+    torch.cuda.synchronize()
+    got = got.cpu().numpy()
+    want = oracle.softmax(len(lens), V, off, vals, scaler)
+    assert np.abs(got.astype(np.float64) - want.astype(np.float64)).max() <= 2e-3
+    g = got.astype(np.float64).reshape(-1, V)
+    for i, n in enumerate(lens):
+        if n:
+            assert np.all(np.abs(g[off[i]:off[i + 1]].sum(axis=0) - 1) < 1e-2)
+    # a large common offset must not overflow: softmax is shift invariant
+    big = (vals.astype(np.float32) + 30000).astype(np.float16)
+    shifted = sspmm_amd.csr_softmax(None, dev(off), dev(big), 1.0, V).cpu().numpy()
+    assert np.isfinite(shifted).all()
+
+
+def test_batched_ops_match_looped_single_calls(oracle, built_library):
+    V, K, F, batch = 8, 160, 64, 5
+    vs = _pattern(16, K, V, 0.85, seed=9)
+    rng = np.random.default_rng(10)
+    q = rng.standard_normal((batch, vs.m_vec * V, F)).astype(np.float16)
+    k = rng.standard_normal((batch, K, F)).astype(np.float16)
+    off, col = dev(vs.row_offsets), dev(vs.col_idx)
+    w = sspmm_amd.bsddmm(None, off, col, dev(q), dev(k), V)
+    p = sspmm_amd.bcsr_softmax(None, off, w, 0.125, V, batch)
+    torch.cuda.synchronize()
+    assert w.shape == (batch, vs.col_idx.size * V) and p.shape == w.shape
+    for b in range(batch):
+        assert torch.equal(w[b], sspmm_amd.sddmm(None, off, col, dev(q[b]), dev(k[b]), V))
+        assert torch.equal(p[b], sspmm_amd.csr_softmax(None, off, w[b].contiguous(), 0.125, V))
+
+
+@pytest.mark.parametrize("V", [8, 16])
+def test_sparse_attention_matches_dense_masked_attention(built_library, V):
+    """The reference's block (sddmm -> softmax -> spmm) against torch attention with a -inf mask."""
+    seq, d, batch = 256, 64, 6
+    vs = _pattern(seq // V, seq, V, 0.8, seed=11)
+    g = torch.Generator("cuda").manual_seed(12)
+    q, k, v = (torch.randn(batch, seq, d, device="cuda", generator=g).half() for _ in range(3))
+    out = sspmm_amd.sparse_attention(None, dev(vs.row_offsets), dev(vs.col_idx), q, k, v, 1.0 / math.sqrt(d), V)
+    torch.cuda.synchronize()
+    mask = torch.full((seq, seq), float("-inf"), device="cuda")
+    for i in range(vs.m_vec):
+        cols = torch.from_numpy(vs.col_idx[vs.row_offsets[i]:vs.row_offsets[i + 1]].astype(np.int64)).cuda()
+        mask[i * V:(i + 1) * V, cols] = 0
+    scores = q.float() @ k.float().transpose(1, 2) / math.sqrt(d) + mask
+    want = torch.softmax(scores, dim=-1) @ v.float()
+    assert out.shape == (batch, seq, d) and out.dtype == torch.float16
+    assert max_rel_err(out.float().cpu().numpy(), want.cpu().numpy()) <= 1e-2
+
+
+def test_argument_errors(built_library):
+    off = torch.zeros(3, dtype=torch.int32, device="cuda")
+    col = torch.zeros(0, dtype=torch.int32, device="cuda")
+    with pytest.raises(ValueError):
+        sspmm_amd.sddmm(None, off, col, torch.zeros(16, 64, device="cuda").half(), torch.zeros(8, 64, device="cuda").half(), 4)
+    with pytest.raises(ValueError):
+        sspmm_amd.sddmm(None, off, col, torch.zeros(16, 64, device="cuda").half(), torch.zeros(8, 32, device="cuda").half(), 8)
+    with pytest.raises(TypeError):
+        sspmm_amd.csr_softmax(None, off, torch.zeros(0, device="cuda"), 1.0, 8)
+    with pytest.raises(RuntimeError):  # F must be a multiple of 8
+        sspmm_amd.sddmm(None, off, col, torch.zeros(16, 12, device="cuda").half(), torch.zeros(8, 12, device="cuda").half(), 8)

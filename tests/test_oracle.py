@@ -181,3 +181,62 @@ def test_sorted_row_swizzle_invariants(oracle):
     assert sorted(perm.tolist()) == list(range(300))
     assert np.all(np.diff(lens[perm]) <= 0)
     assert np.array_equal(perm, np.argsort(-lens, kind="stable"))
+
+
+@pytest.mark.parametrize("V", [8, 16])
+def test_sddmm_oracle_vs_dense_matmul_sampled_at_the_pattern(oracle, V):
+    """out[j*V+v] must be entry (i*V+v, col_j) of lhs @ rhs.T: a transposed operand, a wrong row or a
+    wrong vector-major index all show up as O(1) errors."""
+    vs = synth.vector_sparse(6 * V, 50, V, 0.7, seed=80 + V)
+    rng = np.random.default_rng(81)
+    F = 40
+    lhs = rng.standard_normal((vs.m_vec * V, F)).astype(np.float16)
+    rhs = rng.standard_normal((50, F)).astype(np.float16)
+    got = oracle.sddmm(vs.m_vec, V, vs.row_offsets, vs.col_idx, lhs, rhs).astype(np.float64).reshape(-1, V)
+    dense = lhs.astype(np.float64) @ rhs.astype(np.float64).T
+    for i in range(vs.m_vec):
+        for j in range(vs.row_offsets[i], vs.row_offsets[i + 1]):
+            want = dense[i * V:(i + 1) * V, vs.col_idx[j]]
+            assert np.all(np.abs(got[j] - want) <= 2e-3 * max(1.0, np.abs(want).max()) + 2e-3)
+    # exact case: small integers
+    lhs_i = rng.integers(-3, 4, lhs.shape).astype(np.float16)
+    rhs_i = rng.integers(-3, 4, rhs.shape).astype(np.float16)
+    got = oracle.sddmm(vs.m_vec, V, vs.row_offsets, vs.col_idx, lhs_i, rhs_i).astype(np.float64).reshape(-1, V)
+    dense = lhs_i.astype(np.float64) @ rhs_i.astype(np.float64).T
+    for i in range(vs.m_vec):
+        for j in range(vs.row_offsets[i], vs.row_offsets[i + 1]):
+            assert np.array_equal(got[j], dense[i * V:(i + 1) * V, vs.col_idx[j]])
+
+
+@pytest.mark.parametrize("V", [8, 16])
+def test_softmax_oracle_vs_dense_softmax_with_minus_inf_fill(oracle, V):
+    """The reference's own check: softmax over the dense rows with -inf where nothing is stored."""
+    K = 70
+    vs = synth.vector_sparse(5 * V, K, V, 0.6, seed=90 + V)
+    lens = np.diff(vs.row_offsets)
+    rng = np.random.default_rng(91)
+    vals = (rng.standard_normal(vs.col_idx.size * V) * 3).astype(np.float16)
+    scaler = 0.37
+    got = oracle.softmax(vs.m_vec, V, vs.row_offsets, vals, scaler).astype(np.float64).reshape(-1, V)
+    dense = np.full((vs.m_vec * V, K), -np.inf)
+    vv = vals.reshape(-1, V).astype(np.float64)
+    for i in range(vs.m_vec):
+        for j in range(vs.row_offsets[i], vs.row_offsets[i + 1]):
+            dense[i * V:(i + 1) * V, vs.col_idx[j]] = vv[j]
+    x = dense * scaler
+    e = np.exp(x - x.max(axis=1, keepdims=True))
+    ref = e / e.sum(axis=1, keepdims=True)
+    for i in range(vs.m_vec):
+        for j in range(vs.row_offsets[i], vs.row_offsets[i + 1]):
+            want = ref[i * V:(i + 1) * V, vs.col_idx[j]]
+            assert np.all(np.abs(got[j] - want) <= 1e-3 * want + 1e-6)
+    assert lens.min() > 0
+    # each dense row sums to one; a row with a single entry is exactly one
+    sums = np.zeros(vs.m_vec * V)
+    for i in range(vs.m_vec):
+        sums[i * V:(i + 1) * V] = got[vs.row_offsets[i]:vs.row_offsets[i + 1]].sum(axis=0)
+    assert np.all(np.abs(sums - 1) < 5e-3)
+    one = oracle.softmax(1, V, np.array([0, 1], np.int32), np.arange(V).astype(np.float16), 2.0)
+    assert np.array_equal(one, np.ones(V, np.float16))
+    # empty vector-rows write nothing
+    assert oracle.softmax(3, V, np.array([0, 0, 1, 1], np.int32), np.zeros(V, np.float16), 1.0).tolist() == [1.0] * V

@@ -285,6 +285,31 @@ def main():
             "projections": per,
         }
 
+        # the sparse attention block of the reference (bsddmm -> bcsr_softmax -> bspmm) on one mask shared by
+        # 48 heads: 4096 tokens, head size 64, V=8, 90 % of the vectors masked out
+        seqA, dA, VA, bA = 4096, 64, 8, 48
+        mk_a = synth.vector_sparse(seqA, seqA, VA, 0.9, seed=7)
+        offA, colA = torch.from_numpy(mk_a.row_offsets).cuda(), torch.from_numpy(mk_a.col_idx).cuda()
+        qA, kA, vA = (torch.randn(bA, seqA, dA, device="cuda").half() for _ in range(3))
+        nvA = mk_a.col_idx.size
+        wA = sspmm_amd.bsddmm(None, offA, colA, qA, kA, VA)
+        pA = sspmm_amd.bcsr_softmax(None, offA, wA, 0.125, VA, bA)
+        t_sddmm = time_launches(lambda: sspmm_amd.bsddmm(None, offA, colA, qA, kA, VA), st, wu)
+        t_soft = time_launches(lambda: sspmm_amd.bcsr_softmax(None, offA, wA, 0.125, VA, bA), st, wu)
+        t_av = time_launches(lambda: sspmm_amd.bspmm(None, offA, colA, pA, vA, VA), st, wu)
+        t_dense = time_launches(lambda: torch.nn.functional.scaled_dot_product_attention(qA, kA, vA), st, wu)
+        by_sddmm = bA * (2 * seqA * dA * 2 + 2 * nvA * VA) + 4 * nvA + 4 * (mk_a.m_vec + 1)
+        by_soft = bA * 2 * 2 * nvA * VA + 4 * (mk_a.m_vec + 1)
+        by_av = bA * (2 * nvA * VA + 2 * seqA * dA + 2 * seqA * dA) + 4 * nvA + 4 * (mk_a.m_vec + 1)
+        extra["sparse_attention_seq4096_d64_v8_s0.9_heads48"] = {
+            "bsddmm_ms": t_sddmm, "bsddmm_hbm_frac": by_sddmm / t_sddmm / 1e6 / HBM_PEAK_GBPS, "bsddmm_alg_bytes": by_sddmm,
+            "bcsr_softmax_ms": t_soft, "bcsr_softmax_hbm_frac": by_soft / t_soft / 1e6 / HBM_PEAK_GBPS,
+            "bcsr_softmax_alg_bytes": by_soft,
+            "bspmm_ms": t_av, "bspmm_hbm_frac": by_av / t_av / 1e6 / HBM_PEAK_GBPS, "bspmm_alg_bytes": by_av,
+            "block_ms": t_sddmm + t_soft + t_av, "dense_sdpa_ms": t_dense, "nvec": int(nvA),
+        }
+        del qA, kA, vA, wA, pA
+
     line = {
         "metric": "SpMM useful TFLOP/s (2*nnz*N/t), V=8 @90% sparsity, fp16 in / fp32 accumulate",
         "value": main_res["useful_tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,

@@ -239,6 +239,22 @@ def test_slab_kernel_work_item_lists(oracle, built_library, V, batch, m_rows, K,
         assert max_rel_err(out[b], want) <= tol, b
 
 
+@pytest.mark.parametrize("V,K", [(8, 574), (8, 575), (16, 512), (16, 543), (16, 544), (8, 1150), (16, 1100), (8, 1300)])
+def test_slab_kernel_around_its_lds_limits(oracle, built_library, V, K):
+    """K just below and above what two slabs (then one slab) leave room for in LDS; beyond the last limit the
+    forced choice falls back to the gather kernel."""
+    from sspmm_amd import _lib
+    vs = synth.vector_sparse(80 * V, K, V, 0.95, seed=K)
+    B = synth.dense_rhs(K, 192, seed=K + 1)
+    _lib.lib().sspmm_select_kernel(3)
+    try:
+        check(oracle, vs, B, torch.float32)
+        ran = _lib.lib().sspmm_last_kernel()
+    finally:
+        _lib.lib().sspmm_select_kernel(0)
+    assert ran == (3 if K <= 1150 else 2)
+
+
 def test_row_swizzle_matches_oracle(oracle, built_library):
     rng = np.random.default_rng(3)
     for m_vec in [1, 5, 255, 256, 257, 3000]:

@@ -45,15 +45,15 @@ __device__ __forceinline__ void probe_start(uint32_t key, uint32_t mask, uint32_
   lin = 0;
 }
 
+// (written with selects: lanes of a wave are at different points of their probe sequences, and a
+// branch here would make every wave walk both sides)
 __device__ __forceinline__ void probe_next(uint32_t mask, uint32_t &i, uint32_t &perturb, uint32_t &lin) {
-  const uint32_t window = (i + 9u <= mask) ? 9u : 0u;
-  if (lin < window) {
-    ++lin;
-  } else {
-    perturb >>= 5;
-    i = (i * 5u + 1u + perturb) & mask;
-    lin = 0;
-  }
+  const bool in_window = (lin < 9u) & (i + 9u <= mask);
+  const uint32_t shifted = perturb >> 5;
+  const uint32_t jumped = (i * 5u + 1u + shifted) & mask;
+  lin = in_window ? lin + 1u : 0u;
+  perturb = in_window ? perturb : shifted;
+  i = in_window ? i : jumped;
 }
 
 // Slot that holds `key`, or -1.  The table always keeps free slots, so the walk ends.

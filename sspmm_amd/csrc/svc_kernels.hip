@@ -277,7 +277,12 @@ __device__ __forceinline__ void place32(const Table32 &t, uint32_t mask, uint32_
       // a later entry sat here: carry it on from this slot of its own probe sequence
       mine = old;
       probe_start(old & t.key_mask, mask, i, perturb, lin);
-      while (i + lin != s0) probe_next(mask, i, perturb, lin);
+      // nearly always it lost a slot of its first window: no walk needed then
+      const uint32_t d = s0 - i;
+      if ((d <= 9u) & ((i + 9u <= mask) | (d == 0u)))
+        lin = d;
+      else
+        while (i + lin != s0) probe_next(mask, i, perturb, lin);
     }
     probe_next(mask, i, perturb, lin);
   }

@@ -300,85 +300,157 @@ __device__ __forceinline__ void list_store(int *list, int idx, int v) {
   else __hip_atomic_store(list + idx, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// Writes the keys of a table to list[] in slot order and returns their number; with `final`, the
+// table entries are rewritten as (rank, key).  wcount: slots / 64 + 1 words of LDS.  Contains
+// barriers; the table must be complete (a barrier behind the last insert) on entry.
 template <int THREADS, bool LIST_IN_LDS>
-__device__ __forceinline__ uint32_t rebuild_set32(const Table32 &t, uint32_t *wcount, int *list, int &n, int *scratch) {
+__device__ __forceinline__ int compact_table32(const Table32 &t, uint32_t slots, uint32_t *wcount, int *list, bool final) {
   constexpr int WAVES = THREADS / 64;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  (void)scratch;
-  uint32_t slots = 8;
+  const uint32_t words = slots >= 64u ? slots / 64u : 1u;
+  for (uint32_t w = wave; w < words; w += WAVES) {
+    const uint32_t s = w * 64u + lane;
+    const bool occ = s < slots && t.slots[s] != kEmpty32;
+    const unsigned long long m = __ballot(occ);
+    if (lane == 0) wcount[w] = (uint32_t)__popcll(m);
+  }
+  __syncthreads();
+  if (wave == 0) {  // running counts over the words
+    uint32_t carry = 0;
+    for (uint32_t w0 = 0; w0 < words; w0 += 64) {
+      const uint32_t w = w0 + lane;
+      const uint32_t c = w < words ? wcount[w] : 0u;
+      uint32_t incl = c;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t y = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += y;
+      }
+      if (w < words) wcount[w] = carry + incl - c;
+      carry += __shfl(incl, 63, 64);
+    }
+    if (lane == 0) wcount[words] = carry;  // number of keys in the table
+  }
+  __syncthreads();
+  for (uint32_t w = wave; w < words; w += WAVES) {
+    const uint32_t s = w * 64u + lane;
+    const uint32_t x = s < slots ? t.slots[s] : kEmpty32;
+    const bool occ = x != kEmpty32;
+    const unsigned long long m = __ballot(occ);
+    const uint32_t rank = wcount[w] + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+    if (occ) {
+      list_store<LIST_IN_LDS>(list, (int)rank, (int)(x & t.key_mask));
+      if (final) t.slots[s] = (rank << t.key_bits) | (x & t.key_mask);
+    }
+  }
+  const int kept = (int)wcount[words];
+  __syncthreads();
+  return kept;
+}
+
+// The two table regions of a group: consecutive phases of a construction alternate between them,
+// so that a phase can re-insert the previous phase's table straight from its slots.
+struct TableRegions {
+  uint32_t *a, *b;        // LDS
+  uint32_t cap_a, cap_b;  // in slots; cap_a = the largest table of the class
+};
+
+// One `set(list)` of CPython on the keys list[0 .. n): leaves the final table in t (entries
+// (rank in slot order, key)), the keys in slot order in list[], and returns the table's size.
+// A phase inserts the previous phase's keys in its slot order, then further keys of the list in
+// list order; all that first-come-first-served placement needs of the insertion indices is their
+// order, so the previous table's slot number serves as the index of a re-inserted key and no
+// compaction is needed between phases.  Only where the next table does not fit the other region
+// is the old table first compacted into the list.
+template <int THREADS, bool LIST_IN_LDS>
+__device__ __forceinline__ uint32_t rebuild_set32(Table32 &t, const TableRegions &reg, int *list, int &n) {
+  const int tid = threadIdx.x;
+  uint32_t slots = 8, old_slots = 0;
+  uint32_t *cur = nullptr;
+  int prev_cnt = 0;
+  // the largest table must land in region a: start so that the alternation ends there
+  uint32_t phases_to_max = 0;
+  for (uint32_t s8 = 8; s8 < reg.cap_a; s8 <<= 2) ++phases_to_max;
+  bool next_in_a = (phases_to_max & 1u) == 0u;
   for (;;) {
     const uint32_t thr = resize_threshold(slots);
     const int cnt = min(n, (int)thr);
     const uint32_t mask = slots - 1u;
-    for (uint32_t s = tid; s < slots; s += THREADS) t.slots[s] = kEmpty32;
-    __syncthreads();
-    // A thread inserts its keys in list order (idx = tid, tid + THREADS, ...), so the whole group works
-    // through the list in chunks of THREADS keys and a later key rarely arrives before an earlier
-    // one.  The keys are fetched eight at a time ahead of the inserts: one round trip per batch.
-    for (int base = tid; base < cnt; base += 8 * THREADS) {
-      int k8[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int idx = base + j * THREADS;
-        k8[j] = idx < cnt ? list_load<LIST_IN_LDS>(list, idx) : 0;
-      }
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int idx = base + j * THREADS;
-        if (idx < cnt) place32(t, mask, (uint32_t)k8[j], (uint32_t)idx);
-      }
+    uint32_t *nt = next_in_a ? reg.a : reg.b;
+    const uint32_t nt_cap = next_in_a ? reg.cap_a : reg.cap_b;
+    bool from_list = cur == nullptr;
+    if (slots > nt_cap) {
+      // the other region is too small: slot order goes to the list and the table is rebuilt in place
+      Table32 old = t;
+      old.slots = cur;
+      compact_table32<THREADS, LIST_IN_LDS>(old, old_slots, nt, list, false);
+      nt = cur;
+      from_list = true;
     }
+    uint32_t *other = nt == reg.a ? reg.b : reg.a;
+    t.slots = nt;
+    for (uint32_t s = tid; s < slots; s += THREADS) nt[s] = kEmpty32;
     __syncthreads();
-    const bool final = n < (int)thr;
-    const uint32_t words = slots >= 64u ? slots / 64u : 1u;
-    for (uint32_t w = wave; w < words; w += WAVES) {
-      const uint32_t s = w * 64u + lane;
-      const bool occ = s < slots && t.slots[s] != kEmpty32;
-      const unsigned long long m = __ballot(occ);
-      if (lane == 0) wcount[w] = (uint32_t)__popcll(m);
-    }
-    __syncthreads();
-    if (wave == 0) {  // running counts over the words
-      uint32_t carry = 0;
-      for (uint32_t w0 = 0; w0 < words; w0 += 64) {
-        const uint32_t w = w0 + lane;
-        const uint32_t c = w < words ? wcount[w] : 0u;
-        uint32_t incl = c;
+    if (from_list) {
+      // A thread inserts its keys in list order (idx = tid, tid + THREADS, ...), so the whole group works
+      // through the list in chunks of THREADS keys and a later key rarely arrives before an earlier
+      // one.  The keys are fetched eight at a time ahead of the inserts: one round trip per batch.
+      for (int base = tid; base < cnt; base += 8 * THREADS) {
+        int k8[8];
 #pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-          const uint32_t y = __shfl_up(incl, d, 64);
-          if (lane >= d) incl += y;
+        for (int j = 0; j < 8; ++j) {
+          const int idx = base + j * THREADS;
+          k8[j] = idx < cnt ? list_load<LIST_IN_LDS>(list, idx) : 0;
         }
-        if (w < words) wcount[w] = carry + incl - c;
-        carry += __shfl(incl, 63, 64);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int idx = base + j * THREADS;
+          if (idx < cnt) place32(t, mask, (uint32_t)k8[j], (uint32_t)idx);
+        }
       }
-      if (lane == 0) wcount[words] = carry;  // number of keys in the table
+    } else {
+      // the previous table's keys, indexed by their slot, and the list keys behind them
+      for (uint32_t base = tid; base < old_slots; base += 8 * THREADS) {
+        uint32_t x8[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const uint32_t s = base + j * THREADS;
+          x8[j] = s < old_slots ? cur[s] : kEmpty32;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if (x8[j] != kEmpty32) place32(t, mask, x8[j] & t.key_mask, base + j * THREADS);
+      }
+      for (int base = prev_cnt + tid; base < cnt; base += 8 * THREADS) {
+        int k8[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int idx = base + j * THREADS;
+          k8[j] = idx < cnt ? list_load<LIST_IN_LDS>(list, idx) : 0;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int idx = base + j * THREADS;
+          if (idx < cnt) place32(t, mask, (uint32_t)k8[j], old_slots + (uint32_t)(idx - prev_cnt));
+        }
+      }
     }
     __syncthreads();
-    for (uint32_t w = wave; w < words; w += WAVES) {
-      const uint32_t s = w * 64u + lane;
-      const uint32_t x = s < slots ? t.slots[s] : kEmpty32;
-      const bool occ = x != kEmpty32;
-      const unsigned long long m = __ballot(occ);
-      const uint32_t rank = wcount[w] + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
-      if (occ) {
-        list_store<LIST_IN_LDS>(list, (int)rank, (int)(x & t.key_mask));
-        if (final) t.slots[s] = (rank << t.key_bits) | (x & t.key_mask);
-      }
-    }
-    const int kept = (int)wcount[words];
-    __syncthreads();
-    if (final) {
-      n = kept;
+    if (n < (int)thr) {
+      n = compact_table32<THREADS, LIST_IN_LDS>(t, slots, other, list, true);
       return slots;
     }
+    cur = nt;
+    old_slots = slots;
+    prev_cnt = cnt;
+    next_in_a = nt != reg.a;
     slots = resized_slots(thr);
   }
 }
 
 template <int THREADS, bool LIST_IN_LDS>
 __global__ __launch_bounds__(THREADS) void svc_merge_fast_kernel(const SvcArgs a, int class_lo, int class_hi,
-                                                                 uint32_t key_bits, uint32_t max_slots) {
+                                                                 uint32_t key_bits, uint32_t max_slots, uint32_t small_slots) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int grp = blockIdx.x;
   const int r0 = grp * a.V, r1 = min(a.M, r0 + a.V);
@@ -392,10 +464,12 @@ __global__ __launch_bounds__(THREADS) void svc_merge_fast_kernel(const SvcArgs a
   t.slots = reinterpret_cast<uint32_t *>(smem + 128);
   t.key_bits = key_bits;
   t.key_mask = (1u << key_bits) - 1u;
-  const uint32_t max_words = max_slots >= 64u ? max_slots / 64u : 1u;
-  uint32_t *wcount = reinterpret_cast<uint32_t *>(smem + 128 + (size_t)max_slots * 4);  // max_words + 1 entries
-  int *list = LIST_IN_LDS ? reinterpret_cast<int *>(smem + 128 + (size_t)max_slots * 4 + (size_t)(max_words + 1) * 4)
-                          : a.tmp_cols + e0;
+  TableRegions reg;
+  reg.a = t.slots;
+  reg.cap_a = max_slots;
+  reg.b = t.slots + max_slots;
+  reg.cap_b = small_slots;
+  int *list = LIST_IN_LDS ? reinterpret_cast<int *>(smem + 128 + ((size_t)max_slots + small_slots) * 4) : a.tmp_cols + e0;
   const int cap = LIST_IN_LDS ? min(class_hi, bound) : bound;
 
   int n = 0;
@@ -419,7 +493,7 @@ __global__ __launch_bounds__(THREADS) void svc_merge_fast_kernel(const SvcArgs a
     }
     n = min(n + appended, cap);  // the cap only bites for invalid input (repeated columns)
     __syncthreads();
-    slots = rebuild_set32<THREADS, LIST_IN_LDS>(t, wcount, list, n, scratch);
+    slots = rebuild_set32<THREADS, LIST_IN_LDS>(t, reg, list, n);
   }
 
   if (tid == 0) a.vec_row_ptr[grp + 1] = n;
@@ -552,15 +626,19 @@ static hipError_t launch_lds_class(const SvcArgs &base, int m_vec, int lo, int h
 template <int THREADS, bool LIST_IN_LDS>
 static hipError_t launch_fast_class(const SvcArgs &a, int m_vec, int lo, int hi, uint32_t slots, uint32_t key_bits,
                                     hipStream_t stream) {
-  const uint32_t words = slots >= 64u ? slots / 64u : 1u;
-  const size_t lds = 128 + (size_t)slots * 4 + (size_t)(words + 1) * 4 + (LIST_IN_LDS ? (size_t)hi * 4 : 0);
+  // second table region: a quarter of the first (what the phase before the largest needs), less where LDS is short;
+  // it also serves as the running-count array of the compaction of a table in the first region (slots / 64 + 1 words)
+  uint32_t small_slots = slots / 4u;
+  while (128 + ((size_t)slots + small_slots) * 4 + (LIST_IN_LDS ? (size_t)hi * 4 : 0) > 160 * 1024) small_slots /= 4u;
+  if (small_slots < slots / 64u + 1u) return hipErrorInvalidValue;
+  const size_t lds = 128 + ((size_t)slots + small_slots) * 4 + (LIST_IN_LDS ? (size_t)hi * 4 : 0);
   auto kern = svc_merge_fast_kernel<THREADS, LIST_IN_LDS>;
   if (lds > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
   }
-  hipLaunchKernelGGL(kern, dim3(m_vec), dim3(THREADS), lds, stream, a, lo, hi, key_bits, slots);
+  hipLaunchKernelGGL(kern, dim3(m_vec), dim3(THREADS), lds, stream, a, lo, hi, key_bits, slots, small_slots);
   return hipGetLastError();
 }
 

@@ -689,21 +689,23 @@ hipError_t launch_svc_count(const SvcArgs &a, int order, hipStream_t stream) {
     int top = kLargeKeys;
     if (key_bits <= 17) {
       // 32-bit table entries: 15 bits of insertion index are enough up to 19 660 keys
-      if ((e = launch_fast_class<64, true>(a, m_vec, -1, kSmallKeys, 512, key_bits, st[0])) != hipSuccess) return e;
-      if ((e = launch_fast_class<256, true>(a, m_vec, kSmallKeys, kMediumKeys, 2048, key_bits, st[1])) != hipSuccess)
+      // the classes of the largest groups go out first, the largest on the caller's stream: a single group of
+      // thousands of keys takes longer than all the small groups together
+      if ((e = launch_fast_class<1024, false>(a, m_vec, kLargeKeys, kXLargeKeys, 32768, key_bits, st[0])) != hipSuccess)
         return e;
-      if ((e = launch_fast_class<1024, true>(a, m_vec, kMediumKeys, kLargeKeys, 8192, key_bits, st[2])) != hipSuccess)
+      if ((e = launch_fast_class<1024, true>(a, m_vec, kMediumKeys, kLargeKeys, 8192, key_bits, st[1])) != hipSuccess)
         return e;
-      if ((e = launch_fast_class<1024, false>(a, m_vec, kLargeKeys, kXLargeKeys, 32768, key_bits, st[3])) != hipSuccess)
+      if ((e = launch_fast_class<256, true>(a, m_vec, kSmallKeys, kMediumKeys, 2048, key_bits, st[2])) != hipSuccess)
         return e;
+      if ((e = launch_fast_class<64, true>(a, m_vec, -1, kSmallKeys, 512, key_bits, st[3])) != hipSuccess) return e;
       top = kXLargeKeys;
     } else {
       if ((e = launch_lds_class<64>(a, m_vec, -1, kSmallKeys, 512, st[0])) != hipSuccess) return e;
       if ((e = launch_lds_class<256>(a, m_vec, kSmallKeys, kMediumKeys, 2048, st[1])) != hipSuccess) return e;
       if ((e = launch_lds_class<1024>(a, m_vec, kMediumKeys, kLargeKeys, 8192, st[2])) != hipSuccess) return e;
     }
-    hipLaunchKernelGGL((svc_merge_cpython_kernel<1024, false>), dim3(m_vec), dim3(1024), 128, st[3], a, top, 0x7fffffff,
-                       0);
+    hipLaunchKernelGGL((svc_merge_cpython_kernel<1024, false>), dim3(m_vec), dim3(1024), 128,
+                       key_bits <= 17 ? st[0] : st[3], a, top, 0x7fffffff, 0);
     if ((e = hipGetLastError()) != hipSuccess) return e;
     if (ss) {
       for (int i = 0; i < 3; ++i) {

@@ -247,6 +247,7 @@ __global__ __launch_bounds__(THREADS) void svc_merge_cpython_kernel(const SvcArg
 // population of every word, wave 0 turns them into running counts, and a second pass writes
 // list[count[word] + rank in word] = key, so nothing is scanned per thread.
 static constexpr uint32_t kEmpty32 = 0xffffffffu;
+static constexpr int kGaveUp = -1;  // vec_row_ptr entry of a group whose launch found it too large
 
 struct Table32 {
   uint32_t *slots;  // LDS
@@ -450,13 +451,16 @@ __device__ __forceinline__ uint32_t rebuild_set32(Table32 &t, const TableRegions
 
 template <int THREADS, bool LIST_IN_LDS>
 __global__ __launch_bounds__(THREADS) void svc_merge_fast_kernel(const SvcArgs a, int class_lo, int class_hi,
-                                                                 uint32_t key_bits, uint32_t max_slots, uint32_t small_slots) {
+                                                                 uint32_t key_bits, uint32_t max_slots, uint32_t small_slots,
+                                                                 int only_flagged) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int grp = blockIdx.x;
   const int r0 = grp * a.V, r1 = min(a.M, r0 + a.V);
   const int e0 = a.row_ptr[r0], e1 = a.row_ptr[r1];
   const int bound = min(e1 - e0, a.K);
   if (!in_class(bound, class_lo, class_hi)) return;  // uniform over the group
+  // second chance for a group that an earlier launch on this stream gave up on (see kGaveUp)
+  if (only_flagged && a.vec_row_ptr[grp + 1] != kGaveUp) return;
   const int tid = threadIdx.x;
 
   int *scratch = reinterpret_cast<int *>(smem);  // 32 ints
@@ -493,6 +497,12 @@ __global__ __launch_bounds__(THREADS) void svc_merge_fast_kernel(const SvcArgs a
     }
     n = min(n + appended, cap);  // the cap only bites for invalid input (repeated columns)
     __syncthreads();
+    if ((uint32_t)n >= resize_threshold(max_slots)) {
+      // more distinct columns than this launch's tables take: only a group admitted on the strength of its
+      // distinct columns being fewer than its non-zeros gets here; it is left to the launch that follows
+      if (tid == 0) a.vec_row_ptr[grp + 1] = kGaveUp;
+      return;
+    }
     slots = rebuild_set32<THREADS, LIST_IN_LDS>(t, reg, list, n);
   }
 
@@ -606,7 +616,7 @@ size_t svc_workspace_layout(int64_t nnz, size_t *off_pos, size_t *off_tables) {
   return cols + pos + tables;
 }
 
-static constexpr int kSmallKeys = 306, kMediumKeys = 1228, kLargeKeys = 4914, kXLargeKeys = 19660;
+static constexpr int kSmallKeys = 306, kMediumKeys = 1228, kLargeKeys = 4914, kHopefulKeys = 7600, kXLargeKeys = 19660;
 
 template <int THREADS>
 static hipError_t launch_lds_class(const SvcArgs &base, int m_vec, int lo, int hi, int slots, hipStream_t stream) {
@@ -625,7 +635,7 @@ static hipError_t launch_lds_class(const SvcArgs &base, int m_vec, int lo, int h
 
 template <int THREADS, bool LIST_IN_LDS>
 static hipError_t launch_fast_class(const SvcArgs &a, int m_vec, int lo, int hi, uint32_t slots, uint32_t key_bits,
-                                    hipStream_t stream) {
+                                    hipStream_t stream, int only_flagged = 0) {
   // second table region: a quarter of the first (what the phase before the largest needs), less where LDS is short;
   // it also serves as the running-count array of the compaction of a table in the first region (slots / 64 + 1 words)
   uint32_t small_slots = slots / 4u;
@@ -638,7 +648,7 @@ static hipError_t launch_fast_class(const SvcArgs &a, int m_vec, int lo, int hi,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
   }
-  hipLaunchKernelGGL(kern, dim3(m_vec), dim3(THREADS), lds, stream, a, lo, hi, key_bits, slots, small_slots);
+  hipLaunchKernelGGL(kern, dim3(m_vec), dim3(THREADS), lds, stream, a, lo, hi, key_bits, slots, small_slots, only_flagged);
   return hipGetLastError();
 }
 
@@ -689,11 +699,16 @@ hipError_t launch_svc_count(const SvcArgs &a, int order, hipStream_t stream) {
     int top = kLargeKeys;
     if (key_bits <= 17) {
       // 32-bit table entries: 15 bits of insertion index are enough up to 19 660 keys
-      // the classes of the largest groups go out first, the largest on the caller's stream: a single group of
-      // thousands of keys takes longer than all the small groups together
-      if ((e = launch_fast_class<1024, false>(a, m_vec, kLargeKeys, kXLargeKeys, 32768, key_bits, st[0])) != hipSuccess)
+      // The classes of the largest groups go out first, the 8192-slot class on the caller's stream: a single
+      // group of thousands of keys takes longer than all the small groups together.
+      // A group's class is decided from its non-zeros, an upper bound of its distinct columns.  Groups a little
+      // above the limit of the 8192-slot class are tried there all the same (a merged group of long rows repeats
+      // many columns); one that does outgrow the table marks itself and is redone by the launch behind it.
+      if ((e = launch_fast_class<1024, true>(a, m_vec, kMediumKeys, kHopefulKeys, 8192, key_bits, st[0])) != hipSuccess)
         return e;
-      if ((e = launch_fast_class<1024, true>(a, m_vec, kMediumKeys, kLargeKeys, 8192, key_bits, st[1])) != hipSuccess)
+      if ((e = launch_fast_class<1024, false>(a, m_vec, kLargeKeys, kHopefulKeys, 32768, key_bits, st[0], 1)) != hipSuccess)
+        return e;
+      if ((e = launch_fast_class<1024, false>(a, m_vec, kHopefulKeys, kXLargeKeys, 32768, key_bits, st[1])) != hipSuccess)
         return e;
       if ((e = launch_fast_class<256, true>(a, m_vec, kSmallKeys, kMediumKeys, 2048, key_bits, st[2])) != hipSuccess)
         return e;

@@ -75,7 +75,7 @@ def test_against_python_set_directly(oracle, built_library, V):
     assert vrp.tolist() == ptr and vcol.tolist() == flat
 
 
-@pytest.mark.parametrize("keys", [300, 310, 1200, 1240, 4800, 5000, 9000])
+@pytest.mark.parametrize("keys", [300, 310, 1200, 1240, 4800, 5000, 7590, 7610, 9000])
 def test_every_group_size_class(oracle, built_library, keys):
     """Groups whose distinct-column bound falls into each kernel class (LDS 64 / 256 / 1024 threads,
     and tables in the workspace), next to empty and tiny groups."""
@@ -90,6 +90,28 @@ def test_every_group_size_class(oracle, built_library, keys):
     csr = synth.Csr(40, K, ptr, cols, rng.standard_normal(cols.size).astype(np.float16))
     _compare_with_oracle(oracle, csr, V)
     _compare_with_oracle(oracle, csr, 16)
+
+
+@pytest.mark.parametrize("distinct", [3000, 4914, 4915, 5600])
+def test_groups_admitted_on_the_hope_of_repeated_columns(oracle, built_library, distinct):
+    """A group with 6400 non-zeros is tried in the class that takes up to 4914 distinct columns; whether it
+    finishes there (its rows repeat columns) or has to be redone by the next launch, the result is the same."""
+    rng = np.random.default_rng(distinct)
+    V, K, per_row = 8, 16384, 800
+    pool = rng.permutation(K)[:distinct]
+    rows = []
+    covered = 0
+    for r in range(V):  # every pool column occurs, rows repeat columns of one another
+        must = pool[covered:covered + per_row]
+        covered += must.size
+        rest = rng.choice(pool, per_row - must.size, replace=False) if must.size < per_row else np.empty(0, np.int64)
+        rows.append(np.unique(np.concatenate([must, rest])))
+    lens = np.array([0] * 8 + [len(x) for x in rows] + [5] * 8)
+    cols = np.concatenate([np.empty(0, np.int64)] * 8 + rows + [rng.permutation(K)[:5] for _ in range(8)]).astype(np.int32)
+    ptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    csr = synth.Csr(24, K, ptr, cols, rng.standard_normal(cols.size).astype(np.float16))
+    vrp, _, _ = _compare_with_oracle(oracle, csr, V)
+    assert vrp[2] - vrp[1] == distinct
 
 
 def test_cfg1_rowmerge_returns_the_vector_pattern(oracle, built_library):

@@ -587,10 +587,14 @@ __global__ __launch_bounds__(THREADS) void svc_fill_kernel(const SvcArgs a, cons
   if (vec_col)
     for (int p = threadIdx.x; p < n; p += THREADS) vec_col[v0 + p] = a.tmp_cols[e0 + p];
   if (!vec_val) return;
-  // A group's value region starts at v0 * V halfs: a multiple of 4 bytes whenever V is even.
+  // A group's value region starts at v0 * V halfs and holds n * V of them: whole 16-byte pieces when V is a
+  // multiple of 8 (and vec_val is 16-byte aligned), 4-byte pieces whenever V is even.
   const int64_t halfs = (int64_t)n * a.V;
   uint16_t *out = vec_val + (int64_t)v0 * a.V;
-  if ((a.V & 1) == 0) {
+  if ((a.V & 7) == 0 && (reinterpret_cast<uintptr_t>(vec_val) & 15) == 0) {
+    uint4 *out128 = reinterpret_cast<uint4 *>(out);
+    for (int64_t t = threadIdx.x; t < halfs / 8; t += THREADS) out128[t] = uint4{0u, 0u, 0u, 0u};
+  } else if ((a.V & 1) == 0) {
     uint32_t *out32 = reinterpret_cast<uint32_t *>(out);
     for (int64_t t = threadIdx.x; t < halfs / 2; t += THREADS) out32[t] = 0u;
   } else {
@@ -720,7 +724,7 @@ hipError_t launch_svc_count(const SvcArgs &a, int order, hipStream_t stream) {
       if ((e = launch_lds_class<1024>(a, m_vec, kMediumKeys, kLargeKeys, 8192, st[2])) != hipSuccess) return e;
     }
     hipLaunchKernelGGL((svc_merge_cpython_kernel<1024, false>), dim3(m_vec), dim3(1024), 128,
-                       key_bits <= 17 ? st[0] : st[3], a, top, 0x7fffffff, 0);
+                       key_bits <= 17 ? st[1] : st[3], a, top, 0x7fffffff, 0);
     if ((e = hipGetLastError()) != hipSuccess) return e;
     if (ss) {
       for (int i = 0; i < 3; ++i) {
@@ -748,7 +752,7 @@ hipError_t launch_svc_count(const SvcArgs &a, int order, hipStream_t stream) {
 hipError_t launch_svc_fill(const SvcArgs &a, const uint16_t *csr_val, const int32_t *vec_row_ptr, int32_t *vec_col,
                            uint16_t *vec_val, hipStream_t stream) {
   const int m_vec = (a.M + a.V - 1) / a.V;
-  hipLaunchKernelGGL((svc_fill_kernel<256>), dim3(m_vec), dim3(256), 0, stream, a, csr_val, vec_row_ptr, vec_col,
+  hipLaunchKernelGGL((svc_fill_kernel<512>), dim3(m_vec), dim3(512), 0, stream, a, csr_val, vec_row_ptr, vec_col,
                      csr_val ? vec_val : nullptr);
   return hipGetLastError();
 }

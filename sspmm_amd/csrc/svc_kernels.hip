@@ -309,11 +309,19 @@ __device__ __forceinline__ int compact_table32(const Table32 &t, uint32_t slots,
   constexpr int WAVES = THREADS / 64;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t words = slots >= 64u ? slots / 64u : 1u;
-  for (uint32_t w = wave; w < words; w += WAVES) {
-    const uint32_t s = w * 64u + lane;
-    const bool occ = s < slots && t.slots[s] != kEmpty32;
-    const unsigned long long m = __ballot(occ);
-    if (lane == 0) wcount[w] = (uint32_t)__popcll(m);
+  // (four words per trip, their loads in flight together: these passes are chains of LDS round trips)
+  for (uint32_t w0 = wave; w0 < words; w0 += 4 * WAVES) {
+    uint32_t x[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t s = (w0 + j * WAVES) * 64u + lane;
+      x[j] = s < slots ? t.slots[s] : kEmpty32;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const unsigned long long m = __ballot(x[j] != kEmpty32);
+      if (lane == 0 && w0 + j * WAVES < words) wcount[w0 + j * WAVES] = (uint32_t)__popcll(m);
+    }
   }
   __syncthreads();
   if (wave == 0) {  // running counts over the words
@@ -333,15 +341,25 @@ __device__ __forceinline__ int compact_table32(const Table32 &t, uint32_t slots,
     if (lane == 0) wcount[words] = carry;  // number of keys in the table
   }
   __syncthreads();
-  for (uint32_t w = wave; w < words; w += WAVES) {
-    const uint32_t s = w * 64u + lane;
-    const uint32_t x = s < slots ? t.slots[s] : kEmpty32;
-    const bool occ = x != kEmpty32;
-    const unsigned long long m = __ballot(occ);
-    const uint32_t rank = wcount[w] + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
-    if (occ) {
-      list_store<LIST_IN_LDS>(list, (int)rank, (int)(x & t.key_mask));
-      if (final) t.slots[s] = (rank << t.key_bits) | (x & t.key_mask);
+  for (uint32_t w0 = wave; w0 < words; w0 += 4 * WAVES) {
+    uint32_t x[4], before[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t w = w0 + j * WAVES;
+      const uint32_t s = w * 64u + lane;
+      x[j] = s < slots ? t.slots[s] : kEmpty32;
+      before[j] = w < words ? wcount[w] : 0u;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t s = (w0 + j * WAVES) * 64u + lane;
+      const bool occ = x[j] != kEmpty32;
+      const unsigned long long m = __ballot(occ);
+      const uint32_t rank = before[j] + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+      if (occ) {
+        list_store<LIST_IN_LDS>(list, (int)rank, (int)(x[j] & t.key_mask));
+        if (final) t.slots[s] = (rank << t.key_bits) | (x[j] & t.key_mask);
+      }
     }
   }
   const int kept = (int)wcount[words];
@@ -356,19 +374,60 @@ struct TableRegions {
   uint32_t cap_a, cap_b;  // in slots; cap_a = the largest table of the class
 };
 
+// The inserts of one phase by STRIDE cooperating threads, `me` the caller's index among them: either
+// list[0 .. cnt) (insertion index = list index), or the previous table's keys, indexed by their
+// slot, and the list keys [prev_cnt, cnt) behind them.  A thread inserts its keys in order
+// (me, me + STRIDE, ...), so the threads work through the keys in chunks and a later key rarely
+// arrives before an earlier one; keys are fetched eight at a time ahead of the inserts.
+template <int STRIDE, bool LIST_IN_LDS>
+__device__ __forceinline__ void phase_insert(const Table32 &t, uint32_t mask, const int *list, int cnt, const uint32_t *old_table,
+                                             uint32_t old_slots, int prev_cnt, int me) {
+  if (old_table != nullptr) {
+    for (uint32_t base = me; base < old_slots; base += 8 * STRIDE) {
+      uint32_t x8[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const uint32_t s = base + j * STRIDE;
+        x8[j] = s < old_slots ? old_table[s] : kEmpty32;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (x8[j] != kEmpty32) place32(t, mask, x8[j] & t.key_mask, base + j * STRIDE);
+    }
+  }
+  const uint32_t first_index = old_table != nullptr ? old_slots : 0u;
+  for (int base = prev_cnt + me; base < cnt; base += 8 * STRIDE) {
+    int k8[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int idx = base + j * STRIDE;
+      k8[j] = idx < cnt ? list_load<LIST_IN_LDS>(list, idx) : 0;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int idx = base + j * STRIDE;
+      if (idx < cnt) place32(t, mask, (uint32_t)k8[j], first_index + (uint32_t)(idx - prev_cnt));
+    }
+  }
+}
+
 // One `set(list)` of CPython on the keys list[0 .. n): leaves the final table in t (entries
 // (rank in slot order, key)), the keys in slot order in list[], and returns the table's size.
 // A phase inserts the previous phase's keys in its slot order, then further keys of the list in
 // list order; all that first-come-first-served placement needs of the insertion indices is their
 // order, so the previous table's slot number serves as the index of a re-inserted key and no
 // compaction is needed between phases.  Only where the next table does not fit the other region
-// is the old table first compacted into the list.
+// is the old table first compacted into the list.  The phases of the smallest tables (a few dozen
+// keys) are run by the first wave alone, without workgroup barriers.
+static constexpr uint32_t kSoloSlots = 128;
 template <int THREADS, bool LIST_IN_LDS>
 __device__ __forceinline__ uint32_t rebuild_set32(Table32 &t, const TableRegions &reg, int *list, int &n) {
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   uint32_t slots = 8, old_slots = 0;
   uint32_t *cur = nullptr;
   int prev_cnt = 0;
+  bool solo_pending = false;  // the first wave ran phases on its own that the others have not waited for yet
   // the largest table must land in region a: start so that the alternation ends there
   uint32_t phases_to_max = 0;
   for (uint32_t s8 = 8; s8 < reg.cap_a; s8 <<= 2) ++phases_to_max;
@@ -379,65 +438,40 @@ __device__ __forceinline__ uint32_t rebuild_set32(Table32 &t, const TableRegions
     const uint32_t mask = slots - 1u;
     uint32_t *nt = next_in_a ? reg.a : reg.b;
     const uint32_t nt_cap = next_in_a ? reg.cap_a : reg.cap_b;
-    bool from_list = cur == nullptr;
+    const bool solo = THREADS > 64 && slots <= kSoloSlots && slots <= nt_cap;
+    if (!solo && solo_pending) {
+      __syncthreads();
+      solo_pending = false;
+    }
     if (slots > nt_cap) {
       // the other region is too small: slot order goes to the list and the table is rebuilt in place
       Table32 old = t;
       old.slots = cur;
+      prev_cnt = 0;
       compact_table32<THREADS, LIST_IN_LDS>(old, old_slots, nt, list, false);
       nt = cur;
-      from_list = true;
+      cur = nullptr;
     }
     uint32_t *other = nt == reg.a ? reg.b : reg.a;
     t.slots = nt;
-    for (uint32_t s = tid; s < slots; s += THREADS) nt[s] = kEmpty32;
-    __syncthreads();
-    if (from_list) {
-      // A thread inserts its keys in list order (idx = tid, tid + THREADS, ...), so the whole group works
-      // through the list in chunks of THREADS keys and a later key rarely arrives before an earlier
-      // one.  The keys are fetched eight at a time ahead of the inserts: one round trip per batch.
-      for (int base = tid; base < cnt; base += 8 * THREADS) {
-        int k8[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int idx = base + j * THREADS;
-          k8[j] = idx < cnt ? list_load<LIST_IN_LDS>(list, idx) : 0;
-        }
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int idx = base + j * THREADS;
-          if (idx < cnt) place32(t, mask, (uint32_t)k8[j], (uint32_t)idx);
-        }
+    if (solo) {
+      if (wave == 0) {
+        for (uint32_t s = lane; s < slots; s += 64) nt[s] = kEmpty32;
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");  // the wave's LDS operations execute in order
+        __builtin_amdgcn_wave_barrier();
+        phase_insert<64, LIST_IN_LDS>(t, mask, list, cnt, cur, old_slots, prev_cnt, lane);
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
+        __builtin_amdgcn_wave_barrier();
       }
+      solo_pending = true;
     } else {
-      // the previous table's keys, indexed by their slot, and the list keys behind them
-      for (uint32_t base = tid; base < old_slots; base += 8 * THREADS) {
-        uint32_t x8[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const uint32_t s = base + j * THREADS;
-          x8[j] = s < old_slots ? cur[s] : kEmpty32;
-        }
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-          if (x8[j] != kEmpty32) place32(t, mask, x8[j] & t.key_mask, base + j * THREADS);
-      }
-      for (int base = prev_cnt + tid; base < cnt; base += 8 * THREADS) {
-        int k8[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int idx = base + j * THREADS;
-          k8[j] = idx < cnt ? list_load<LIST_IN_LDS>(list, idx) : 0;
-        }
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int idx = base + j * THREADS;
-          if (idx < cnt) place32(t, mask, (uint32_t)k8[j], old_slots + (uint32_t)(idx - prev_cnt));
-        }
-      }
+      for (uint32_t s = tid; s < slots; s += THREADS) nt[s] = kEmpty32;
+      __syncthreads();
+      phase_insert<THREADS, LIST_IN_LDS>(t, mask, list, cnt, cur, old_slots, prev_cnt, tid);
+      __syncthreads();
     }
-    __syncthreads();
     if (n < (int)thr) {
+      if (solo_pending) __syncthreads();
       n = compact_table32<THREADS, LIST_IN_LDS>(t, slots, other, list, true);
       return slots;
     }

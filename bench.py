@@ -310,6 +310,40 @@ def main():
         }
         del qA, kA, vA, wA, pA
 
+        # row reordering ahead of the SVC: 16384 rows that are noisy copies of 256 prototype rows, shuffled
+        rc_csr = synth.clustered_csr(16384, 16384, 256, 128, seed=6, keep=0.9, extras=1)
+        rrp, rci, rcv = (torch.from_numpy(x).cuda() for x in (rc_csr.row_ptr, rc_csr.col_ind, rc_csr.values))
+        plain = sspmm_amd.svc(rrp, rci, rcv, rc_csr.M, rc_csr.K, 8, order="sorted")
+        reo = sspmm_amd.svc_reordered(rrp, rci, rcv, rc_csr.M, rc_csr.K, 8, order="sorted")
+        rws = torch.empty(L.svc_reorder_workspace_bytes(rc_csr.M), dtype=torch.uint8, device="cuda")
+        rperm = torch.empty(rc_csr.M, dtype=torch.int32, device="cuda")
+        o_rp, o_ci, o_cv = torch.empty_like(rrp), torch.empty_like(rci), torch.empty_like(rcv)
+
+        def reorder_order():
+            rc = L.svc_reorder_minhash(rc_csr.M, rrp.data_ptr(), rci.data_ptr(), rperm.data_ptr(), rws.data_ptr(),
+                                       rws.numel(), stream)
+            assert rc == 0, rc
+
+        def reorder_apply():
+            rc = L.svc_permute_csr(rc_csr.M, rperm.data_ptr(), rrp.data_ptr(), rci.data_ptr(), rcv.data_ptr(),
+                                   o_rp.data_ptr(), o_ci.data_ptr(), o_cv.data_ptr(), rws.data_ptr(), rws.numel(),
+                                   stream)
+            assert rc == 0, rc
+
+        reorder_order()
+        t_order = time_launches(reorder_order, 20, 3)
+        t_apply = time_launches(reorder_apply, 20, 3)
+        rnnz = int(rc_csr.col_ind.size)
+        by_order = 4 * (rc_csr.M + 1) + 4 * rnnz + 4 * rc_csr.M   # row pointer + columns read, order written
+        by_apply = 4 * rc_csr.M + 2 * 4 * (rc_csr.M + 1) + 2 * (4 + 2) * rnnz  # CSR read once, written once
+        extra["reorder_clustered_16384_v8"] = {
+            "workload": "16384 x 16384 CSR, rows = noisy copies of 256 prototypes (nnz %d), shuffled; V=8" % rnnz,
+            "order_ms": t_order, "order_alg_bytes": by_order, "order_hbm_gbps": by_order / t_order / 1e6,
+            "apply_ms": t_apply, "apply_alg_bytes": by_apply, "apply_hbm_gbps": by_apply / t_apply / 1e6,
+            "nvec_without_reordering": int(plain.num_vec), "nvec_with_reordering": int(reo.svc.num_vec),
+            "fill_without_reordering": rnnz / (plain.num_vec * 8.0), "fill_with_reordering": rnnz / (reo.svc.num_vec * 8.0),
+        }
+
     line = {
         "metric": "SpMM useful TFLOP/s (2*nnz*N/t), V=8 @90% sparsity, fp16 in / fp32 accumulate",
         "value": main_res["useful_tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,

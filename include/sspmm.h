@@ -155,6 +155,30 @@ int svc_fill(int M, int K, int V, const int32_t *row_ptr, const int32_t *col_ind
              int64_t nnz, int order, const int32_t *vec_row_ptr, void *workspace, int32_t *vec_col,
              sspmm_half_t *vec_val, void *hip_stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Row reordering ahead of the SVC: the step the reference runs as `python row_merge_reorder.py`
+ * (reference README.md:36) to write its dataset-v8 / dataset-v16 folders, which the harness
+ * reads when its `reorder` argument is 1 (reference SSpMM/sspmm_test.cpp:304, 313-320).  The
+ * reference's reorder module itself is absent from its sources (RowMerge/row_merge.py:8 imports
+ * it in a comment only), so the ordering method is this library's own: rows are sorted by a
+ * 64-bit key of two min-hashes of their column sets, ties in source order, which places rows
+ * with equal column sets next to each other and rows with similar ones near each other.
+ *
+ *   svc_reorder_minhash  writes perm[M]: row i of the reordered matrix is source row perm[i].
+ *   svc_permute_csr      writes the reordered CSR arrays (out_row_ptr[M+1], out_col[nnz] and,
+ *                        when csr_val != NULL, out_val[nnz]); feed them to svc_count / svc_fill.
+ * Both take a workspace of svc_reorder_workspace_bytes(M) bytes (0 = no usable device).
+ * perm must be a permutation of 0..M-1; entries outside that range give empty rows.
+ * ---------------------------------------------------------------------------------------- */
+size_t svc_reorder_workspace_bytes(int M);
+
+int svc_reorder_minhash(int M, const int32_t *row_ptr, const int32_t *col_ind, int32_t *perm, void *workspace,
+                        size_t workspace_bytes, void *hip_stream);
+
+int svc_permute_csr(int M, const int32_t *perm, const int32_t *row_ptr, const int32_t *col_ind,
+                    const sspmm_half_t *csr_val, int32_t *out_row_ptr, int32_t *out_col, sspmm_half_t *out_val,
+                    void *workspace, size_t workspace_bytes, void *hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -44,6 +44,10 @@ def lib():
         L.oracle_sddmm_f16.argtypes = [ctypes.c_int32] * 3 + [i32p, i32p, u16p, u16p, u16p]
         L.oracle_softmax_f16.restype = None
         L.oracle_softmax_f16.argtypes = [ctypes.c_int32] * 2 + [i32p, u16p, ctypes.c_float, u16p]
+        L.oracle_minhash_order.restype = None
+        L.oracle_minhash_order.argtypes = [ctypes.c_int32, i32p, i32p, i32p, ctypes.POINTER(ctypes.c_uint64)]
+        L.oracle_permute_csr.restype = None
+        L.oracle_permute_csr.argtypes = [ctypes.c_int32, i32p, i32p, i32p, u16p, i32p, i32p, u16p]
         L.oracle_h2f.restype = ctypes.c_float
         L.oracle_h2f.argtypes = [ctypes.c_uint16]
         L.oracle_f2h.restype = ctypes.c_uint16
@@ -139,6 +143,30 @@ def sorted_row_swizzle(row_offsets):
     out = np.empty(max(rows, 1), dtype=np.int32)
     lib().oracle_sorted_row_swizzle(rows, _p(row_offsets, ctypes.c_int32), _p(out, ctypes.c_int32))
     return out[:rows].copy()
+
+
+def minhash_order(M, row_ptr, col_ind, return_keys=False):
+    """Row order of the reordering step: stable argsort of the rows' two-min-hash keys."""
+    row_ptr, col_ind = _i32(row_ptr), _i32(col_ind)
+    perm = np.empty(max(M, 1), dtype=np.int32)
+    keys = np.empty(max(M, 1), dtype=np.uint64)
+    lib().oracle_minhash_order(M, _p(row_ptr, ctypes.c_int32), _p(col_ind, ctypes.c_int32), _p(perm, ctypes.c_int32),
+                               _p(keys, ctypes.c_uint64))
+    return (perm[:M].copy(), keys[:M].copy()) if return_keys else perm[:M].copy()
+
+
+def permute_csr(M, perm, row_ptr, col_ind, val=None):
+    """CSR arrays with row i taken from source row perm[i]."""
+    perm, row_ptr, col_ind = _i32(perm), _i32(row_ptr), _i32(col_ind)
+    nnz = int(row_ptr[M]) if M else 0
+    out_ptr = np.zeros(M + 1, dtype=np.int32)
+    out_col = np.empty(max(nnz, 1), dtype=np.int32)
+    v = None if val is None else _u16(val)
+    out_val = None if val is None else np.empty(max(nnz, 1), dtype=np.uint16)
+    lib().oracle_permute_csr(M, _p(perm, ctypes.c_int32), _p(row_ptr, ctypes.c_int32), _p(col_ind, ctypes.c_int32),
+                             None if v is None else _p(v, ctypes.c_uint16), _p(out_ptr, ctypes.c_int32),
+                             _p(out_col, ctypes.c_int32), None if v is None else _p(out_val, ctypes.c_uint16))
+    return out_ptr, out_col[:nnz].copy(), None if val is None else out_val[:nnz].copy().view(np.float16)
 
 
 def rowmerge_python(M, V, col_lists):

@@ -47,6 +47,17 @@
  *                           fp32, fp16 result.  Pinned by: numpy softmax of the
  *                           densified rows with -inf fill (the recipe of
  *                           end2end/sspmm_e2e/verify/softmax.py:36-38).
+ *   oracle_minhash_order /  the row reordering that runs ahead of the merge (the
+ *   oracle_permute_csr      reference's row_merge_reorder.py step, README.md:36).
+ *                           The reference's reorder module is not in its sources,
+ *                           so there is nothing of the reference to restate: this
+ *                           is the CPU statement of the library's own method
+ *                           (stable sort of the rows by two min-hashes of their
+ *                           column sets).  PARITY UNPINNED against the reference;
+ *                           checked by what the definition fixes (a permutation,
+ *                           equal column sets adjacent, keys independent of the
+ *                           column order within a row, empty rows last) and by
+ *                           numpy's stable argsort on the same keys.
  */
 #include <math.h>
 #include <stdint.h>
@@ -348,6 +359,61 @@ void oracle_sorted_row_swizzle(int32_t rows, const int32_t *row_offsets, int32_t
   qsort(t, rows, sizeof(lenidx), cmp_lenidx_desc);
   for (int32_t i = 0; i < rows; ++i) row_indices[i] = t[i].idx;
   free(t);
+}
+
+/* -------------------------------------------------------- row reordering */
+
+static uint32_t mix32(uint32_t x) {
+  x ^= x >> 16;
+  x *= 0x85ebca6bu;
+  x ^= x >> 13;
+  x *= 0xc2b2ae35u;
+  x ^= x >> 16;
+  return x;
+}
+
+typedef struct {
+  uint64_t key;
+  int32_t idx;
+} keyidx;
+
+static int cmp_keyidx(const void *a, const void *b) {
+  const keyidx *x = (const keyidx *)a, *y = (const keyidx *)b;
+  if (x->key != y->key) return (x->key > y->key) - (x->key < y->key);
+  return (x->idx > y->idx) - (x->idx < y->idx);
+}
+
+/* keys[i] = min over the row's columns of mix32(c ^ seed1), << 32, | the same with seed2;
+ * perm = argsort of the keys, ties by ascending row.  keys may be NULL. */
+void oracle_minhash_order(int32_t M, const int32_t *row_ptr, const int32_t *col_ind, int32_t *perm, uint64_t *keys) {
+  keyidx *t = (keyidx *)malloc((size_t)(M > 0 ? M : 1) * sizeof(keyidx));
+  for (int32_t i = 0; i < M; ++i) {
+    uint32_t h1 = 0xffffffffu, h2 = 0xffffffffu;
+    for (int32_t e = row_ptr[i]; e < row_ptr[i + 1]; ++e) {
+      const uint32_t c = (uint32_t)col_ind[e];
+      const uint32_t a = mix32(c ^ 0x9e3779b9u), b = mix32(c ^ 0x7f4a7c15u);
+      if (a < h1) h1 = a;
+      if (b < h2) h2 = b;
+    }
+    t[i].key = ((uint64_t)h1 << 32) | h2;
+    t[i].idx = i;
+    if (keys) keys[i] = t[i].key;
+  }
+  qsort(t, M, sizeof(keyidx), cmp_keyidx);
+  for (int32_t i = 0; i < M; ++i) perm[i] = t[i].idx;
+  free(t);
+}
+
+/* out row i = source row perm[i]; val / out_val may be NULL. */
+void oracle_permute_csr(int32_t M, const int32_t *perm, const int32_t *row_ptr, const int32_t *col_ind,
+                        const uint16_t *val, int32_t *out_row_ptr, int32_t *out_col, uint16_t *out_val) {
+  out_row_ptr[0] = 0;
+  for (int32_t i = 0; i < M; ++i) {
+    const int32_t s0 = row_ptr[perm[i]], n = row_ptr[perm[i] + 1] - s0, d0 = out_row_ptr[i];
+    memcpy(out_col + d0, col_ind + s0, (size_t)n * sizeof(int32_t));
+    if (val) memcpy(out_val + d0, val + s0, (size_t)n * sizeof(uint16_t));
+    out_row_ptr[i + 1] = d0 + n;
+  }
 }
 
 /* ------------------------------------------------- sparse attention steps */

@@ -11,6 +11,7 @@ operator raises.
 from .spmm import spmm, bspmm, sorted_row_swizzle  # noqa: F401
 from .svc import svc, SvcResult  # noqa: F401
 from .attention import sddmm, bsddmm, csr_softmax, bcsr_softmax, sparse_attention  # noqa: F401
+from .reorder import minhash_order, permute_csr, svc_reordered  # noqa: F401
 from .layers import SparseLinear, SparseEncoderLayer  # noqa: F401
 from .formats import Cvse, read_smtx, write_smtx, read_cvse, write_cvse, cvse_text  # noqa: F401
 from ._lib import build_library, library_path  # noqa: F401

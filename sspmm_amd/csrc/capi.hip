@@ -4,6 +4,7 @@
 
 #include "../../include/sspmm.h"
 #include "attention_kernels.h"
+#include "reorder_kernels.h"
 #include "spmm_kernels.h"
 #include "svc_kernels.h"
 
@@ -209,6 +210,28 @@ int svc_fill(int M, int K, int V, const int32_t *row_ptr, const int32_t *col_ind
   if (rc) return rc;
   if (M == 0) return 0;
   return (int)sspmm::launch_svc_fill(a, csr_val, vec_row_ptr, vec_col, vec_val, static_cast<hipStream_t>(hip_stream));
+}
+
+size_t svc_reorder_workspace_bytes(int M) { return sspmm::reorder_workspace_bytes(M); }
+
+int svc_reorder_minhash(int M, const int32_t *row_ptr, const int32_t *col_ind, int32_t *perm, void *workspace,
+                        size_t workspace_bytes, void *hip_stream) {
+  if (M < 0) return kInvalid;
+  if (M == 0) return 0;
+  if (!row_ptr || !perm || !workspace) return kInvalid;
+  return (int)sspmm::launch_minhash_order(M, row_ptr, col_ind, perm, workspace, workspace_bytes,
+                                          static_cast<hipStream_t>(hip_stream));
+}
+
+int svc_permute_csr(int M, const int32_t *perm, const int32_t *row_ptr, const int32_t *col_ind,
+                    const sspmm_half_t *csr_val, int32_t *out_row_ptr, int32_t *out_col, sspmm_half_t *out_val,
+                    void *workspace, size_t workspace_bytes, void *hip_stream) {
+  if (M < 0 || !out_row_ptr) return kInvalid;
+  if (M > 0 && (!perm || !row_ptr || !workspace)) return kInvalid;
+  if (csr_val && !out_val) return kInvalid;
+  return (int)sspmm::launch_permute_csr(M, perm, row_ptr, col_ind, csr_val, out_row_ptr, out_col,
+                                        csr_val ? out_val : nullptr, workspace, workspace_bytes,
+                                        static_cast<hipStream_t>(hip_stream));
 }
 
 }  // extern "C"

@@ -10,6 +10,12 @@ dense ROW x COL copy of the matrix (`:176-188`); here the count is m_vec * COL -
 number, from the merged row pointer.
 
     python -m sspmm_amd.rowmerge <src_dir> <dest_dir> <paths.txt> <vec_len> [--csv stats.csv] [--order cpython|sorted]
+                                 [--reorder]
+
+`--reorder` is the reference's second pass (`python row_merge_reorder.py`, README.md:36, which
+writes the dataset-v8 / dataset-v16 folders): the rows are first brought into the order of
+sspmm_amd.reorder.minhash_order, then merged; the row order is written next to each output file
+as `<file>.perm` (one line of space-separated source row numbers).
 """
 import argparse
 import csv
@@ -45,27 +51,35 @@ def csv_row(index, stats):
     return [str(index)] + [str(stats[c]) for c in CSV_COLUMNS]
 
 
-def convert_file(src_path, dest_path, vec_len, order="cpython"):
+def convert_file(src_path, dest_path, vec_len, order="cpython", reorder=False):
     """One `.smtx` file -> one CVSE file, merged on the GPU.  Returns the statistics dict."""
     import torch
 
     from . import formats
     from .svc import svc
     M, K, nnz, row_ptr, col_ind = formats.read_smtx(src_path)
-    r = svc(torch.from_numpy(row_ptr).cuda(), torch.from_numpy(col_ind).cuda(), None, M, K, vec_len, order=order)
-    vec_row_ptr = r.vec_row_ptr.cpu().numpy()
+    rp, ci = torch.from_numpy(row_ptr).cuda(), torch.from_numpy(col_ind).cuda()
     os.makedirs(os.path.dirname(os.path.abspath(dest_path)), exist_ok=True)
+    if reorder:
+        from .reorder import minhash_order, permute_csr
+        perm = minhash_order(rp, ci, M)
+        rp, ci, _ = permute_csr(rp, ci, None, perm)
+        with open(dest_path + ".perm", "w") as f:
+            f.write(" ".join(map(str, perm.cpu().tolist())))
+    r = svc(rp, ci, None, M, K, vec_len, order=order)
+    vec_row_ptr = r.vec_row_ptr.cpu().numpy()
     formats.write_cvse(dest_path, vec_row_ptr.size - 1, K, nnz, vec_row_ptr, r.vec_col.cpu().numpy())
     return statistics(M, K, nnz, vec_len, vec_row_ptr)
 
 
-def generate_cvse_files(src_dir, dest_dir, paths_txt, vec_len, csv_path=None, order="cpython", log=None):
+def generate_cvse_files(src_dir, dest_dir, paths_txt, vec_len, csv_path=None, order="cpython", log=None,
+                        reorder=False):
     """Every file named in paths_txt (first token of each line, relative to src_dir / dest_dir)."""
     with open(paths_txt) as f:
         names = [line.split()[0] for line in f if line.split()]
     rows = []
     for i, name in enumerate(names):
-        stats = convert_file(os.path.join(src_dir, name), os.path.join(dest_dir, name), vec_len, order)
+        stats = convert_file(os.path.join(src_dir, name), os.path.join(dest_dir, name), vec_len, order, reorder)
         rows.append(csv_row(i, stats))
         if log:
             log("No. %d  OK  %s" % (i, os.path.join(dest_dir, name)))
@@ -83,8 +97,10 @@ def main(argv=None):
     ap.add_argument("vec_len", type=int, choices=[8, 16])
     ap.add_argument("--csv", default=None, help="append the statistics rows to this file")
     ap.add_argument("--order", default="cpython", choices=["cpython", "sorted"])
+    ap.add_argument("--reorder", action="store_true", help="sort the rows by min-hash key before merging")
     a = ap.parse_args(argv)
-    rows = generate_cvse_files(a.src_dir, a.dest_dir, a.paths_txt, a.vec_len, a.csv, a.order, log=print)
+    rows = generate_cvse_files(a.src_dir, a.dest_dir, a.paths_txt, a.vec_len, a.csv, a.order, log=print,
+                               reorder=a.reorder)
     print("Row-Merge (V = %d) format transformation finish: %d files" % (a.vec_len, len(rows)))
     return 0
 

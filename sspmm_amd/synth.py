@@ -4,6 +4,8 @@ vector_sparse():  a matrix that is already vector-sparse: every group of V rows 
                   column set (round((1 - sparsity) * K) distinct columns per vector-row, uniform
                   without replacement, stored ascending), values N(0, std).
 zipf_csr():       an unstructured CSR matrix with power-law row lengths, the input of the SVC.
+clustered_csr():  rows that are noisy copies of a few prototype rows, in shuffled order: the case
+                  a row reordering ahead of the SVC is for.
 """
 import collections
 
@@ -69,6 +71,27 @@ def zipf_csr(M, K, seed, mean=16, max_len=2048, s=1.5, std=1.0):
             col_ind[row_ptr[r]:row_ptr[r + 1]] = np.sort(rng.choice(K, size=n, replace=False))
     values = (rng.standard_normal(col_ind.size) * std).astype(np.float16)
     # fp16 rounding may produce exact zeros; keep the pattern meaningful for the densify round trip
+    values[values == 0] = np.float16(std)
+    return Csr(M, K, row_ptr, col_ind, values)
+
+
+def clustered_csr(M, K, prototypes, cols_per_prototype, seed, keep=0.9, extras=1, std=1.0):
+    """Row r copies prototype (r mod prototypes) before the shuffle: each of the prototype's columns
+    with probability `keep`, plus `extras` columns drawn from all K."""
+    rng = np.random.default_rng(seed)
+    protos = [np.sort(rng.choice(K, size=cols_per_prototype, replace=False)) for _ in range(prototypes)]
+    rows = []
+    for r in range(M):
+        p = protos[r % prototypes]
+        cols = p[rng.random(p.size) < keep]
+        if extras:
+            cols = np.union1d(cols, rng.choice(K, size=extras, replace=False))
+        rows.append(np.sort(cols))
+    rows = [rows[i] for i in rng.permutation(M)]
+    lens = np.array([r.size for r in rows], dtype=np.int64)
+    row_ptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    col_ind = np.concatenate(rows + [np.zeros(0, np.int64)]).astype(np.int32)
+    values = (rng.standard_normal(col_ind.size) * std).astype(np.float16)
     values[values == 0] = np.float16(std)
     return Csr(M, K, row_ptr, col_ind, values)
 

@@ -164,17 +164,17 @@ int sspmm_softmax_f16(int m_vec, int V, const int32_t *row_indices, const int32_
 }
 
 size_t svc_workspace_bytes(int M, int64_t nnz, int V) {
-  (void)M;
-  (void)V;
-  return sspmm::svc_workspace_layout(nnz, nullptr, nullptr);
+  if (M < 0 || V < 1) return 0;
+  return sspmm::svc_workspace_layout(nnz, (M + V - 1) / V, nullptr, nullptr, nullptr);
 }
 
 static int svc_args(int M, int K, int V, const int32_t *row_ptr, const int32_t *col_ind, int64_t nnz, void *workspace,
                     sspmm::SvcArgs *a) {
   if (M < 0 || K < 0 || V < 1 || V > 64 || nnz < 0 || nnz >= (1ll << 28)) return kInvalid;
   if (!row_ptr || !workspace || (nnz > 0 && !col_ind)) return kInvalid;
-  size_t off_pos, off_tables;
-  sspmm::svc_workspace_layout(nnz, &off_pos, &off_tables);
+  size_t off_pos, off_tables, off_lists;
+  const int m_vec = (M + V - 1) / V;
+  sspmm::svc_workspace_layout(nnz, m_vec, &off_pos, &off_tables, &off_lists);
   unsigned char *w = static_cast<unsigned char *>(workspace);
   a->M = M;
   a->K = K;
@@ -185,6 +185,9 @@ static int svc_args(int M, int K, int V, const int32_t *row_ptr, const int32_t *
   a->pos = reinterpret_cast<int32_t *>(w + off_pos);
   a->big_tables = reinterpret_cast<unsigned long long *>(w + off_tables);
   a->lds_table_slots = 0;
+  a->class_counts = reinterpret_cast<int32_t *>(w + off_lists);
+  a->class_lists = a->class_counts + 64;
+  a->list_stride = m_vec > 0 ? m_vec : 1;
   return 0;
 }
 
@@ -202,14 +205,15 @@ int svc_count(int M, int K, int V, const int32_t *row_ptr, const int32_t *col_in
 int svc_fill(int M, int K, int V, const int32_t *row_ptr, const int32_t *col_ind, const sspmm_half_t *csr_val,
              int64_t nnz, int order, const int32_t *vec_row_ptr, void *workspace, int32_t *vec_col,
              sspmm_half_t *vec_val, void *hip_stream) {
-  (void)order;
   sspmm::SvcArgs a{};
+  if (order != SVC_ORDER_CPYTHON && order != SVC_ORDER_SORTED) return kInvalid;
   if (!vec_row_ptr) return kInvalid;
   if (csr_val && !vec_val) return kInvalid;
   const int rc = svc_args(M, K, V, row_ptr, col_ind, nnz, workspace, &a);
   if (rc) return rc;
   if (M == 0) return 0;
-  return (int)sspmm::launch_svc_fill(a, csr_val, vec_row_ptr, vec_col, vec_val, static_cast<hipStream_t>(hip_stream));
+  return (int)sspmm::launch_svc_fill(a, order, csr_val, vec_row_ptr, vec_col, vec_val,
+                                     static_cast<hipStream_t>(hip_stream));
 }
 
 size_t svc_reorder_workspace_bytes(int M) { return sspmm::reorder_workspace_bytes(M); }

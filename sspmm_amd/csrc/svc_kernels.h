@@ -18,14 +18,26 @@ struct SvcArgs {
   int32_t *pos;                  // [nnz]   position of every non-zero's column inside its group
   unsigned long long *big_tables;  // [8*nnz] hash tables of groups too large for LDS
   int lds_table_slots;           // filled by the launcher
+  // direct mode (svc_direct): set by launch_svc_fill, null otherwise
+  const int32_t *scanned;        // the finished vec_row_ptr: group g owns vectors [scanned[g], scanned[g + 1])
+  int32_t *vec_col;              // final outputs, written by the merge kernels themselves
+  uint16_t *vec_val;
+  const uint16_t *csr_val;
+  // direct mode: the groups filed by size class (written by svc_count, read by svc_fill)
+  int32_t *class_counts;         // [5]
+  int32_t *class_lists;          // [5][list_stride]
+  int list_stride;
 };
 
-// Total workspace bytes; optional byte offsets of the pos and table views.
-size_t svc_workspace_layout(int64_t nnz, size_t *off_pos, size_t *off_tables);
+// True when svc_count only counts (bitmap pass) and svc_fill runs the merge and writes the outputs directly.
+bool svc_direct(int order, int K);
+
+// Total workspace bytes; optional byte offsets of the pos, table and class-list views.
+size_t svc_workspace_layout(int64_t nnz, int m_vec, size_t *off_pos, size_t *off_tables, size_t *off_lists);
 
 hipError_t launch_svc_count(const SvcArgs &a, int order, hipStream_t stream);
-hipError_t launch_svc_fill(const SvcArgs &a, const uint16_t *csr_val, const int32_t *vec_row_ptr, int32_t *vec_col,
-                           uint16_t *vec_val, hipStream_t stream);
+hipError_t launch_svc_fill(const SvcArgs &a, int order, const uint16_t *csr_val, const int32_t *vec_row_ptr,
+                           int32_t *vec_col, uint16_t *vec_val, hipStream_t stream);
 
 }  // namespace sspmm
 #endif

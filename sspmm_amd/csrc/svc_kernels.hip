@@ -23,9 +23,20 @@
 //
 // One workgroup owns one vector-row group.  The list and the table live in LDS (64-thread groups
 // for up to 306 keys, 256 threads up to 1228, 1024 threads up to 4914) or, beyond that, in the
-// caller's workspace.  svc_count runs the replay and leaves the ordered columns and every
-// non-zero's position in the workspace; svc_fill copies them to their final offsets and scatters
-// the values into zero-filled V-wide vectors.
+// caller's workspace.
+//
+// Which phase does what.  The caller sizes the outputs from svc_count's row pointer, so the count
+// must come first, but the count of a group (its distinct columns) needs no order: for column
+// indices of up to 17 bits svc_count is a bitmap pass plus the prefix sum, a few microseconds,
+// and svc_fill runs the replay with every group already knowing its size class exactly and its
+// final offset, so the workgroup that has ordered a group writes the group's columns and
+// zero-filled value vectors straight to their place ("direct" mode; nothing waits behind the
+// longest group but its own output).  The prefix-sum kernel also files every group under its size
+// class, so a class kernel walks a list of exactly its groups with a grid sized for the chip: the
+// largest groups start at once instead of behind thousands of workgroups that look at a group and
+// leave, and a class without groups costs an empty launch of a few workgroups.  Wider matrices and SVC_ORDER_SORTED keep the older split:
+// svc_count runs the merge and leaves the ordered columns and every non-zero's position in the
+// workspace; svc_fill copies them to their final offsets and scatters the values.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -37,6 +48,11 @@ namespace sspmm {
 
 typedef unsigned long long u64;
 static constexpr u64 kEmpty = ~0ull;
+
+// Size classes by a group's number of columns: the largest sets CPython keeps in tables of 512, 2048, 8192 and
+// 32768 slots, and everything beyond.
+static constexpr int kSmallKeys = 306, kMediumKeys = 1228, kLargeKeys = 4914, kXLargeKeys = 19660;
+static constexpr int kClasses = 5, kClassBeyond = 4;
 
 __device__ __forceinline__ void probe_start(uint32_t key, uint32_t mask, uint32_t &i, uint32_t &perturb,
                                             uint32_t &lin) {
@@ -179,15 +195,82 @@ __device__ __forceinline__ uint32_t rebuild_set(u64 *table, int *list, int &n, i
 // Class of a vector-row group by its key bound: which kernel instance handles it.
 __device__ __forceinline__ bool in_class(int bound, int lo, int hi) { return bound > lo && bound <= hi; }
 
-template <int THREADS, bool IN_LDS>
-__global__ __launch_bounds__(THREADS) void svc_merge_cpython_kernel(const SvcArgs a, int class_lo, int class_hi,
-                                                                    int list_cap) {
+// Direct mode: number of distinct columns of every group, from a K-bit occupancy bitmap in LDS.
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void svc_count_distinct_kernel(const SvcArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int grp = blockIdx.x;
   const int r0 = grp * a.V, r1 = min(a.M, r0 + a.V);
   const int e0 = a.row_ptr[r0], e1 = a.row_ptr[r1];
-  const int bound = min(e1 - e0, a.K);
-  if (!in_class(bound, class_lo, class_hi)) return;  // uniform over the group
+  if (e1 - e0 <= 1) {  // nothing to deduplicate
+    if (threadIdx.x == 0) a.vec_row_ptr[grp + 1] = e1 - e0;
+    return;
+  }
+  int *scratch = reinterpret_cast<int *>(smem);
+  uint32_t *bits = reinterpret_cast<uint32_t *>(smem + 128);
+  const int words = (a.K + 31) / 32;
+  for (int w = threadIdx.x; w < words; w += THREADS) bits[w] = 0;
+  __syncthreads();
+  // a thread counts the bits it is the first to set: no second pass over the bitmap
+  int mine = 0;
+  for (int idx = e0 + (int)threadIdx.x; idx < e1; idx += THREADS) {
+    const uint32_t c = (uint32_t)a.col_ind[idx], bit = 1u << (c & 31u);
+    mine += (atomicOr(&bits[c >> 5], bit) & bit) ? 0 : 1;
+  }
+  int total;
+  block_exclusive_scan<THREADS>(mine, &total, scratch);
+  if (threadIdx.x == 0) a.vec_row_ptr[grp + 1] = total;
+}
+
+// Direct mode: a group's ordered columns and value vectors go to their final place.  list[0 .. n) are the
+// ordered columns; position_of(column) is the column's index in that list.  The group owns
+// scanned[grp + 1] - scanned[grp] vectors; n equals that count unless a CSR row repeats a column (invalid
+// input), in which case surplus vectors stay zero with column 0.
+template <int THREADS, typename PositionOf>
+__device__ __forceinline__ void write_group_output(const SvcArgs &a, int grp, int r0, int r1, const int *list, int n,
+                                                   PositionOf position_of) {
+  const int v0 = a.scanned[grp], n_out = a.scanned[grp + 1] - v0;
+  if (a.vec_col)
+    for (int p = threadIdx.x; p < n_out; p += THREADS) a.vec_col[v0 + p] = p < n ? list[p] : 0;
+  if (!a.vec_val) return;
+  // The value region starts at v0 * V halfs and holds n_out * V of them: whole 16-byte pieces when V is a
+  // multiple of 8 (and vec_val is 16-byte aligned), 4-byte pieces whenever V is even.
+  const int64_t halfs = (int64_t)n_out * a.V;
+  uint16_t *out = a.vec_val + (int64_t)v0 * a.V;
+  if ((a.V & 7) == 0 && (reinterpret_cast<uintptr_t>(a.vec_val) & 15) == 0) {
+    uint4 *out128 = reinterpret_cast<uint4 *>(out);
+    for (int64_t t = threadIdx.x; t < halfs / 8; t += THREADS) out128[t] = uint4{0u, 0u, 0u, 0u};
+  } else if ((a.V & 1) == 0 && (reinterpret_cast<uintptr_t>(a.vec_val) & 3) == 0) {
+    uint32_t *out32 = reinterpret_cast<uint32_t *>(out);
+    for (int64_t t = threadIdx.x; t < halfs / 2; t += THREADS) out32[t] = 0u;
+  } else {
+    for (int64_t t = threadIdx.x; t < halfs; t += THREADS) out[t] = 0;
+  }
+  __syncthreads();
+  if (n == 0) return;
+  for (int r = r0; r < r1; ++r) {
+    const int b = a.row_ptr[r], e = a.row_ptr[r + 1];
+    for (int idx = b + (int)threadIdx.x; idx < e; idx += THREADS) {
+      const int p = position_of((uint32_t)a.col_ind[idx]);
+      if (p >= 0 && p < n_out) out[(int64_t)p * a.V + (r - r0)] = a.csr_val[idx];
+    }
+  }
+}
+
+template <int THREADS, bool IN_LDS>
+__global__ __launch_bounds__(THREADS) void svc_merge_cpython_kernel(const SvcArgs a, int class_lo, int class_hi,
+                                                                    int list_cap) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  // Direct mode walks the list of the groups of its class (kClassBeyond); otherwise there is one workgroup per
+  // group, which leaves unless the group's bound on its columns falls into the launch's class.
+  const bool listed = a.scanned != nullptr;
+  const int n_groups = listed ? a.class_counts[kClassBeyond] : (a.M + a.V - 1) / a.V;
+  for (int li = blockIdx.x; li < n_groups; li += gridDim.x) {
+  const int grp = listed ? a.class_lists[(int64_t)kClassBeyond * a.list_stride + li] : li;
+  const int r0 = grp * a.V, r1 = min(a.M, r0 + a.V);
+  const int e0 = a.row_ptr[r0], e1 = a.row_ptr[r1];
+  const int bound = listed ? a.scanned[grp + 1] - a.scanned[grp] : min(e1 - e0, a.K);
+  if (!listed && !in_class(bound, class_lo, class_hi)) continue;  // uniform over the group
 
   int *scratch = reinterpret_cast<int *>(smem);  // 32 ints
   int *list;
@@ -196,7 +279,7 @@ __global__ __launch_bounds__(THREADS) void svc_merge_cpython_kernel(const SvcArg
     table = reinterpret_cast<u64 *>(smem + 128);
     list = reinterpret_cast<int *>(smem + 128 + (size_t)a.lds_table_slots * 8);
   } else {
-    list_cap = e1 - e0;
+    list_cap = listed ? bound : e1 - e0;
     list = a.tmp_cols + e0;
     table = a.big_tables + (int64_t)e0 * 8;
   }
@@ -225,6 +308,14 @@ __global__ __launch_bounds__(THREADS) void svc_merge_cpython_kernel(const SvcArg
     slots = rebuild_set<THREADS>(table, list, n, scratch);
   }
 
+  if (listed) {
+    write_group_output<THREADS>(a, grp, r0, r1, list, n, [&](uint32_t key) {
+      const int s = find_slot(table, slots - 1u, key);
+      return s >= 0 ? (int)(table[s] >> 32) : -1;
+    });
+    __syncthreads();  // the next group reuses the table
+    continue;
+  }
   if (threadIdx.x == 0) a.vec_row_ptr[grp + 1] = n;
   if (IN_LDS)
     for (int p = threadIdx.x; p < n; p += THREADS) a.tmp_cols[e0 + p] = list[p];
@@ -233,6 +324,7 @@ __global__ __launch_bounds__(THREADS) void svc_merge_cpython_kernel(const SvcArg
       const int s = find_slot(table, slots - 1u, (uint32_t)a.col_ind[idx]);
       a.pos[idx] = s >= 0 ? (int)(table[s] >> 32) : 0;  // s < 0 only for invalid (capped) input
     }
+  }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -247,7 +339,6 @@ __global__ __launch_bounds__(THREADS) void svc_merge_cpython_kernel(const SvcArg
 // population of every word, wave 0 turns them into running counts, and a second pass writes
 // list[count[word] + rank in word] = key, so nothing is scanned per thread.
 static constexpr uint32_t kEmpty32 = 0xffffffffu;
-static constexpr int kGaveUp = -1;  // vec_row_ptr entry of a group whose launch found it too large
 
 struct Table32 {
   uint32_t *slots;  // LDS
@@ -484,18 +575,21 @@ __device__ __forceinline__ uint32_t rebuild_set32(Table32 &t, const TableRegions
 }
 
 template <int THREADS, bool LIST_IN_LDS>
-__global__ __launch_bounds__(THREADS) void svc_merge_fast_kernel(const SvcArgs a, int class_lo, int class_hi,
-                                                                 uint32_t key_bits, uint32_t max_slots, uint32_t small_slots,
-                                                                 int only_flagged) {
+__global__ __launch_bounds__(THREADS) void svc_merge_fast_kernel(const SvcArgs a, int cls, int cls_last,
+                                                                 uint32_t key_bits, uint32_t max_slots, uint32_t small_slots) {
   extern __shared__ __align__(16) unsigned char smem[];
-  const int grp = blockIdx.x;
-  const int r0 = grp * a.V, r1 = min(a.M, r0 + a.V);
-  const int e0 = a.row_ptr[r0], e1 = a.row_ptr[r1];
-  const int bound = min(e1 - e0, a.K);
-  if (!in_class(bound, class_lo, class_hi)) return;  // uniform over the group
-  // second chance for a group that an earlier launch on this stream gave up on (see kGaveUp)
-  if (only_flagged && a.vec_row_ptr[grp + 1] != kGaveUp) return;
+  // direct mode only: the groups of this launch's classes are listed, and a group's column count is known.
+  // A launch takes the classes cls, cls - 1, ..., cls_last (largest groups first).
   const int tid = threadIdx.x;
+  int n_groups = 0;
+  for (int c = cls; c >= cls_last; --c) n_groups += a.class_counts[c];
+  for (int li = blockIdx.x; li < n_groups; li += gridDim.x) {
+  int c = cls, at = li;
+  while (at >= a.class_counts[c]) at -= a.class_counts[c--];
+  const int grp = a.class_lists[(int64_t)c * a.list_stride + at];
+  const int r0 = grp * a.V, r1 = min(a.M, r0 + a.V);
+  const int count = a.scanned[grp + 1] - a.scanned[grp];
+  const int e0 = a.row_ptr[r0];
 
   int *scratch = reinterpret_cast<int *>(smem);  // 32 ints
   Table32 t;
@@ -508,7 +602,7 @@ __global__ __launch_bounds__(THREADS) void svc_merge_fast_kernel(const SvcArgs a
   reg.b = t.slots + max_slots;
   reg.cap_b = small_slots;
   int *list = LIST_IN_LDS ? reinterpret_cast<int *>(smem + 128 + ((size_t)max_slots + small_slots) * 4) : a.tmp_cols + e0;
-  const int cap = LIST_IN_LDS ? min(class_hi, bound) : bound;
+  const int cap = count;
 
   int n = 0;
   uint32_t slots = 0;
@@ -529,25 +623,17 @@ __global__ __launch_bounds__(THREADS) void svc_merge_fast_kernel(const SvcArgs a
       if (is_new && n + appended + rank < cap) list_store<LIST_IN_LDS>(list, n + appended + rank, (int)k);
       appended += total;
     }
-    n = min(n + appended, cap);  // the cap only bites for invalid input (repeated columns)
+    n = min(n + appended, cap);  // the cap only bites for invalid input (a row that repeats a column)
     __syncthreads();
-    if ((uint32_t)n >= resize_threshold(max_slots)) {
-      // more distinct columns than this launch's tables take: only a group admitted on the strength of its
-      // distinct columns being fewer than its non-zeros gets here; it is left to the launch that follows
-      if (tid == 0) a.vec_row_ptr[grp + 1] = kGaveUp;
-      return;
-    }
     slots = rebuild_set32<THREADS, LIST_IN_LDS>(t, reg, list, n);
   }
 
-  if (tid == 0) a.vec_row_ptr[grp + 1] = n;
-  if (LIST_IN_LDS)
-    for (int p = tid; p < n; p += THREADS) a.tmp_cols[e0 + p] = list[p];
-  if (n > 0)
-    for (int idx = e0 + tid; idx < e1; idx += THREADS) {
-      const int sl = find_slot32(t, slots - 1u, (uint32_t)a.col_ind[idx]);
-      a.pos[idx] = sl >= 0 ? (int)(t.slots[sl] >> key_bits) : 0;  // sl < 0 only for invalid (capped) input
-    }
+  write_group_output<THREADS>(a, grp, r0, r1, list, n, [&](uint32_t key) {
+    const int sl = find_slot32(t, slots - 1u, key);
+    return sl >= 0 ? (int)(t.slots[sl] >> key_bits) : -1;
+  });
+  __syncthreads();  // the next group reuses the table and the list
+  }
 }
 
 // Ascending order: a K-bit occupancy bitmap per group plus a per-word running popcount.
@@ -589,6 +675,38 @@ __global__ __launch_bounds__(THREADS) void svc_merge_sorted_kernel(const SvcArgs
     const uint32_t c = (uint32_t)a.col_ind[idx];
     a.pos[idx] = prefix[c >> 5] + __popc(bits[c >> 5] & ((1u << (c & 31u)) - 1u));
   }
+}
+
+// Direct mode: the scan above, and every group filed under its size class.  class_lists[c * stride + i] is the
+// i-th group of class c (in no particular order), class_counts[c] how many there are.
+__global__ __launch_bounds__(1024) void svc_scan_classify_kernel(int m_vec, int32_t *vec_row_ptr, int32_t *class_lists,
+                                                                 int32_t *class_counts, int list_stride) {
+  __shared__ int scratch[32];
+  __shared__ int filed[kClasses];
+  if (threadIdx.x < kClasses) filed[threadIdx.x] = 0;
+  if (threadIdx.x == 0) vec_row_ptr[0] = 0;
+  int carry = 0;
+  const int lane = threadIdx.x & 63;
+  for (int base = 0; base < m_vec; base += 1024) {
+    const int i = base + (int)threadIdx.x;
+    const int x = i < m_vec ? vec_row_ptr[i + 1] : 0;
+    int total;
+    const int ex = block_exclusive_scan<1024>(x, &total, scratch);  // (its barriers also cover filed[]'s set-up)
+    if (i < m_vec) vec_row_ptr[i + 1] = carry + ex + x;
+    carry += total;
+    const int cls = i >= m_vec ? -1 : x <= kSmallKeys ? 0 : x <= kMediumKeys ? 1 : x <= kLargeKeys ? 2 : x <= kXLargeKeys ? 3 : 4;
+#pragma unroll
+    for (int c = 0; c < kClasses; ++c) {
+      const unsigned long long members = __ballot(cls == c);
+      if (members == 0) continue;  // uniform over the wave
+      int at = 0;
+      if (lane == 0) at = atomicAdd(&filed[c], __popcll(members));
+      at = __shfl(at, 0, 64);
+      if (cls == c) class_lists[(int64_t)c * list_stride + at + __popcll(members & ((1ull << lane) - 1ull))] = i;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < kClasses) class_counts[threadIdx.x] = filed[threadIdx.x];
 }
 
 // In-place inclusive scan of vec_row_ptr[1..m_vec], vec_row_ptr[0] = 0.  One workgroup walks the
@@ -644,17 +762,17 @@ __global__ __launch_bounds__(THREADS) void svc_fill_kernel(const SvcArgs a, cons
 
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
-size_t svc_workspace_layout(int64_t nnz, size_t *off_pos, size_t *off_tables) {
+size_t svc_workspace_layout(int64_t nnz, int m_vec, size_t *off_pos, size_t *off_tables, size_t *off_lists) {
   const size_t n = (size_t)(nnz > 0 ? nnz : 1);
   const size_t cols = align256(n * 4);
   const size_t pos = align256(n * 4);
   const size_t tables = align256(n * 64);
+  const size_t lists = align256(((size_t)kClasses * (size_t)(m_vec > 0 ? m_vec : 1) + 64) * 4);  // counts, then lists
   if (off_pos) *off_pos = cols;
   if (off_tables) *off_tables = cols + pos;
-  return cols + pos + tables;
+  if (off_lists) *off_lists = cols + pos + tables;
+  return cols + pos + tables + lists;
 }
-
-static constexpr int kSmallKeys = 306, kMediumKeys = 1228, kLargeKeys = 4914, kHopefulKeys = 7600, kXLargeKeys = 19660;
 
 template <int THREADS>
 static hipError_t launch_lds_class(const SvcArgs &base, int m_vec, int lo, int hi, int slots, hipStream_t stream) {
@@ -672,21 +790,22 @@ static hipError_t launch_lds_class(const SvcArgs &base, int m_vec, int lo, int h
 }
 
 template <int THREADS, bool LIST_IN_LDS>
-static hipError_t launch_fast_class(const SvcArgs &a, int m_vec, int lo, int hi, uint32_t slots, uint32_t key_bits,
-                                    hipStream_t stream, int only_flagged = 0) {
+static hipError_t launch_fast_class(const SvcArgs &a, int grid, int cls, int cls_last, int hi, uint32_t slots,
+                                    uint32_t key_bits, hipStream_t stream, size_t min_lds = 0) {
   // second table region: a quarter of the first (what the phase before the largest needs), less where LDS is short;
   // it also serves as the running-count array of the compaction of a table in the first region (slots / 64 + 1 words)
   uint32_t small_slots = slots / 4u;
   while (128 + ((size_t)slots + small_slots) * 4 + (LIST_IN_LDS ? (size_t)hi * 4 : 0) > 160 * 1024) small_slots /= 4u;
   if (small_slots < slots / 64u + 1u) return hipErrorInvalidValue;
-  const size_t lds = 128 + ((size_t)slots + small_slots) * 4 + (LIST_IN_LDS ? (size_t)hi * 4 : 0);
+  size_t lds = 128 + ((size_t)slots + small_slots) * 4 + (LIST_IN_LDS ? (size_t)hi * 4 : 0);
+  if (lds < min_lds) lds = min_lds;  // asking for more than half of a CU's LDS keeps a workgroup alone on its CU
   auto kern = svc_merge_fast_kernel<THREADS, LIST_IN_LDS>;
   if (lds > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return e;
   }
-  hipLaunchKernelGGL(kern, dim3(m_vec), dim3(THREADS), lds, stream, a, lo, hi, key_bits, slots, small_slots, only_flagged);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(THREADS), lds, stream, a, cls, cls_last, key_bits, slots, small_slots);
   return hipGetLastError();
 }
 
@@ -717,55 +836,57 @@ static SideStreams *side_streams() {
   return &ss;
 }
 
+static uint32_t bits_of(int K) {
+  uint32_t key_bits = 1;
+  while (key_bits < 31 && (1u << key_bits) < (uint32_t)K) ++key_bits;
+  return key_bits;
+}
+
+bool svc_direct(int order, int K) { return order == 0 && bits_of(K) <= 17; }
+
+// Forks the helper streams from `stream`; st[0] is the caller's stream.
+static hipError_t fork_streams(SideStreams *ss, hipStream_t stream, hipStream_t (&st)[4], int helpers = 3) {
+  for (int i = 0; i < 4; ++i) st[i] = stream;
+  if (!ss) return hipSuccess;
+  hipError_t e = hipEventRecord(ss->fork, stream);
+  if (e != hipSuccess) return e;
+  for (int i = 0; i < helpers; ++i) {
+    if ((e = hipStreamWaitEvent(ss->s[i], ss->fork, 0)) != hipSuccess) return e;
+    st[i + 1] = ss->s[i];
+  }
+  return hipSuccess;
+}
+
+static hipError_t join_streams(SideStreams *ss, hipStream_t stream, int helpers = 3) {
+  if (!ss) return hipSuccess;
+  for (int i = 0; i < helpers; ++i) {
+    hipError_t e = hipEventRecord(ss->join[i], ss->s[i]);
+    if (e != hipSuccess) return e;
+    if ((e = hipStreamWaitEvent(stream, ss->join[i], 0)) != hipSuccess) return e;
+  }
+  return hipSuccess;
+}
+
 hipError_t launch_svc_count(const SvcArgs &a, int order, hipStream_t stream) {
   const int m_vec = (a.M + a.V - 1) / a.V;
   hipError_t e;
-  if (order == 0) {
+  if (svc_direct(order, a.K)) {
+    const size_t lds = 128 + (size_t)((a.K + 31) / 32) * 4;  // at most 16 KB
+    hipLaunchKernelGGL((svc_count_distinct_kernel<256>), dim3(m_vec), dim3(256), lds, stream, a);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+  } else if (order == 0) {
     // One pass over the groups per size class, each taking the groups of its class; a group's class
     // is decided from min(non-zeros of the group, K), an upper bound of its distinct columns.
-    uint32_t key_bits = 1;
-    while (key_bits < 31 && (1u << key_bits) < (uint32_t)a.K) ++key_bits;
     SideStreams *ss = side_streams();
-    hipStream_t st[4] = {stream, stream, stream, stream};
-    if (ss) {
-      if ((e = hipEventRecord(ss->fork, stream)) != hipSuccess) return e;
-      for (int i = 0; i < 3; ++i) {
-        if ((e = hipStreamWaitEvent(ss->s[i], ss->fork, 0)) != hipSuccess) return e;
-        st[i + 1] = ss->s[i];
-      }
-    }
-    int top = kLargeKeys;
-    if (key_bits <= 17) {
-      // 32-bit table entries: 15 bits of insertion index are enough up to 19 660 keys
-      // The classes of the largest groups go out first, the 8192-slot class on the caller's stream: a single
-      // group of thousands of keys takes longer than all the small groups together.
-      // A group's class is decided from its non-zeros, an upper bound of its distinct columns.  Groups a little
-      // above the limit of the 8192-slot class are tried there all the same (a merged group of long rows repeats
-      // many columns); one that does outgrow the table marks itself and is redone by the launch behind it.
-      if ((e = launch_fast_class<1024, true>(a, m_vec, kMediumKeys, kHopefulKeys, 8192, key_bits, st[0])) != hipSuccess)
-        return e;
-      if ((e = launch_fast_class<1024, false>(a, m_vec, kLargeKeys, kHopefulKeys, 32768, key_bits, st[0], 1)) != hipSuccess)
-        return e;
-      if ((e = launch_fast_class<1024, false>(a, m_vec, kHopefulKeys, kXLargeKeys, 32768, key_bits, st[1])) != hipSuccess)
-        return e;
-      if ((e = launch_fast_class<256, true>(a, m_vec, kSmallKeys, kMediumKeys, 2048, key_bits, st[2])) != hipSuccess)
-        return e;
-      if ((e = launch_fast_class<64, true>(a, m_vec, -1, kSmallKeys, 512, key_bits, st[3])) != hipSuccess) return e;
-      top = kXLargeKeys;
-    } else {
-      if ((e = launch_lds_class<64>(a, m_vec, -1, kSmallKeys, 512, st[0])) != hipSuccess) return e;
-      if ((e = launch_lds_class<256>(a, m_vec, kSmallKeys, kMediumKeys, 2048, st[1])) != hipSuccess) return e;
-      if ((e = launch_lds_class<1024>(a, m_vec, kMediumKeys, kLargeKeys, 8192, st[2])) != hipSuccess) return e;
-    }
-    hipLaunchKernelGGL((svc_merge_cpython_kernel<1024, false>), dim3(m_vec), dim3(1024), 128,
-                       key_bits <= 17 ? st[1] : st[3], a, top, 0x7fffffff, 0);
+    hipStream_t st[4];
+    if ((e = fork_streams(ss, stream, st)) != hipSuccess) return e;
+    if ((e = launch_lds_class<64>(a, m_vec, -1, kSmallKeys, 512, st[0])) != hipSuccess) return e;
+    if ((e = launch_lds_class<256>(a, m_vec, kSmallKeys, kMediumKeys, 2048, st[1])) != hipSuccess) return e;
+    if ((e = launch_lds_class<1024>(a, m_vec, kMediumKeys, kLargeKeys, 8192, st[2])) != hipSuccess) return e;
+    hipLaunchKernelGGL((svc_merge_cpython_kernel<1024, false>), dim3(m_vec), dim3(1024), 128, st[3], a, kLargeKeys,
+                       0x7fffffff, 0);
     if ((e = hipGetLastError()) != hipSuccess) return e;
-    if (ss) {
-      for (int i = 0; i < 3; ++i) {
-        if ((e = hipEventRecord(ss->join[i], ss->s[i])) != hipSuccess) return e;
-        if ((e = hipStreamWaitEvent(stream, ss->join[i], 0)) != hipSuccess) return e;
-      }
-    }
+    if ((e = join_streams(ss, stream)) != hipSuccess) return e;
   } else {
     const int words = (a.K + 31) / 32;
     const size_t lds = 128 + (size_t)words * 8;
@@ -779,16 +900,55 @@ hipError_t launch_svc_count(const SvcArgs &a, int order, hipStream_t stream) {
     hipLaunchKernelGGL(kern, dim3(m_vec), dim3(256), lds, stream, a);
     if ((e = hipGetLastError()) != hipSuccess) return e;
   }
-  hipLaunchKernelGGL(svc_scan_kernel, dim3(1), dim3(1024), 0, stream, m_vec, a.vec_row_ptr);
+  if (svc_direct(order, a.K))
+    hipLaunchKernelGGL(svc_scan_classify_kernel, dim3(1), dim3(1024), 0, stream, m_vec, a.vec_row_ptr, a.class_lists,
+                       a.class_counts, a.list_stride);
+  else
+    hipLaunchKernelGGL(svc_scan_kernel, dim3(1), dim3(1024), 0, stream, m_vec, a.vec_row_ptr);
   return hipGetLastError();
 }
 
-hipError_t launch_svc_fill(const SvcArgs &a, const uint16_t *csr_val, const int32_t *vec_row_ptr, int32_t *vec_col,
-                           uint16_t *vec_val, hipStream_t stream) {
-  const int m_vec = (a.M + a.V - 1) / a.V;
-  hipLaunchKernelGGL((svc_fill_kernel<512>), dim3(m_vec), dim3(512), 0, stream, a, csr_val, vec_row_ptr, vec_col,
-                     csr_val ? vec_val : nullptr);
-  return hipGetLastError();
+hipError_t launch_svc_fill(const SvcArgs &args, int order, const uint16_t *csr_val, const int32_t *vec_row_ptr,
+                           int32_t *vec_col, uint16_t *vec_val, hipStream_t stream) {
+  const int m_vec = (args.M + args.V - 1) / args.V;
+  if (!svc_direct(order, args.K)) {
+    hipLaunchKernelGGL((svc_fill_kernel<512>), dim3(m_vec), dim3(512), 0, stream, args, csr_val, vec_row_ptr, vec_col,
+                       csr_val ? vec_val : nullptr);
+    return hipGetLastError();
+  }
+  // Direct mode: the merge itself, one launch per size class over the groups of that class (known exactly from
+  // the row pointer), every group writing its own output.  The classes are independent kernels over disjoint
+  // groups; the class of the largest groups goes out first, on the caller's stream: a single group of
+  // thousands of columns takes longer than all the small groups together.
+  SvcArgs a = args;
+  a.scanned = vec_row_ptr;
+  a.vec_col = vec_col;
+  a.vec_val = csr_val ? vec_val : nullptr;
+  a.csr_val = csr_val;
+  const uint32_t key_bits = bits_of(a.K);
+  hipError_t e;
+  SideStreams *ss = side_streams();
+  hipStream_t st[4];
+  if ((e = fork_streams(ss, stream, st, 1)) != hipSuccess) return e;
+  // Grids: what the chip holds at once for the class's workgroup size and LDS, at most one workgroup per group.
+  // The two classes of 1229 .. 4914 and 307 .. 1228 columns share a launch on the caller's stream (1024 threads
+  // and 8192-slot tables for both): with one such workgroup per CU resident every group (up to the number of CUs) of either
+  // class starts at once, and nothing that could outlast the largest group waits on a helper stream to begin.
+  // These workgroups are chains of LDS round trips: each gets a CU to itself (by asking for more than half its LDS).
+  // The many small groups, and the two classes that are nearly always empty, follow each other on one helper
+  // stream: one fork and one join.
+  const int cus = 256;
+  if ((e = launch_fast_class<1024, true>(a, min(m_vec, cus), 2, 1, kLargeKeys, 8192, key_bits, st[0], 81 * 1024)) !=
+      hipSuccess)
+    return e;
+  if ((e = launch_fast_class<64, true>(a, min(m_vec, 32 * cus), 0, 0, kSmallKeys, 512, key_bits, st[1])) != hipSuccess)
+    return e;
+  if ((e = launch_fast_class<1024, false>(a, min(m_vec, cus), 3, 3, kXLargeKeys, 32768, key_bits, st[1])) != hipSuccess)
+    return e;
+  // more columns than a 32768-slot table takes: 64-bit entries in the workspace
+  hipLaunchKernelGGL((svc_merge_cpython_kernel<1024, false>), dim3(min(m_vec, cus)), dim3(1024), 128, st[1], a, 0, 0, 0);
+  if ((e = hipGetLastError()) != hipSuccess) return e;
+  return join_streams(ss, stream, 1);
 }
 
 }  // namespace sspmm

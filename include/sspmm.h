@@ -135,8 +135,11 @@ int sspmm_softmax_batched_f16(int batch, int m_vec, int V, const int32_t *row_in
  *   1. svc_count  writes vec_row_ptr[m_vec+1]; nvec = vec_row_ptr[m_vec] (read it back, or
  *                 skip the read and size the outputs for the bound nvec <= nnz).
  *   2. svc_fill   writes vec_col[nvec] and, when csr_val != NULL, vec_val[nvec*V] (zero filled).
- * Both phases take the same workspace of svc_workspace_bytes(M, nnz, V) bytes; svc_fill
- * consumes what svc_count left there.
+ * Both phases take the same workspace of svc_workspace_bytes(M, nnz, V) bytes and the same
+ * `order`; svc_fill consumes what svc_count left in the workspace.  How the work is split
+ * between the two is internal: for SVC_ORDER_CPYTHON with K <= 131072 svc_count only counts
+ * each group's distinct columns (a few microseconds) and svc_fill runs the merge, every group
+ * writing its output in place; otherwise svc_count runs the merge and svc_fill copies.
  *
  * order: SVC_ORDER_CPYTHON reproduces the column order of the reference's output files (the
  * iteration order of CPython's set in `list(set(acc + row))`), bit for bit;

@@ -93,9 +93,9 @@ def test_every_group_size_class(oracle, built_library, keys):
 
 
 @pytest.mark.parametrize("distinct", [3000, 4914, 4915, 5600])
-def test_groups_admitted_on_the_hope_of_repeated_columns(oracle, built_library, distinct):
-    """A group with 6400 non-zeros is tried in the class that takes up to 4914 distinct columns; whether it
-    finishes there (its rows repeat columns) or has to be redone by the next launch, the result is the same."""
+def test_a_groups_class_comes_from_its_distinct_columns(oracle, built_library, distinct):
+    """A group with 6400 non-zeros and 3000 .. 5600 distinct columns (its rows repeat columns of one another):
+    the table it is merged in is chosen from the distinct count, either side of the 4914-column class limit."""
     rng = np.random.default_rng(distinct)
     V, K, per_row = 8, 16384, 800
     pool = rng.permutation(K)[:distinct]
@@ -112,6 +112,37 @@ def test_groups_admitted_on_the_hope_of_repeated_columns(oracle, built_library, 
     csr = synth.Csr(24, K, ptr, cols, rng.standard_normal(cols.size).astype(np.float16))
     vrp, _, _ = _compare_with_oracle(oracle, csr, V)
     assert vrp[2] - vrp[1] == distinct
+
+
+def test_more_groups_of_a_class_than_workgroups_in_its_launch(oracle, built_library):
+    """V = 1 makes every row a group: 9000 short rows (the launch of the smallest class has 8192 workgroups),
+    and 300 + 260 + 270 rows of 1300, 400 and 5000 columns (one workgroup per CU for those classes), so that
+    workgroups walk on to a second group and reuse their tables."""
+    rng = np.random.default_rng(77)
+    K = 16384
+    lens = np.concatenate([rng.integers(0, 20, 9000), np.full(300, 1300), np.full(260, 400), np.full(270, 5000)])
+    rng.shuffle(lens)
+    ptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cols = np.concatenate([np.sort(rng.choice(K, n, replace=False)) for n in lens]).astype(np.int32)
+    csr = synth.Csr(lens.size, K, ptr, cols, rng.standard_normal(cols.size).astype(np.float16))
+    _compare_with_oracle(oracle, csr, 1)
+
+
+def test_a_row_that_repeats_a_column_stays_inside_its_group(built_library):
+    """Invalid input (the contract forbids repeated columns in a row): the column order is then unspecified,
+    but the counts are the distinct columns and every write stays inside the group's own vectors."""
+    rng = np.random.default_rng(78)
+    K, V = 4096, 8
+    rows = [np.concatenate([c, c[: len(c) // 2]]) for c in (rng.choice(K, n, replace=False) for n in [5, 300, 0, 1500, 40, 2, 9, 700] * 3)]
+    lens = np.array([len(r) for r in rows])
+    ptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cols = np.concatenate(rows).astype(np.int32)
+    vals = np.ones(cols.size, np.float16)
+    vrp, vcol, vval, nvec = gpu_svc(len(rows), K, V, ptr, cols, vals)
+    want = [np.unique(cols[ptr[g]:ptr[min(len(rows), g + V)]]).size for g in range(0, len(rows), V)]
+    assert np.array_equal(np.diff(vrp), want)
+    assert vcol.size == nvec and vval.size == nvec * V
+    assert ((vcol >= 0) & (vcol < K)).all() and np.isin(vval, [0.0, 1.0]).all()
 
 
 def test_cfg1_rowmerge_returns_the_vector_pattern(oracle, built_library):

@@ -131,11 +131,25 @@ def main():
         del src, dst
 
     M, K, V, sparsity, N = 2048, 512, 8, 0.9, 256
-    kernel_names = {1: "spmm_generic_kernel<8,float>", 2: "spmm_gather_kernel<8,float>", 3: "spmm_slab_kernel<8,float,true>"}
+    kernel_names = {1: "spmm_generic_kernel<8,float>", 2: "spmm_gather_kernel<8,float>", 3: "spmm_slab_kernel<8,float,true>",
+                    4: "spmm_gather_split_kernel<8,float>"}
     main_res, (vs, vals, B, C) = spmm_case(L, torch, synth, M, K, V, sparsity, N, args.batch, True, 0.02, 2,
                                            args.steps, args.warmup, dense=not args.quick)
     torch.cuda.synchronize()
     main_kernel = kernel_names.get(L.sspmm_last_kernel(), "unknown")
+
+    # what this box's memory system sustains for plain streams of the same size class, measured the same way
+    # (50 launches after warm-up): a device copy (half reads, half writes) and a fill (writes only)
+    ceilings = None
+    if not args.quick:
+        src = torch.ones(256 * 1024 * 1024, dtype=torch.float32, device="cuda")  # 1 GiB: beyond the memory-side cache
+        dst = torch.empty_like(src)
+        copy_ms = time_launches(lambda: dst.copy_(src), 50, 5)
+        fill_ms = time_launches(lambda: dst.fill_(1.0), 50, 5)
+        ceilings = {"device_copy_1GiB_gbps": 2 * src.numel() * 4 / copy_ms / 1e6,
+                    "device_fill_1GiB_gbps": src.numel() * 4 / fill_ms / 1e6}
+        ceilings["frac_of_device_copy"] = main_res["hbm_gbps"] / ceilings["device_copy_1GiB_gbps"]
+        del src, dst
 
     # parity of batch element 0 against the CPU oracle, and the CPU baseline on the same element
     cpu = None
@@ -354,7 +368,8 @@ def main():
         "roofline": {"bound": "hbm", "achieved": main_res["hbm_gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": main_res["hbm_frac"],
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.batch) if args.kernel == "auto" else None,
-                     "kernel": main_kernel, "alg_bytes_per_launch": main_res["alg_bytes"]},
+                     "kernel": main_kernel, "alg_bytes_per_launch": main_res["alg_bytes"],
+                     "measured_stream_rates": ceilings},
         "cpu_baseline": cpu,
         "parity_max_rel_err": parity,
         "dense_gemm": {k: main_res[k] for k in main_res if k.startswith("dense") or k.startswith("speedup")},

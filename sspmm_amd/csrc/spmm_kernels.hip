@@ -222,6 +222,154 @@ __global__ __launch_bounds__(64) void spmm_gather_kernel(const SpmmArgs p) {
 }
 
 // ------------------------------------------------------------------------------------------
+// Gather kernel for wide matrices (K above kSplitMinK), where a vector-row may hold thousands of
+// vectors: the merged rows of an unstructured matrix with power-law row lengths do, and one wave
+// per vector-row would keep a few waves busy long after the rest of the grid has drained.
+//
+// A workgroup of kSplitWaves waves owns as many consecutive vector-rows of one 128-column tile.
+// Each wave computes and stores its own row as the kernel above does, unless the row has more
+// than kLongRowSteps steps.  Such a row is left for a second phase in which all waves of the
+// group take a contiguous share of its steps and add their partial tiles up in LDS in wave order,
+// so the result does not depend on timing.  Every wave reads the extents of all rows of its group,
+// so a group without a long row never meets at a barrier.
+static constexpr int kSplitWaves = 4;
+static constexpr int kLongRowSteps = 16;
+static constexpr int kSplitMinK = 4096;
+
+// The partial V x 128 tile of vectors [beg, sub_end) of a vector-row that ends at `end`.
+template <int V>
+__device__ __forceinline__ void gather_accumulate(floatx4 (&acc)[8], const SpmmArgs &p, uint32_t batch, int beg,
+                                                  int sub_end, int end, int lane, int ncol, bool col_ok) {
+  const int m = lane & 15, g = lane >> 4;
+  const uint16_t *vals = p.values + (int64_t)batch * p.stride_values;
+  const uint16_t *bmat = p.B + (int64_t)batch * p.stride_B;
+  const uint32_t b_bytes = (uint32_t)p.K * (uint32_t)p.N * 2u;
+  const __amdgpu_buffer_rsrc_t srd_cols = make_srd(p.col_idx, (uint32_t)end * 4u);
+  const __amdgpu_buffer_rsrc_t srd_vals = make_srd(vals, (uint32_t)end * (V * 2u));
+  const __amdgpu_buffer_rsrc_t srd_b = make_srd(bmat, b_bytes);
+  const uint32_t lane_n2 = col_ok ? (uint32_t)p.N * 2u : 0u;
+  const uint32_t lane_col_off = col_ok ? (uint32_t)ncol * 2u : b_bytes;
+  const uint32_t vals_lane_off = (uint32_t)m * 2u;
+#pragma unroll
+  for (int q = 0; q < 8; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
+  if (beg >= sub_end) return;
+  ChunkHead h0, h1;
+  Chunk c0, c1;
+  load_head<V>(h0, beg, g, srd_cols, srd_vals, vals_lane_off);
+  load_head<V>(h1, beg + 32, g, srd_cols, srd_vals, vals_lane_off);
+  load_body(c0, h0, end, g, srd_b, lane_n2, lane_col_off, b_bytes);
+  int kc = beg + 32;  // first vector of the chunk whose body is loaded next
+  for (;;) {
+    if (kc >= sub_end) {
+      mac_chunk(c0, acc);
+      break;
+    }
+    load_head<V>(h0, kc + 32, g, srd_cols, srd_vals, vals_lane_off);
+    load_body(c1, h1, end, g, srd_b, lane_n2, lane_col_off, b_bytes);
+    mac_chunk(c0, acc);
+    kc += 32;
+    if (kc >= sub_end) {
+      mac_chunk(c1, acc);
+      break;
+    }
+    load_head<V>(h1, kc + 32, g, srd_cols, srd_vals, vals_lane_off);
+    load_body(c0, h0, end, g, srd_b, lane_n2, lane_col_off, b_bytes);
+    mac_chunk(c1, acc);
+    kc += 32;
+  }
+}
+
+template <int V, typename OutT>
+__global__ __launch_bounds__(64 * kSplitWaves) void spmm_gather_split_kernel(const SpmmArgs p) {
+  __shared__ floatx4 part[4][2][64];  // the tile being added up: part[rr][half][lane] = acc[4 * half .. + 3][rr]
+  const uint32_t id = blockIdx.x;
+  const uint32_t w = (id & 7u) * p.per_xcd + (id >> 3);
+  if (w >= p.total_work) return;
+  const uint32_t n_groups = ((uint32_t)p.m_vec + kSplitWaves - 1u) / kSplitWaves;
+  const uint32_t grp = w % n_groups;
+  const uint32_t t = w / n_groups;
+  const uint32_t tile = t % p.n_tiles;
+  const uint32_t batch = t / p.n_tiles;
+
+  const int lane = threadIdx.x & 63, m = lane & 15, g = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  // the rows of the group and their extents (the same in every wave)
+  int g_row[kSplitWaves], g_beg[kSplitWaves], g_end[kSplitWaves];
+  bool any_long = false;
+#pragma unroll
+  for (int j = 0; j < kSplitWaves; ++j) {
+    const int rj = (int)grp * kSplitWaves + j;
+    const bool have = rj < p.m_vec;
+    g_row[j] = have ? (p.row_indices ? p.row_indices[rj] : rj) : -1;
+    g_beg[j] = have ? p.row_offsets[g_row[j]] : 0;
+    g_end[j] = have ? p.row_offsets[g_row[j] + 1] : 0;
+    any_long = any_long || (g_end[j] - g_beg[j] > 32 * kLongRowSteps);
+  }
+  int row = -1, beg = 0, end = 0;
+#pragma unroll
+  for (int j = 0; j < kSplitWaves; ++j)
+    if (j == wave) {
+      row = g_row[j];
+      beg = g_beg[j];
+      end = g_end[j];
+    }
+  const bool is_long = end - beg > 32 * kLongRowSteps;
+  const int ncol = (int)tile * 128 + m * 8;
+  const bool col_ok = ncol < p.N;
+  OutT *cbase = reinterpret_cast<OutT *>(p.C) + (int64_t)batch * p.stride_C;
+
+  floatx4 acc[8];
+  if (row >= 0 && !is_long) {
+    gather_accumulate<V>(acc, p, batch, beg, end, end, lane, ncol, col_ok);
+    if (col_ok) {
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        const int v = 4 * g + rr;
+        if (v < V) {
+          float o[8];
+#pragma unroll
+          for (int q = 0; q < 8; ++q) o[q] = acc[q][rr];
+          Store8<OutT>::run(cbase + ((int64_t)row * V + v) * p.N + ncol, o);
+        }
+      }
+    }
+  }
+  if (!any_long) return;  // uniform over the workgroup
+#pragma unroll
+  for (int j = 0; j < kSplitWaves; ++j) {
+    const int lrow = g_row[j], lbeg = g_beg[j], lend = g_end[j];
+    if (lend - lbeg <= 32 * kLongRowSteps) continue;  // uniform over the workgroup
+    const int steps = (lend - lbeg + 31) >> 5;
+    const int per = (steps + kSplitWaves - 1) / kSplitWaves;
+    const int my_beg = min(lend, lbeg + wave * per * 32);
+    const int my_end = min(lend, my_beg + per * 32);
+    gather_accumulate<V>(acc, p, batch, my_beg, my_end, lend, lane, ncol, col_ok);
+    for (int turn = 0; turn < kSplitWaves; ++turn) {
+      if (wave == turn) {
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr)
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            floatx4 x = {acc[4 * h][rr], acc[4 * h + 1][rr], acc[4 * h + 2][rr], acc[4 * h + 3][rr]};
+            if (turn > 0) x = part[rr][h][lane] + x;
+            part[rr][h][lane] = x;
+          }
+      }
+      __syncthreads();
+    }
+    if (col_ok) {  // wave rr stores output row 4g + rr
+      const int v = 4 * g + wave;
+      if (v < V) {
+        const floatx4 lo = part[wave][0][lane], hi = part[wave][1][lane];
+        const float o[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        Store8<OutT>::run(cbase + ((int64_t)lrow * V + v) * p.N + ncol, o);
+      }
+    }
+    __syncthreads();  // part is rewritten for the next long row
+  }
+}
+
+// ------------------------------------------------------------------------------------------
 // Slab kernel: B resident in LDS, operands formed by LDS transpose reads.
 //
 // When K is small enough that a 64-column slab of B (K rows x 128 bytes) fits in the 160 KB of
@@ -883,7 +1031,15 @@ static hipError_t launch_v(const SpmmArgs &a, int which, hipStream_t stream) {
     p.n_tiles = (uint32_t)((a.N + 127) / 128);
     p.total_work = (uint32_t)a.m_vec * p.n_tiles * (uint32_t)a.batch;
     p.per_xcd = (p.total_work + 7u) / 8u;
-    hipLaunchKernelGGL((spmm_gather_kernel<V, OutT>), dim3(p.per_xcd * 8u), dim3(64), 0, stream, p);
+    if (a.K > kSplitMinK) {
+      g_last_kernel = 4;
+      static_assert(kSplitWaves == 4, "wave rr stores output row 4g + rr");
+      p.total_work = (((uint32_t)a.m_vec + kSplitWaves - 1u) / kSplitWaves) * p.n_tiles * (uint32_t)a.batch;
+      p.per_xcd = (p.total_work + 7u) / 8u;
+      hipLaunchKernelGGL((spmm_gather_split_kernel<V, OutT>), dim3(p.per_xcd * 8u), dim3(64 * kSplitWaves), 0, stream, p);
+    } else {
+      hipLaunchKernelGGL((spmm_gather_kernel<V, OutT>), dim3(p.per_xcd * 8u), dim3(64), 0, stream, p);
+    }
   } else {
     p.n_tiles = (uint32_t)((a.N + 63) / 64);
     p.total_work = (uint32_t)a.m_vec * p.n_tiles * (uint32_t)a.batch;

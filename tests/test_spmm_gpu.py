@@ -166,6 +166,38 @@ def test_skewed_row_lengths(oracle, kernel):
     check(oracle, vs, synth.dense_rhs(K, N, seed=15))
 
 
+@pytest.mark.parametrize("V", [8, 16])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
+def test_wide_matrix_with_long_vector_rows(oracle, built_library, V, out_dtype):
+    """K above 4096 runs the gather kernel's variant that splits long vector-rows over the four waves of a
+    workgroup: rows just below and above the 512-vector limit, thousands of vectors, empty rows, a row count
+    that is no multiple of four, a partial last column tile, row_indices, and a batch."""
+    from sspmm_amd import _lib
+    rng = np.random.default_rng(500 + V)
+    K, N, m_vec = 6000, 200, 23
+    lens = rng.integers(0, 40, m_vec)
+    lens[[0, 5, 6, 7, 13, 22]] = [512, 513, 4100, 0, 1999, 545]
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cols = np.concatenate([rng.permutation(K)[:n] for n in lens]).astype(np.int32)
+    vs = synth.VectorSparse(m_vec * V, K, V, m_vec, off, cols,
+                            (rng.standard_normal(cols.size * V) * 0.05).astype(np.float16), cols.size * V)
+    B = synth.dense_rhs(K, N, seed=16)
+    got, _ = check(oracle, vs, B, out_dtype)
+    assert _lib.lib().sspmm_last_kernel() == 4
+    assert not got[7 * V:8 * V].any()
+    perm = rng.permutation(m_vec).astype(np.int32)
+    assert np.array_equal(run(vs, B, out_dtype, dev(perm)), got)
+    # a batch of three shares the pattern
+    vals3 = (rng.standard_normal((3, cols.size * V)) * 0.05).astype(np.float16)
+    B3 = np.stack([synth.dense_rhs(K, N, seed=20 + b) for b in range(3)])
+    out = sspmm_amd.bspmm(None, dev(vs.row_offsets), dev(vs.col_idx), dev(vals3), dev(B3), V, out_dtype=out_dtype)
+    torch.cuda.synchronize()
+    for b in range(3):
+        one = sspmm_amd.spmm(None, dev(vs.row_offsets), dev(vs.col_idx), dev(vals3[b]), dev(B3[b]), V,
+                             out_dtype=out_dtype)
+        assert torch.equal(out[b], one)
+
+
 def test_linearity_at_full_size(built_library):
     """cfg3 at N = 3136 without the oracle: spmm(A, B1 + B2) == spmm(A, B1) + spmm(A, B2) when the
     sums are exact (small integers), and scaling the values by 2 doubles the result exactly."""

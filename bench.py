@@ -132,7 +132,7 @@ def main():
 
     M, K, V, sparsity, N = 2048, 512, 8, 0.9, 256
     kernel_names = {1: "spmm_generic_kernel<8,float>", 2: "spmm_gather_kernel<8,float>", 3: "spmm_slab_kernel<8,float,true>",
-                    4: "spmm_gather_split_kernel<8,float>"}
+                    4: "spmm_gather_split_kernel<8,float>", 5: "spmm_slab_kernel<8,float,*,2>"}
     main_res, (vs, vals, B, C) = spmm_case(L, torch, synth, M, K, V, sparsity, N, args.batch, True, 0.02, 2,
                                            args.steps, args.warmup, dense=not args.quick)
     torch.cuda.synchronize()

@@ -39,8 +39,9 @@ int sspmm_select_kernel(int which);
 
 /* Companion of sspmm_select_kernel (no counterpart in the reference either): the kernel the latest
  * SpMM call of this process ran, numbered as above, with 4 = the gather kernel's variant for
- * K > 4096 that splits long vector-rows over the waves of a workgroup (selected as 2); 0 before
- * any call.  Not thread-safe. */
+ * K > 4096 that splits long vector-rows over the waves of a workgroup (selected as 2) and
+ * 5 = the LDS-slab kernel with 32-column slabs, for K too tall for 64-column ones (selected
+ * as 3); 0 before any call.  Not thread-safe. */
 int sspmm_last_kernel(void);
 
 /* Static text for a return code of this library. */

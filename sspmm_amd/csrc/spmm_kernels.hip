@@ -399,7 +399,9 @@ __global__ __launch_bounds__(64 * kSplitWaves) void spmm_gather_split_kernel(con
 // zeros: unused k slots of a partial step point there.
 static constexpr int kSlabWaves = 16;
 static constexpr int kSlabThreads = kSlabWaves * 64;
-static constexpr int kSlabRowBytes = 128;       // 64 columns of fp16
+// A slab is NQ tiles of 16 columns wide: 4 (64 columns, 128-byte rows) where K lets it fit in LDS, 2 (32 columns,
+// 64-byte rows) for matrices up to twice as tall.
+static constexpr int slab_row_bytes(int NQ) { return 32 * NQ; }
 // Per-wave LDS: the value tile of a step (32 vectors x V halfs; the V = 8 transpose read touches 16
 // bytes past its 512).
 static constexpr int val_tile_bytes(int V) { return V == 8 ? 528 : 1024; }
@@ -532,7 +534,7 @@ __device__ __forceinline__ void slab_store_line(uintx4 line, __amdgpu_buffer_rsr
 //   * fp16: a lane's four columns are 8 bytes; v_permlane16_swap pairs lane groups g and g + 1 of
 //     two tiles so that a lane owns eight consecutive columns, then the DPP exchange as above
 //     gathers all four tiles of a row into one instruction.
-template <int V, typename OutT>
+template <int V, typename OutT, int NQ>
 struct SlabStore;
 
 __device__ __forceinline__ uint32_t dpp_from_m_minus_8(uint32_t keep, uint32_t src) {  // lanes m >= 8 take src of lane m - 8
@@ -542,9 +544,8 @@ __device__ __forceinline__ uint32_t dpp_from_m_plus_8(uint32_t keep, uint32_t sr
   return (uint32_t)__builtin_amdgcn_update_dpp((int)keep, (int)src, 0x108, 0xf, 0x3, false);
 }
 
-template <int V>
-struct SlabStore<V, float> {
-  static constexpr int kInstr = V / 4;  // 2 tile pairs x (V / 8) row halves
+template <int V, int NQ>
+struct SlabStore<V, float, NQ> {
   uint32_t voff[V / 8];                 // byte offset of the lane's 16 bytes for tile pair 0, per row half
   int col[V / 8];                       // its first column
   __device__ __forceinline__ void init(int lane, int n0, int N) {
@@ -557,9 +558,9 @@ struct SlabStore<V, float> {
       voff[h] = ((uint32_t)row * (uint32_t)N + (uint32_t)col[h]) * 4u;
     }
   }
-  __device__ __forceinline__ void store(const floatx4 (&acc)[4], __amdgpu_buffer_rsrc_t srd, uint32_t crow, int N) const {
+  __device__ __forceinline__ void store(const floatx4 (&acc)[NQ], __amdgpu_buffer_rsrc_t srd, uint32_t crow, int N) const {
 #pragma unroll
-    for (int qp = 0; qp < 2; ++qp) {
+    for (int qp = 0; qp < NQ / 2; ++qp) {
 #pragma unroll
       for (int h = 0; h < V / 8; ++h) {
         uintx4 line;
@@ -577,7 +578,7 @@ struct SlabStore<V, float> {
 };
 
 template <int V>
-struct SlabStore<V, _Float16> {
+struct SlabStore<V, _Float16, 4> {
   uint32_t voff[V / 8];
   int col[V / 8];
   __device__ __forceinline__ void init(int lane, int n0, int N) {
@@ -624,6 +625,40 @@ struct SlabStore<V, _Float16> {
   }
 };
 
+// fp16 with a 32-column slab: after the swap a lane owns eight consecutive columns of row m, four lanes make a
+// row's 64 bytes, and one instruction writes the V rows (with V = 8 the lanes m >= 8 have nothing to write).
+template <int V>
+struct SlabStore<V, _Float16, 2> {
+  uint32_t voff;
+  int col;
+  bool row_ok;
+  __device__ __forceinline__ void init(int lane, int n0, int N) {
+    const int m = lane & 15, g = lane >> 4;
+    col = n0 + 16 * (g & 1) + 8 * (g >> 1);
+    voff = ((uint32_t)m * (uint32_t)N + (uint32_t)col) * 2u;
+    row_ok = m < V;
+  }
+  __device__ __forceinline__ void store(const floatx4 (&acc)[2], __amdgpu_buffer_rsrc_t srd, uint32_t crow, int N) const {
+    uint32_t pk[2][2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int w = 0; w < 2; ++w) {
+        typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+        const half2v hv = {(_Float16)acc[t][2 * w], (_Float16)acc[t][2 * w + 1]};  // round to nearest even
+        pk[t][w] = __builtin_bit_cast(uint32_t, hv);
+      }
+    uintx4 line;
+#pragma unroll
+    for (int w = 0; w < 2; ++w) {
+      const auto sw = __builtin_amdgcn_permlane16_swap(pk[0][w], pk[1][w], false, false);
+      line[w] = sw[0];
+      line[2 + w] = sw[1];
+    }
+    if (row_ok && col < N) slab_store_line(line, srd, voff, crow);
+  }
+};
+
 // Per-lane constants of the inner loop and the operands of the current work item.
 template <int V, typename OutT>
 struct SlabCtx {
@@ -637,10 +672,10 @@ struct SlabCtx {
 
 // One wave's share of a work item: the vector-rows wave, wave + 16, ... of the item's row table
 // against the slab at byte offset slab_base of LDS.
-template <int V, typename OutT>
+template <int V, typename OutT, int NQ>
 __device__ __forceinline__ void slab_process_item(const SlabCtx<V, OutT> &x, unsigned char *lds, uint32_t slab_base,
                                                   const SlabRows &rows, const uint16_t *vals,
-                                                  __amdgpu_buffer_rsrc_t srd_c, const SlabStore<V, OutT> &out) {
+                                                  __amdgpu_buffer_rsrc_t srd_c, const SlabStore<V, OutT, NQ> &out) {
   SlabCursor head;  // issues loads
   head.count = 0;
   cursor_prefetch(head, rows);
@@ -667,9 +702,9 @@ __device__ __forceinline__ void slab_process_item(const SlabCtx<V, OutT> &x, uns
   zero_op.u[0] = zero_op.u[1] = zero_op.u[2] = zero_op.u[3] = 0u;
   asm volatile("" : "+v"(zero_op.u[0]), "+v"(zero_op.u[1]), "+v"(zero_op.u[2]), "+v"(zero_op.u[3]));  // keep it in registers
   const floatx4 zero_c = {0.f, 0.f, 0.f, 0.f};
-  floatx4 acc[4];
+  floatx4 acc[NQ];
 #pragma unroll
-  for (int q = 0; q < 4; ++q) acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(zero_op.h, zero_op.h, zero_c, 0, 0, 0);
+  for (int q = 0; q < NQ; ++q) acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(zero_op.h, zero_op.h, zero_c, 0, 0, 0);
   for (;;) {
 #pragma unroll
     for (int u = 0; u < R; ++u) {
@@ -690,11 +725,12 @@ __device__ __forceinline__ void slab_process_item(const SlabCtx<V, OutT> &x, uns
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
         const uint32_t c = ((int)x.slot0 + 4 * h < left) ? ld[cur].col[h] : x.zero_row;
-        addr[h] = ((c << 7) + lane_base) | ((c << 4) & 0x60u);
+        // row c of the slab, and the swizzle of its 32-byte segments (see slab_unit_dst)
+        addr[h] = NQ == 4 ? (((c << 7) + lane_base) | ((c << 4) & 0x60u)) : (((c << 6) + lane_base) | ((c << 3) & 0x20u));
       }
-      Half8Bits b[4];
+      Half8Bits b[NQ];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
+      for (int q = 0; q < NQ; ++q) {
         const uintx2 lo = lds_read_tr_abs(addr[0] ^ ((uint32_t)q << 5));
         const uintx2 hi = lds_read_tr_abs(addr[1] ^ ((uint32_t)q << 5));
         b[q].u[0] = lo[0]; b[q].u[1] = lo[1]; b[q].u[2] = hi[0]; b[q].u[3] = hi[1];
@@ -704,11 +740,11 @@ __device__ __forceinline__ void slab_process_item(const SlabCtx<V, OutT> &x, uns
       if (ld[nxt].valid) *reinterpret_cast<typename SlabVals<V>::type *>(x.val_dst) = ld[nxt].vraw;
 
 #pragma unroll
-      for (int q = 0; q < 4; ++q) acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[q].h, a.h, acc[q], 0, 0, 0);
+      for (int q = 0; q < NQ; ++q) acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[q].h, a.h, acc[q], 0, 0, 0);
       if (left <= 32) {  // last step of the vector-row: write its V x 64 tile of C and start over from zero
         out.store(acc, srd_c, (uint32_t)ld[cur].row * x.c_vrow_bytes, x.N);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(zero_op.h, zero_op.h, zero_c, 0, 0, 0);
+        for (int q = 0; q < NQ; ++q) acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(zero_op.h, zero_op.h, zero_c, 0, 0, 0);
       }
       if (!ld[nxt].valid) return;
     }
@@ -748,13 +784,21 @@ struct SlabFetch {
   intx4 entry;
 };
 
+template <int NQ>
 __device__ __forceinline__ uint32_t slab_unit_src(const SpmmArgs &p, uint32_t u, uint32_t units, uint32_t n0, uint32_t b_bytes) {
-  const uint32_t col = n0 + (u & 7u) * 8u;
-  return (u < units && col < (uint32_t)p.N) ? __umul24(u >> 3, (uint32_t)p.N * 2u) + col * 2u : b_bytes;  // b_bytes: out of bounds, reads zeros
+  constexpr uint32_t kPerRow = 2u * NQ;  // 16-byte units per slab row
+  const uint32_t col = n0 + (u % kPerRow) * 8u;
+  return (u < units && col < (uint32_t)p.N) ? __umul24(u / kPerRow, (uint32_t)p.N * 2u) + col * 2u : b_bytes;  // b_bytes: out of bounds, reads zeros
 }
+// A 16-lane group of a slab read touches four rows at the same segment; rows 256 bytes apart share banks, so the
+// segment index is XORed with the row bits above that distance: (c >> 1) & 3 for 128-byte rows, (c >> 2) & 1 for
+// 64-byte rows.  Rows then collide only when they agree modulo 8.
+template <int NQ>
 __device__ __forceinline__ uint32_t slab_unit_dst(uint32_t u) {
-  const uint32_t c = u >> 3;
-  return c * kSlabRowBytes + (((u & 7u) * 16u) ^ (((c >> 1) & 3u) << 5));
+  constexpr uint32_t kPerRow = 2u * NQ;
+  const uint32_t c = u / kPerRow;
+  const uint32_t swz = NQ == 4 ? ((c >> 1) & 3u) : ((c >> 2) & 1u);
+  return c * slab_row_bytes(NQ) + (((u % kPerRow) * 16u) ^ (swz << 5));
 }
 
 __device__ __forceinline__ intx4 slab_table_fetch(const SpmmArgs &p, const int32_t *__restrict__ row_offsets,
@@ -770,7 +814,7 @@ __device__ __forceinline__ intx4 slab_table_fetch(const SpmmArgs &p, const int32
   return e;
 }
 
-template <int V, typename OutT, bool DOUBLE>
+template <int V, typename OutT, bool DOUBLE, int NQ>
 __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs p,
                                                                  const int32_t *__restrict__ row_offsets,
                                                                  const int32_t *__restrict__ row_indices) {
@@ -786,7 +830,8 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
   const int tid = threadIdx.x, lane = tid & 63, m = lane & 15, g = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // tell the compiler it is wave-uniform
   const uint32_t b_bytes = (uint32_t)p.K * (uint32_t)p.N * 2u;
-  const uint32_t units = (uint32_t)p.K * 8u;
+  constexpr uint32_t kSlabRowBytes = slab_row_bytes(NQ);
+  const uint32_t units = (uint32_t)p.K * (2u * NQ);
 
   // ---- LDS: slab 0, [slab 1], value tiles, row table 0, row table 1
   const uint32_t zero_row = (uint32_t)p.K;
@@ -794,7 +839,7 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
   const uint32_t tiles_off = slab_bytes * (DOUBLE ? 2u : 1u);
   const uint32_t table_off = tiles_off + kSlabWaves * wave_lds_bytes(V);
   const uint32_t table_bytes = (p.rows_per_block + 1u) * 16u;
-  if (tid < 8) {
+  if (tid < 2 * NQ) {
     *reinterpret_cast<uintx4 *>(lds + zero_row * kSlabRowBytes + tid * 16) = uintx4{0u, 0u, 0u, 0u};
     if (DOUBLE) *reinterpret_cast<uintx4 *>(lds + slab_bytes + zero_row * kSlabRowBytes + tid * 16) = uintx4{0u, 0u, 0u, 0u};
   }
@@ -824,11 +869,11 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
 #pragma unroll
       for (int i = 0; i < 4; ++i)
         d[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(
-                                              srd_b, slab_unit_src(p, u0 + i * kSlabThreads + tid, units, cur.tile * 64u, b_bytes), 0, 0));
+                                              srd_b, slab_unit_src<NQ>(p, u0 + i * kSlabThreads + tid, units, cur.tile * (16u * NQ), b_bytes), 0, 0));
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const uint32_t u = u0 + i * kSlabThreads + tid;
-        if (u < units) *reinterpret_cast<uintx4 *>(lds + slab_unit_dst(u)) = d[i];
+        if (u < units) *reinterpret_cast<uintx4 *>(lds + slab_unit_dst<NQ>(u)) = d[i];
       }
     }
     if ((uint32_t)tid <= p.rows_per_block) *reinterpret_cast<intx4 *>(lds + table_off + tid * 16) = e;
@@ -854,7 +899,7 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
 #pragma unroll
         for (int i = 0; i < kSlabFetchUnits; ++i)
           f.d[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(
-                                                  srd_b, slab_unit_src(p, i * kSlabThreads + ftid, units, nxt.tile * 64u, b_bytes), 0, 0));
+                                                  srd_b, slab_unit_src<NQ>(p, i * kSlabThreads + ftid, units, nxt.tile * (16u * NQ), b_bytes), 0, 0));
       }
     }
 
@@ -864,12 +909,12 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
       rows.table = reinterpret_cast<const intx4 *>(lds + table_off + table_sel * table_bytes);
       rows.n_rows = min(p.m_vec, row_lo + (int)p.rows_per_block) - row_lo;
       rows.wave = wave;
-      SlabStore<V, OutT> out;
-      out.init(lane, (int)cur.tile * 64, p.N);
+      SlabStore<V, OutT, NQ> out;
+      out.init(lane, (int)cur.tile * (16 * NQ), p.N);
       // One buffer descriptor spans this batch element's C (the launcher checks it is below 4 GiB).
       const __amdgpu_buffer_rsrc_t srd_c = make_srd(reinterpret_cast<OutT *>(p.C) + (int64_t)cur.batch * p.stride_C,
                                                     (uint32_t)p.m_vec * x.c_vrow_bytes);
-      slab_process_item<V, OutT>(x, lds, slab_sel * slab_bytes, rows, p.values + (int64_t)cur.batch * p.stride_values,
+      slab_process_item<V, OutT, NQ>(x, lds, slab_sel * slab_bytes, rows, p.values + (int64_t)cur.batch * p.stride_values,
                                  srd_c, out);
     }
     if (!has_next) break;
@@ -883,7 +928,7 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
 #pragma unroll
         for (int i = 0; i < kSlabFetchUnits; ++i) {
           const uint32_t u = i * kSlabThreads + ctid;
-          if (u < units) *reinterpret_cast<uintx4 *>(lds + slab_sel * slab_bytes + slab_unit_dst(u)) = f.d[i];
+          if (u < units) *reinterpret_cast<uintx4 *>(lds + slab_sel * slab_bytes + slab_unit_dst<NQ>(u)) = f.d[i];
         }
       }
       table_sel ^= 1u;
@@ -899,11 +944,11 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
 #pragma unroll
           for (int i = 0; i < 4; ++i)
             d[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(
-                                                  srd_b, slab_unit_src(p, u0 + i * kSlabThreads + ctid, units, nxt.tile * 64u, b_bytes), 0, 0));
+                                                  srd_b, slab_unit_src<NQ>(p, u0 + i * kSlabThreads + ctid, units, nxt.tile * (16u * NQ), b_bytes), 0, 0));
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const uint32_t u = u0 + i * kSlabThreads + ctid;
-            if (u < units) *reinterpret_cast<uintx4 *>(lds + slab_unit_dst(u)) = d[i];
+            if (u < units) *reinterpret_cast<uintx4 *>(lds + slab_unit_dst<NQ>(u)) = d[i];
           }
         }
       }
@@ -960,11 +1005,11 @@ static constexpr uint32_t kSlabMaxRows = 512;  // vector-rows per work item (one
 static constexpr uint32_t kSlabMinRows = 32;   // keeps the copy of the slab a small part of an item's traffic
 
 // LDS bytes of a workgroup: slabs (+ zero rows), value tiles, two row tables.
-static uint32_t slab_lds_bytes(int K, int V, uint32_t rows, bool dbl) {
-  return (uint32_t)(K + 1) * kSlabRowBytes * (dbl ? 2u : 1u) + kSlabWaves * wave_lds_bytes(V) + 2u * 16u * (rows + 1u);
+static uint32_t slab_lds_bytes(int K, int V, uint32_t rows, bool dbl, int NQ) {
+  return (uint32_t)(K + 1) * slab_row_bytes(NQ) * (dbl ? 2u : 1u) + kSlabWaves * wave_lds_bytes(V) + 2u * 16u * (rows + 1u);
 }
 // Largest K the slab kernel takes (one slab, smallest row tables).
-static bool slab_fits(int K, int V) { return slab_lds_bytes(K, V, kSlabMinRows, false) <= kSlabLds; }
+static bool slab_fits(int K, int V, int NQ) { return slab_lds_bytes(K, V, kSlabMinRows, false, NQ) <= kSlabLds; }
 
 static constexpr int kMaxDevices = 64;
 static int current_device() {
@@ -984,9 +1029,9 @@ static uint32_t device_cus() {  // of the current device
   return cus[dev];
 }
 
-template <int V, typename OutT, bool DOUBLE>
+template <int V, typename OutT, bool DOUBLE, int NQ>
 static hipError_t launch_slab_kernel(const SpmmArgs &p, uint32_t grid, uint32_t lds, hipStream_t stream) {
-  auto kern = spmm_slab_kernel<V, OutT, DOUBLE>;
+  auto kern = spmm_slab_kernel<V, OutT, DOUBLE, NQ>;
   static bool raised[kMaxDevices] = {};  // per instantiation and device
   const int dev = current_device();
   if (!raised[dev]) {
@@ -998,10 +1043,10 @@ static hipError_t launch_slab_kernel(const SpmmArgs &p, uint32_t grid, uint32_t 
   return hipGetLastError();
 }
 
-template <int V, typename OutT>
+template <int V, typename OutT, int NQ>
 static hipError_t launch_slab(const SpmmArgs &a, hipStream_t stream) {
   SpmmArgs p = a;
-  p.n_tiles = (uint32_t)((a.N + 63) / 64);
+  p.n_tiles = (uint32_t)((a.N + 16 * NQ - 1) / (16 * NQ));
   p.n_slabs = p.n_tiles * (uint32_t)a.batch;
   p.group_by_batch = a.batch >= 8 ? 1u : 0u;
   const uint32_t wgs_per_xcd = device_cus() / 8u;
@@ -1014,19 +1059,20 @@ static hipError_t launch_slab(const SpmmArgs &a, hipStream_t stream) {
   if (row_blocks > max_blocks) row_blocks = max_blocks;
   if (row_blocks < min_blocks) row_blocks = min_blocks;
   uint32_t rows = ((uint32_t)a.m_vec + row_blocks - 1u) / row_blocks;
-  bool dbl = (uint32_t)a.K * 8u <= (uint32_t)kSlabFetchUnits * kSlabThreads && slab_lds_bytes(a.K, V, rows, true) <= kSlabLds;
-  while (!dbl && slab_lds_bytes(a.K, V, rows, false) > kSlabLds && rows > kSlabMinRows) rows = (rows + 1u) / 2u;  // smaller tables for a tall slab
+  bool dbl = (uint32_t)a.K * (2u * NQ) <= (uint32_t)kSlabFetchUnits * kSlabThreads && slab_lds_bytes(a.K, V, rows, true, NQ) <= kSlabLds;
+  while (!dbl && slab_lds_bytes(a.K, V, rows, false, NQ) > kSlabLds && rows > kSlabMinRows) rows = (rows + 1u) / 2u;  // smaller tables for a tall slab
   p.rows_per_block = rows;
   p.row_blocks = ((uint32_t)a.m_vec + rows - 1u) / rows;
-  const uint32_t lds = slab_lds_bytes(a.K, V, rows, dbl);
+  const uint32_t lds = slab_lds_bytes(a.K, V, rows, dbl, NQ);
   const uint32_t grid = 8u * wgs_per_xcd;
-  return dbl ? launch_slab_kernel<V, OutT, true>(p, grid, lds, stream) : launch_slab_kernel<V, OutT, false>(p, grid, lds, stream);
+  return dbl ? launch_slab_kernel<V, OutT, true, NQ>(p, grid, lds, stream) : launch_slab_kernel<V, OutT, false, NQ>(p, grid, lds, stream);
 }
 
 template <int V, typename OutT>
 static hipError_t launch_v(const SpmmArgs &a, int which, hipStream_t stream) {
   SpmmArgs p = a;
-  if (which == 3) return launch_slab<V, OutT>(a, stream);
+  if (which == 3) return launch_slab<V, OutT, 4>(a, stream);
+  if (which == 5) return launch_slab<V, OutT, 2>(a, stream);
   if (which == 2) {
     p.n_tiles = (uint32_t)((a.N + 127) / 128);
     p.total_work = (uint32_t)a.m_vec * p.n_tiles * (uint32_t)a.batch;
@@ -1065,10 +1111,18 @@ hipError_t launch_spmm(const SpmmArgs &a, int V, bool out_f16, hipStream_t strea
     const uint64_t slabs = (uint64_t)((a.N + 63) / 64) * (uint64_t)a.batch;
     const uint64_t blocks = slabs * (uint64_t)((a.m_vec + 31) / 32);
     // The slab kernel addresses one batch element's C through a 32-bit buffer descriptor.
-    const bool slab_ok = slab_fits(a.K, V) && (uint64_t)a.m_vec * (V == 8 ? 8u : 16u) * (uint64_t)a.N * out_size < 0xffffffffull;
+    const bool c_ok = (uint64_t)a.m_vec * (V == 8 ? 8u : 16u) * (uint64_t)a.N * out_size < 0xffffffffull;
+    const bool slab_ok = slab_fits(a.K, V, 4) && c_ok;
+    // Matrices too tall for a 64-column slab can take slabs 32 columns wide, twice as many.  A tall slab is not
+    // double-buffered, so it pays only where many vector-rows share it, and only for V = 8: with V = 16 a
+    // gathered row of B already serves 16 output rows (measured: 1.2-1.3x over the gather kernel for V = 8 from
+    // 256 vector-rows on, 0.8-0.9x for V = 16, 0.5-0.7x with 64 vector-rows at 90 % sparsity and above).
+    const bool narrow_ok = !slab_ok && slab_fits(a.K, V, 2) && c_ok;
     which = (slab_ok && a.m_vec >= 64 && blocks >= 1024) ? 3 : 2;
+    if (narrow_ok && V == 8 && a.m_vec >= 256 && 2u * blocks >= 1024) which = 5;
     if (g_kernel_override == 2) which = 2;
     if (g_kernel_override == 3 && slab_ok) which = 3;
+    if (g_kernel_override == 3 && narrow_ok) which = 5;
   }
   if (g_kernel_override == 1) which = 1;
   g_last_kernel = which;

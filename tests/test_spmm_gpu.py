@@ -53,8 +53,8 @@ def test_cfg2_ffn_v8(oracle, kernel, shape, sparsity):
     vs = synth.vector_sparse(shape[0], shape[1], 8, sparsity, seed=2, std=0.02)
     check(oracle, vs, synth.dense_rhs(shape[1], 256, seed=12))
     from sspmm_amd import _lib
-    if kernel != "auto" and shape[1] == 512:  # the forced kernel is the one that ran (K = 2048 is too tall for the slab)
-        assert _lib.lib().sspmm_last_kernel() == KERNELS[kernel]
+    if kernel != "auto":  # the forced kernel is the one that ran (K = 2048 takes the 32-column slab)
+        assert _lib.lib().sspmm_last_kernel() == (5 if kernel == "slab" and shape[1] == 2048 else KERNELS[kernel])
 
 
 @pytest.mark.parametrize("shape,sparsity,N", [((1024, 2304), 0.8, 256), ((2048, 1024), 0.95, 256),
@@ -271,10 +271,12 @@ def test_slab_kernel_work_item_lists(oracle, built_library, V, batch, m_rows, K,
         assert max_rel_err(out[b], want) <= tol, b
 
 
-@pytest.mark.parametrize("V,K", [(8, 574), (8, 575), (16, 512), (16, 543), (16, 544), (8, 1150), (16, 1100), (8, 1300)])
-def test_slab_kernel_around_its_lds_limits(oracle, built_library, V, K):
-    """K just below and above what two slabs (then one slab) leave room for in LDS; beyond the last limit the
-    forced choice falls back to the gather kernel."""
+@pytest.mark.parametrize("V,K,expect", [(8, 574, 3), (8, 575, 3), (16, 512, 3), (16, 543, 3), (16, 544, 3), (8, 1150, 3),
+                                        (16, 1100, 3), (8, 1300, 5), (16, 1024, 3), (8, 1025, 3), (16, 2286, 5),
+                                        (16, 2287, 2), (8, 2410, 5), (8, 2411, 2)])
+def test_slab_kernel_around_its_lds_limits(oracle, built_library, V, K, expect):
+    """K just below and above what two slabs (then one slab) leave room for in LDS, for the 64-column slab and,
+    above its limit, for the 32-column one; beyond that the forced choice falls back to the gather kernel."""
     from sspmm_amd import _lib
     vs = synth.vector_sparse(80 * V, K, V, 0.95, seed=K)
     B = synth.dense_rhs(K, 192, seed=K + 1)
@@ -284,7 +286,42 @@ def test_slab_kernel_around_its_lds_limits(oracle, built_library, V, K):
         ran = _lib.lib().sspmm_last_kernel()
     finally:
         _lib.lib().sspmm_select_kernel(0)
-    assert ran == (3 if K <= 1150 else 2)
+    assert ran == expect
+
+
+@pytest.mark.parametrize("V", [8, 16])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("N", [32, 72, 200, 256])
+def test_narrow_slab_kernel(oracle, built_library, V, out_dtype, N):
+    """The 32-column slab (K between the 64-column slab's limit and twice that): column tails, ragged and empty
+    rows, unsorted columns, row_indices, a batch that shares slabs between row blocks."""
+    from sspmm_amd import _lib
+    rng = np.random.default_rng(900 + V + N)
+    K, m_vec = 2048, 70
+    lens = rng.integers(0, 90, m_vec)
+    lens[[0, 9, 33]] = [0, 700, 31]
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cols = np.concatenate([rng.permutation(K)[:n] for n in lens]).astype(np.int32)
+    vs = synth.VectorSparse(m_vec * V, K, V, m_vec, off, cols,
+                            (rng.standard_normal(cols.size * V) * 0.1).astype(np.float16), cols.size * V)
+    B = synth.dense_rhs(K, N, seed=N)
+    _lib.lib().sspmm_select_kernel(3)
+    try:
+        got, _ = check(oracle, vs, B, out_dtype)
+        assert _lib.lib().sspmm_last_kernel() == 5
+        assert not got[:V].any()
+        perm = rng.permutation(m_vec).astype(np.int32)
+        assert np.array_equal(run(vs, B, out_dtype, dev(perm)), got)
+        vals5 = (rng.standard_normal((5, cols.size * V)) * 0.1).astype(np.float16)
+        B5 = np.stack([synth.dense_rhs(K, N, seed=40 + b) for b in range(5)])
+        out = sspmm_amd.bspmm(None, dev(vs.row_offsets), dev(vs.col_idx), dev(vals5), dev(B5), V, out_dtype=out_dtype)
+        torch.cuda.synchronize()
+        assert _lib.lib().sspmm_last_kernel() == 5
+        for b in range(5):
+            want = oracle.spmm(vs.m_vec, V, N, K, vs.row_offsets, vs.col_idx, vals5[b], B5[b], threads=8)
+            assert max_rel_err(out[b].cpu().numpy(), want) <= (TIGHT_F32 if out_dtype == torch.float32 else TIGHT_F16)
+    finally:
+        _lib.lib().sspmm_select_kernel(0)
 
 
 def test_row_swizzle_matches_oracle(oracle, built_library):

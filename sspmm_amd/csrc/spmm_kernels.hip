@@ -335,9 +335,13 @@ __global__ __launch_bounds__(64 * kSplitWaves) void spmm_gather_split_kernel(con
     }
   }
   if (!any_long) return;  // uniform over the workgroup
-#pragma unroll
+  // (one copy of the loop body: the extents are read again rather than indexed out of registers)
+#pragma nounroll
   for (int j = 0; j < kSplitWaves; ++j) {
-    const int lrow = g_row[j], lbeg = g_beg[j], lend = g_end[j];
+    const int rj = (int)grp * kSplitWaves + j;
+    if (rj >= p.m_vec) break;
+    const int lrow = p.row_indices ? p.row_indices[rj] : rj;
+    const int lbeg = p.row_offsets[lrow], lend = p.row_offsets[lrow + 1];
     if (lend - lbeg <= 32 * kLongRowSteps) continue;  // uniform over the workgroup
     const int steps = (lend - lbeg + 31) >> 5;
     const int per = (steps + kSplitWaves - 1) / kSplitWaves;
@@ -357,7 +361,7 @@ __global__ __launch_bounds__(64 * kSplitWaves) void spmm_gather_split_kernel(con
       }
       __syncthreads();
     }
-    if (col_ok) {  // wave rr stores output row 4g + rr
+    if (col_ok && wave < 4) {  // wave rr stores output row 4g + rr
       const int v = 4 * g + wave;
       if (v < V) {
         const floatx4 lo = part[wave][0][lane], hi = part[wave][1][lane];
@@ -1079,7 +1083,7 @@ static hipError_t launch_v(const SpmmArgs &a, int which, hipStream_t stream) {
     p.per_xcd = (p.total_work + 7u) / 8u;
     if (a.K > kSplitMinK) {
       g_last_kernel = 4;
-      static_assert(kSplitWaves == 4, "wave rr stores output row 4g + rr");
+      static_assert(kSplitWaves >= 4, "wave rr < 4 stores output row 4g + rr");
       p.total_work = (((uint32_t)a.m_vec + kSplitWaves - 1u) / kSplitWaves) * p.n_tiles * (uint32_t)a.batch;
       p.per_xcd = (p.total_work + 7u) / 8u;
       hipLaunchKernelGGL((spmm_gather_split_kernel<V, OutT>), dim3(p.per_xcd * 8u), dim3(64 * kSplitWaves), 0, stream, p);

@@ -80,6 +80,27 @@ struct Store8<_Float16> {
   }
 };
 
+template <typename OutT, int CPL>
+struct StoreRow;
+template <typename OutT>
+struct StoreRow<OutT, 8> {
+  static __device__ __forceinline__ void run(OutT *p, const float (&v)[8]) { Store8<OutT>::run(p, v); }
+};
+template <>
+struct StoreRow<float, 4> {
+  static __device__ __forceinline__ void run(float *p, const float (&v)[4]) {
+    *reinterpret_cast<floatx4 *>(p) = floatx4{v[0], v[1], v[2], v[3]};
+  }
+};
+template <>
+struct StoreRow<_Float16, 4> {
+  static __device__ __forceinline__ void run(_Float16 *p, const float (&v)[4]) {
+    typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+    const half4v h = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};  // round to nearest even
+    *reinterpret_cast<half4v *>(p) = h;
+  }
+};
+
 // One chunk = 32 consecutive non-zero vectors of a vector-row.  Its loads form a chain of two
 // memory round trips (column indices, then the rows of B they name), so they are issued in two
 // stages, one step apart: while chunk s is contracted, the gathers of chunk s + 1 and the column
@@ -89,8 +110,27 @@ struct ChunkHead {   // stage 1: what does not depend on other loads
   uint16_t a16[8];   // a16[j] = values[(k slot 8g+j), v = m]
   int kc;            // first vector of the chunk
 };
+// CPL = columns per lane: 8 (a wave covers 128 columns) or, for narrow right-hand sides such as attention heads
+// of 64 features, 4 (64 columns: all sixteen lanes of a row group stay useful).
+template <int CPL>
+struct ChunkRaw;
+template <>
+struct ChunkRaw<8> {
+  typedef uintx4 type;
+  static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t srd, uint32_t off) {
+    return __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd, off, 0, 0));
+  }
+};
+template <>
+struct ChunkRaw<4> {
+  typedef uintx2 type;
+  static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t srd, uint32_t off) {
+    return __builtin_bit_cast(uintx2, __builtin_amdgcn_raw_buffer_load_b64(srd, off, 0, 0));
+  }
+};
+template <int CPL = 8>
 struct Chunk {
-  uintx4 raw[8];     // raw[j] = 8 halfs (columns n0+8m..+7) of the row of B named by k slot 8g+j
+  typename ChunkRaw<CPL>::type raw[8];  // raw[j] = CPL halfs (columns n0+CPL*m..) of the row of B named by k slot 8g+j
   uint16_t a16[8];
 };
 
@@ -108,7 +148,8 @@ __device__ __forceinline__ void load_head(ChunkHead &h, int kc, int g, __amdgpu_
     h.a16[j] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(srd_vals, voff + j * V * 2, 0, 0);
 }
 
-__device__ __forceinline__ void load_body(Chunk &c, const ChunkHead &h, int end, int g, __amdgpu_buffer_rsrc_t srd_b,
+template <int CPL>
+__device__ __forceinline__ void load_body(Chunk<CPL> &c, const ChunkHead &h, int end, int g, __amdgpu_buffer_rsrc_t srd_b,
                                           uint32_t lane_n2, uint32_t lane_col_off, uint32_t b_bytes) {
   const int kb = h.kc + 8 * g;
   uint32_t off[8];
@@ -123,17 +164,18 @@ __device__ __forceinline__ void load_body(Chunk &c, const ChunkHead &h, int end,
   }
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
-    c.raw[j] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_b, off[j], 0, 0));
+    c.raw[j] = ChunkRaw<CPL>::load(srd_b, off[j]);
     c.a16[j] = h.a16[j];
   }
 }
 
-__device__ __forceinline__ void mac_chunk(const Chunk &c, floatx4 (&acc)[8]) {
+template <int CPL>
+__device__ __forceinline__ void mac_chunk(const Chunk<CPL> &c, floatx4 (&acc)[CPL]) {
   Half8Bits a;
 #pragma unroll
   for (int d = 0; d < 4; ++d) a.u[d] = (uint32_t)c.a16[2 * d] | ((uint32_t)c.a16[2 * d + 1] << 16);
 #pragma unroll
-  for (int q = 0; q < 8; ++q) {
+  for (int q = 0; q < CPL; ++q) {
     Half8Bits b;
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
@@ -144,7 +186,7 @@ __device__ __forceinline__ void mac_chunk(const Chunk &c, floatx4 (&acc)[8]) {
   }
 }
 
-template <int V, typename OutT>
+template <int V, typename OutT, int CPL>
 __global__ __launch_bounds__(64) void spmm_gather_kernel(const SpmmArgs p) {
   const uint32_t id = blockIdx.x;
   const uint32_t w = (id & 7u) * p.per_xcd + (id >> 3);
@@ -166,22 +208,22 @@ __global__ __launch_bounds__(64) void spmm_gather_kernel(const SpmmArgs p) {
   const __amdgpu_buffer_rsrc_t srd_vals = make_srd(vals, (uint32_t)end * (V * 2u));
   const __amdgpu_buffer_rsrc_t srd_b = make_srd(bmat, b_bytes);
 
-  const int ncol = (int)tile * 128 + m * 8;
+  const int ncol = (int)tile * (16 * CPL) + m * CPL;
   const bool col_ok = ncol < p.N;
   // Lanes whose columns lie beyond N aim every gather at the first byte past B.
   const uint32_t lane_n2 = col_ok ? (uint32_t)p.N * 2u : 0u;
   const uint32_t lane_col_off = col_ok ? (uint32_t)ncol * 2u : b_bytes;
   const uint32_t vals_lane_off = (uint32_t)m * 2u;
 
-  floatx4 acc[8];
+  floatx4 acc[CPL];
 #pragma unroll
-  for (int q = 0; q < 8; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int q = 0; q < CPL; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
 
   if (beg < end) {
     // Heads run two chunks ahead of the arithmetic, bodies one (two buffers of each, used alternately).
     // A head past the end of the row reads zeros and is never turned into a body.
     ChunkHead h0, h1;
-    Chunk c0, c1;
+    Chunk<CPL> c0, c1;
     load_head<V>(h0, beg, g, srd_cols, srd_vals, vals_lane_off);
     load_head<V>(h1, beg + 32, g, srd_cols, srd_vals, vals_lane_off);
     load_body(c0, h0, end, g, srd_b, lane_n2, lane_col_off, b_bytes);
@@ -212,10 +254,10 @@ __global__ __launch_bounds__(64) void spmm_gather_kernel(const SpmmArgs p) {
     for (int rr = 0; rr < 4; ++rr) {
       const int v = 4 * g + rr;
       if (v < V) {
-        float o[8];
+        float o[CPL];
 #pragma unroll
-        for (int q = 0; q < 8; ++q) o[q] = acc[q][rr];
-        Store8<OutT>::run(cbase + ((int64_t)row * V + v) * p.N + ncol, o);
+        for (int q = 0; q < CPL; ++q) o[q] = acc[q][rr];
+        StoreRow<OutT, CPL>::run(cbase + ((int64_t)row * V + v) * p.N + ncol, o);
       }
     }
   }
@@ -254,7 +296,7 @@ __device__ __forceinline__ void gather_accumulate(floatx4 (&acc)[8], const SpmmA
   for (int q = 0; q < 8; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
   if (beg >= sub_end) return;
   ChunkHead h0, h1;
-  Chunk c0, c1;
+  Chunk<8> c0, c1;
   load_head<V>(h0, beg, g, srd_cols, srd_vals, vals_lane_off);
   load_head<V>(h1, beg + 32, g, srd_cols, srd_vals, vals_lane_off);
   load_body(c0, h0, end, g, srd_b, lane_n2, lane_col_off, b_bytes);
@@ -1087,8 +1129,13 @@ static hipError_t launch_v(const SpmmArgs &a, int which, hipStream_t stream) {
       p.total_work = (((uint32_t)a.m_vec + kSplitWaves - 1u) / kSplitWaves) * p.n_tiles * (uint32_t)a.batch;
       p.per_xcd = (p.total_work + 7u) / 8u;
       hipLaunchKernelGGL((spmm_gather_split_kernel<V, OutT>), dim3(p.per_xcd * 8u), dim3(64 * kSplitWaves), 0, stream, p);
+    } else if (a.N <= 64) {
+      p.n_tiles = 1;
+      p.total_work = (uint32_t)a.m_vec * (uint32_t)a.batch;
+      p.per_xcd = (p.total_work + 7u) / 8u;
+      hipLaunchKernelGGL((spmm_gather_kernel<V, OutT, 4>), dim3(p.per_xcd * 8u), dim3(64), 0, stream, p);
     } else {
-      hipLaunchKernelGGL((spmm_gather_kernel<V, OutT>), dim3(p.per_xcd * 8u), dim3(64), 0, stream, p);
+      hipLaunchKernelGGL((spmm_gather_kernel<V, OutT, 8>), dim3(p.per_xcd * 8u), dim3(64), 0, stream, p);
     }
   } else {
     p.n_tiles = (uint32_t)((a.N + 63) / 64);

@@ -74,6 +74,34 @@ def test_column_tails(oracle, kernel, V, N):
 
 
 @pytest.mark.parametrize("V", [8, 16])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("N", [8, 40, 56, 64])
+def test_narrow_right_hand_sides(oracle, built_library, V, out_dtype, N):
+    """N <= 64 (an attention head's features) runs the gather kernel with four columns per lane: ragged rows
+    with partial last chunks, rows of several chunks, empty rows, a batch."""
+    from sspmm_amd import _lib
+    rng = np.random.default_rng(700 + V + N)
+    K, m_vec = 900, 37
+    lens = rng.integers(0, 70, m_vec)
+    lens[[0, 4, 20]] = [0, 333, 32]
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cols = np.concatenate([rng.permutation(K)[:n] for n in lens]).astype(np.int32)
+    vs = synth.VectorSparse(m_vec * V, K, V, m_vec, off, cols,
+                            (rng.standard_normal(cols.size * V) * 0.1).astype(np.float16), cols.size * V)
+    B = synth.dense_rhs(K, N, seed=N)
+    got, _ = check(oracle, vs, B, out_dtype)
+    assert _lib.lib().sspmm_last_kernel() == 2
+    assert not got[:V].any()
+    vals3 = (rng.standard_normal((3, cols.size * V)) * 0.1).astype(np.float16)
+    B3 = np.stack([synth.dense_rhs(K, N, seed=60 + b) for b in range(3)])
+    out = sspmm_amd.bspmm(None, dev(vs.row_offsets), dev(vs.col_idx), dev(vals3), dev(B3), V, out_dtype=out_dtype)
+    torch.cuda.synchronize()
+    for b in range(3):
+        want = oracle.spmm(vs.m_vec, V, N, K, vs.row_offsets, vs.col_idx, vals3[b], B3[b], threads=8)
+        assert max_rel_err(out[b].cpu().numpy(), want) <= (TIGHT_F32 if out_dtype == torch.float32 else TIGHT_F16)
+
+
+@pytest.mark.parametrize("V", [8, 16])
 @pytest.mark.parametrize("N", [1, 3, 17, 66, 130])
 def test_odd_widths_take_the_generic_kernel_and_match_the_oracle_bit_for_bit(oracle, built_library, V, N):
     """N % 8 != 0 runs the scalar kernel, which adds in the oracle's order: fp32 results are identical."""

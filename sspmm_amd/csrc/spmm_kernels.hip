@@ -101,13 +101,53 @@ struct StoreRow<_Float16, 4> {
   }
 };
 
+// The value tile of a step: 32 vectors x V halfs as they lie in memory (vector-major), written to LDS with one
+// 8- or 16-byte store per lane and read back as the MFMA operand (lane (v, g): k = 8g .. 8g+7 of row v) by two
+// ds_read_b64_tr_b16.  The V = 8 transpose read touches 16 bytes past its 512.
+static constexpr int val_tile_bytes(int V) { return V == 8 ? 528 : 1024; }
+
+typedef short shortx4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) shortx4 lds_shortx4;
+
+// The same read at an absolute LDS byte address (saves adding the base of the dynamic LDS array,
+// which the compiler does not fold, to every address).
+__device__ __forceinline__ uintx2 lds_read_tr_abs(uint32_t lds_addr) {
+  const shortx4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4 *)(uintptr_t)lds_addr);
+  return __builtin_bit_cast(uintx2, v);
+}
+__device__ __forceinline__ uint32_t lds_address(const unsigned char *p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const unsigned char *)p;
+}
+__device__ __forceinline__ uintx2 lds_read_tr(const unsigned char *lds_base, uint32_t byte_off) {
+  const shortx4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4 *)(lds_base + byte_off));
+  return __builtin_bit_cast(uintx2, v);
+}
+
+template <int V>
+struct SlabVals;  // the 32 x V halfs of a step, spread over the 64 lanes
+template <>
+struct SlabVals<8> {
+  typedef uintx2 type;  // 8 bytes per lane
+  static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t srd, uint32_t off) {
+    return __builtin_bit_cast(uintx2, __builtin_amdgcn_raw_buffer_load_b64(srd, off, 0, 0));
+  }
+};
+template <>
+struct SlabVals<16> {
+  typedef uintx4 type;  // 16 bytes per lane
+  static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t srd, uint32_t off) {
+    return __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd, off, 0, 0));
+  }
+};
+
 // One chunk = 32 consecutive non-zero vectors of a vector-row.  Its loads form a chain of two
 // memory round trips (column indices, then the rows of B they name), so they are issued in two
 // stages, one step apart: while chunk s is contracted, the gathers of chunk s + 1 and the column
 // indices of chunk s + 2 are in flight.
+template <int V>
 struct ChunkHead {   // stage 1: what does not depend on other loads
   uintx4 c0, c1;     // column indices of k slots 8g .. 8g+7
-  uint16_t a16[8];   // a16[j] = values[(k slot 8g+j), v = m]
+  typename SlabVals<V>::type vraw;  // the lane's share of the chunk's 32 x V values, as they lie in memory
   int kc;            // first vector of the chunk
 };
 // CPL = columns per lane: 8 (a wave covers 128 columns) or, for narrow right-hand sides such as attention heads
@@ -131,26 +171,25 @@ struct ChunkRaw<4> {
 template <int CPL = 8>
 struct Chunk {
   typename ChunkRaw<CPL>::type raw[8];  // raw[j] = CPL halfs (columns n0+CPL*m..) of the row of B named by k slot 8g+j
-  uint16_t a16[8];
 };
 
 template <int V>
-__device__ __forceinline__ void load_head(ChunkHead &h, int kc, int g, __amdgpu_buffer_rsrc_t srd_cols,
+__device__ __forceinline__ void load_head(ChunkHead<V> &h, int kc, int g, __amdgpu_buffer_rsrc_t srd_cols,
                                           __amdgpu_buffer_rsrc_t srd_vals, uint32_t vals_lane_off) {
   const int kb = kc + 8 * g;
   h.kc = kc;
   // srd_cols / srd_vals end at this vector-row's last vector: slots past it read as zero.
   h.c0 = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_cols, kb * 4, 0, 0));
   h.c1 = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_cols, kb * 4 + 16, 0, 0));
-  const uint32_t voff = (uint32_t)kb * (V * 2) + vals_lane_off;
-#pragma unroll
-  for (int j = 0; j < 8; ++j)
-    h.a16[j] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(srd_vals, voff + j * V * 2, 0, 0);
+  // one coalesced load of the chunk's values (vals_lane_off = lane * V bytes); vectors past the row read as zero
+  h.vraw = SlabVals<V>::load(srd_vals, (uint32_t)kc * (V * 2) + vals_lane_off);
 }
 
-template <int CPL>
-__device__ __forceinline__ void load_body(Chunk<CPL> &c, const ChunkHead &h, int end, int g, __amdgpu_buffer_rsrc_t srd_b,
-                                          uint32_t lane_n2, uint32_t lane_col_off, uint32_t b_bytes) {
+// (also sends the chunk's values to the value tile `tile_lane` points into: the lane's slot of the tile)
+template <int CPL, int V>
+__device__ __forceinline__ void load_body(Chunk<CPL> &c, const ChunkHead<V> &h, int end, int g, __amdgpu_buffer_rsrc_t srd_b,
+                                          uint32_t lane_n2, uint32_t lane_col_off, uint32_t b_bytes,
+                                          unsigned char *tile_lane) {
   const int kb = h.kc + 8 * g;
   uint32_t off[8];
 #pragma unroll
@@ -165,15 +204,19 @@ __device__ __forceinline__ void load_body(Chunk<CPL> &c, const ChunkHead &h, int
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
     c.raw[j] = ChunkRaw<CPL>::load(srd_b, off[j]);
-    c.a16[j] = h.a16[j];
   }
+  *reinterpret_cast<typename SlabVals<V>::type *>(tile_lane) = h.vraw;
 }
 
-template <int CPL>
-__device__ __forceinline__ void mac_chunk(const Chunk<CPL> &c, floatx4 (&acc)[CPL]) {
+// tile_op: the lane's address for the transpose reads of the chunk's value tile
+template <int CPL, int V>
+__device__ __forceinline__ void mac_chunk(const Chunk<CPL> &c, floatx4 (&acc)[CPL], const unsigned char *tile_op) {
   Half8Bits a;
-#pragma unroll
-  for (int d = 0; d < 4; ++d) a.u[d] = (uint32_t)c.a16[2 * d] | ((uint32_t)c.a16[2 * d + 1] << 16);
+  {
+    const uintx2 lo = lds_read_tr(tile_op, 0);
+    const uintx2 hi = lds_read_tr(tile_op, 4u * (V * 2u));
+    a.u[0] = lo[0]; a.u[1] = lo[1]; a.u[2] = hi[0]; a.u[3] = hi[1];
+  }
 #pragma unroll
   for (int q = 0; q < CPL; ++q) {
     Half8Bits b;
@@ -188,6 +231,7 @@ __device__ __forceinline__ void mac_chunk(const Chunk<CPL> &c, floatx4 (&acc)[CP
 
 template <int V, typename OutT, int CPL>
 __global__ __launch_bounds__(64) void spmm_gather_kernel(const SpmmArgs p) {
+  __shared__ __align__(16) unsigned char val_tiles[2][val_tile_bytes(V)];  // the value tiles of two chunks in turn
   const uint32_t id = blockIdx.x;
   const uint32_t w = (id & 7u) * p.per_xcd + (id >> 3);
   if (w >= p.total_work) return;
@@ -213,7 +257,12 @@ __global__ __launch_bounds__(64) void spmm_gather_kernel(const SpmmArgs p) {
   // Lanes whose columns lie beyond N aim every gather at the first byte past B.
   const uint32_t lane_n2 = col_ok ? (uint32_t)p.N * 2u : 0u;
   const uint32_t lane_col_off = col_ok ? (uint32_t)ncol * 2u : b_bytes;
-  const uint32_t vals_lane_off = (uint32_t)m * 2u;
+  constexpr uint32_t kLaneBytes = V * 2u * 32u / 64u;
+  const uint32_t vals_lane_off = (uint32_t)lane * kLaneBytes;
+  // where the lane writes its share of a value tile, and where its transpose reads start (rows 8g + m/4 of the tile)
+  unsigned char *const tw0 = val_tiles[0] + lane * kLaneBytes, *const tw1 = val_tiles[1] + lane * kLaneBytes;
+  const uint32_t a_off = (uint32_t)(8 * g + (m >> 2)) * (V * 2u) + (uint32_t)(m & 3) * 8u;
+  const unsigned char *const tr0 = val_tiles[0] + a_off, *const tr1 = val_tiles[1] + a_off;
 
   floatx4 acc[CPL];
 #pragma unroll
@@ -222,28 +271,28 @@ __global__ __launch_bounds__(64) void spmm_gather_kernel(const SpmmArgs p) {
   if (beg < end) {
     // Heads run two chunks ahead of the arithmetic, bodies one (two buffers of each, used alternately).
     // A head past the end of the row reads zeros and is never turned into a body.
-    ChunkHead h0, h1;
+    ChunkHead<V> h0, h1;
     Chunk<CPL> c0, c1;
     load_head<V>(h0, beg, g, srd_cols, srd_vals, vals_lane_off);
     load_head<V>(h1, beg + 32, g, srd_cols, srd_vals, vals_lane_off);
-    load_body(c0, h0, end, g, srd_b, lane_n2, lane_col_off, b_bytes);
+    load_body(c0, h0, end, g, srd_b, lane_n2, lane_col_off, b_bytes, tw0);
     int kc = beg + 32;  // first vector of the chunk whose body is loaded next
     for (;;) {
       if (kc >= end) {
-        mac_chunk(c0, acc);
+        mac_chunk<CPL, V>(c0, acc, tr0);
         break;
       }
       load_head<V>(h0, kc + 32, g, srd_cols, srd_vals, vals_lane_off);
-      load_body(c1, h1, end, g, srd_b, lane_n2, lane_col_off, b_bytes);
-      mac_chunk(c0, acc);
+      load_body(c1, h1, end, g, srd_b, lane_n2, lane_col_off, b_bytes, tw1);
+      mac_chunk<CPL, V>(c0, acc, tr0);
       kc += 32;
       if (kc >= end) {
-        mac_chunk(c1, acc);
+        mac_chunk<CPL, V>(c1, acc, tr1);
         break;
       }
       load_head<V>(h1, kc + 32, g, srd_cols, srd_vals, vals_lane_off);
-      load_body(c0, h0, end, g, srd_b, lane_n2, lane_col_off, b_bytes);
-      mac_chunk(c1, acc);
+      load_body(c0, h0, end, g, srd_b, lane_n2, lane_col_off, b_bytes, tw0);
+      mac_chunk<CPL, V>(c1, acc, tr1);
       kc += 32;
     }
   }
@@ -281,7 +330,8 @@ static constexpr int kSplitMinK = 4096;
 // The partial V x 128 tile of vectors [beg, sub_end) of a vector-row that ends at `end`.
 template <int V>
 __device__ __forceinline__ void gather_accumulate(floatx4 (&acc)[8], const SpmmArgs &p, uint32_t batch, int beg,
-                                                  int sub_end, int end, int lane, int ncol, bool col_ok) {
+                                                  int sub_end, int end, int lane, int ncol, bool col_ok,
+                                                  unsigned char (*val_tiles)[val_tile_bytes(V)]) {
   const int m = lane & 15, g = lane >> 4;
   const uint16_t *vals = p.values + (int64_t)batch * p.stride_values;
   const uint16_t *bmat = p.B + (int64_t)batch * p.stride_B;
@@ -291,32 +341,36 @@ __device__ __forceinline__ void gather_accumulate(floatx4 (&acc)[8], const SpmmA
   const __amdgpu_buffer_rsrc_t srd_b = make_srd(bmat, b_bytes);
   const uint32_t lane_n2 = col_ok ? (uint32_t)p.N * 2u : 0u;
   const uint32_t lane_col_off = col_ok ? (uint32_t)ncol * 2u : b_bytes;
-  const uint32_t vals_lane_off = (uint32_t)m * 2u;
+  constexpr uint32_t kLaneBytes = V * 2u * 32u / 64u;
+  const uint32_t vals_lane_off = (uint32_t)lane * kLaneBytes;
+  unsigned char *const tw0 = val_tiles[0] + lane * kLaneBytes, *const tw1 = val_tiles[1] + lane * kLaneBytes;
+  const uint32_t a_off = (uint32_t)(8 * g + (m >> 2)) * (V * 2u) + (uint32_t)(m & 3) * 8u;
+  const unsigned char *const tr0 = val_tiles[0] + a_off, *const tr1 = val_tiles[1] + a_off;
 #pragma unroll
   for (int q = 0; q < 8; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
   if (beg >= sub_end) return;
-  ChunkHead h0, h1;
+  ChunkHead<V> h0, h1;
   Chunk<8> c0, c1;
   load_head<V>(h0, beg, g, srd_cols, srd_vals, vals_lane_off);
   load_head<V>(h1, beg + 32, g, srd_cols, srd_vals, vals_lane_off);
-  load_body(c0, h0, end, g, srd_b, lane_n2, lane_col_off, b_bytes);
+  load_body(c0, h0, end, g, srd_b, lane_n2, lane_col_off, b_bytes, tw0);
   int kc = beg + 32;  // first vector of the chunk whose body is loaded next
   for (;;) {
     if (kc >= sub_end) {
-      mac_chunk(c0, acc);
+      mac_chunk<8, V>(c0, acc, tr0);
       break;
     }
     load_head<V>(h0, kc + 32, g, srd_cols, srd_vals, vals_lane_off);
-    load_body(c1, h1, end, g, srd_b, lane_n2, lane_col_off, b_bytes);
-    mac_chunk(c0, acc);
+    load_body(c1, h1, end, g, srd_b, lane_n2, lane_col_off, b_bytes, tw1);
+    mac_chunk<8, V>(c0, acc, tr0);
     kc += 32;
     if (kc >= sub_end) {
-      mac_chunk(c1, acc);
+      mac_chunk<8, V>(c1, acc, tr1);
       break;
     }
     load_head<V>(h1, kc + 32, g, srd_cols, srd_vals, vals_lane_off);
-    load_body(c0, h0, end, g, srd_b, lane_n2, lane_col_off, b_bytes);
-    mac_chunk(c1, acc);
+    load_body(c0, h0, end, g, srd_b, lane_n2, lane_col_off, b_bytes, tw0);
+    mac_chunk<8, V>(c1, acc, tr1);
     kc += 32;
   }
 }
@@ -324,6 +378,7 @@ __device__ __forceinline__ void gather_accumulate(floatx4 (&acc)[8], const SpmmA
 template <int V, typename OutT>
 __global__ __launch_bounds__(64 * kSplitWaves) void spmm_gather_split_kernel(const SpmmArgs p) {
   __shared__ floatx4 part[4][2][64];  // the tile being added up: part[rr][half][lane] = acc[4 * half .. + 3][rr]
+  __shared__ __align__(16) unsigned char val_tiles_all[kSplitWaves][2][val_tile_bytes(V)];  // per wave: value tiles of two chunks
   const uint32_t id = blockIdx.x;
   const uint32_t w = (id & 7u) * p.per_xcd + (id >> 3);
   if (w >= p.total_work) return;
@@ -362,7 +417,7 @@ __global__ __launch_bounds__(64 * kSplitWaves) void spmm_gather_split_kernel(con
 
   floatx4 acc[8];
   if (row >= 0 && !is_long) {
-    gather_accumulate<V>(acc, p, batch, beg, end, end, lane, ncol, col_ok);
+    gather_accumulate<V>(acc, p, batch, beg, end, end, lane, ncol, col_ok, val_tiles_all[wave]);
     if (col_ok) {
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
@@ -389,7 +444,7 @@ __global__ __launch_bounds__(64 * kSplitWaves) void spmm_gather_split_kernel(con
     const int per = (steps + kSplitWaves - 1) / kSplitWaves;
     const int my_beg = min(lend, lbeg + wave * per * 32);
     const int my_end = min(lend, my_beg + per * 32);
-    gather_accumulate<V>(acc, p, batch, my_beg, my_end, lend, lane, ncol, col_ok);
+    gather_accumulate<V>(acc, p, batch, my_beg, my_end, lend, lane, ncol, col_ok, val_tiles_all[wave]);
     for (int turn = 0; turn < kSplitWaves; ++turn) {
       if (wave == turn) {
 #pragma unroll
@@ -450,46 +505,11 @@ static constexpr int kSlabThreads = kSlabWaves * 64;
 static constexpr int slab_row_bytes(int NQ) { return 32 * NQ; }
 // Per-wave LDS: the value tile of a step (32 vectors x V halfs; the V = 8 transpose read touches 16
 // bytes past its 512).
-static constexpr int val_tile_bytes(int V) { return V == 8 ? 528 : 1024; }
 static constexpr int wave_lds_bytes(int V) { return val_tile_bytes(V); }
 
 // steps whose loads are in flight or waiting in registers (bounded by the 128 registers a lane has
 // with 16 waves per CU)
 static constexpr int slab_ring(int V) { return V == 8 ? 6 : 5; }
-
-typedef short shortx4 __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) shortx4 lds_shortx4;
-
-// The same read at an absolute LDS byte address (saves adding the base of the dynamic LDS array,
-// which the compiler does not fold, to every address).
-__device__ __forceinline__ uintx2 lds_read_tr_abs(uint32_t lds_addr) {
-  const shortx4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4 *)(uintptr_t)lds_addr);
-  return __builtin_bit_cast(uintx2, v);
-}
-__device__ __forceinline__ uint32_t lds_address(const unsigned char *p) {
-  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const unsigned char *)p;
-}
-__device__ __forceinline__ uintx2 lds_read_tr(const unsigned char *lds_base, uint32_t byte_off) {
-  const shortx4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4 *)(lds_base + byte_off));
-  return __builtin_bit_cast(uintx2, v);
-}
-
-template <int V>
-struct SlabVals;  // the 32 x V halfs of a step, spread over the 64 lanes
-template <>
-struct SlabVals<8> {
-  typedef uintx2 type;  // 8 bytes per lane
-  static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t srd, uint32_t off) {
-    return __builtin_bit_cast(uintx2, __builtin_amdgcn_raw_buffer_load_b64(srd, off, 0, 0));
-  }
-};
-template <>
-struct SlabVals<16> {
-  typedef uintx4 type;  // 16 bytes per lane
-  static __device__ __forceinline__ type load(__amdgpu_buffer_rsrc_t srd, uint32_t off) {
-    return __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd, off, 0, 0));
-  }
-};
 
 template <int V>
 struct SlabLoads {    // what the head records for a step; the step consumes it slab_ring(V) - 1 steps later

@@ -138,6 +138,28 @@ def main():
     torch.cuda.synchronize()
     main_kernel = kernel_names.get(L.sspmm_last_kernel(), "unknown")
 
+    # the same workload as 128 separate launches, one batch element each, rotating through the 335 MB of distinct
+    # operands (nothing a launch touches is still in a cache from the launch before): per-launch time when
+    # launches are small and cold
+    cold = None
+    if not args.quick and args.batch >= 8:
+        ro_d, ci_d = torch.from_numpy(vs.row_offsets).cuda(), torch.from_numpy(vs.col_idx).cuda()
+        st0 = torch.cuda.current_stream().cuda_stream
+        turn = [0]
+
+        def one_cold():
+            i = turn[0] % args.batch
+            turn[0] += 1
+            rc = L.sspmm_f16_f32(vs.m_vec, V, N, K, None, ro_d.data_ptr(), ci_d.data_ptr(), vals[i].data_ptr(),
+                                 B[i].data_ptr(), C[i].data_ptr(), st0)
+            assert rc == 0, rc
+
+        cold_ms = time_launches(one_cold, 4 * args.batch, args.batch)
+        one_bytes = synth.spmm_algorithmic_bytes(vs.m_vec, V, vs.col_idx.size, K, N, 4)
+        cold = {"workload": "one batch element per launch, %d distinct operand sets in rotation" % args.batch,
+                "ms": cold_ms, "useful_tflops": 2.0 * vs.nnz * N / cold_ms / 1e9, "alg_bytes": one_bytes,
+                "hbm_gbps": one_bytes / cold_ms / 1e6, "hbm_frac": one_bytes / cold_ms / 1e6 / HBM_PEAK_GBPS}
+
     # what this box's memory system sustains for plain streams of the same size class, measured the same way
     # (50 launches after warm-up): a device copy (half reads, half writes) and a fill (writes only)
     ceilings = None
@@ -181,6 +203,8 @@ def main():
     del vals, B, C
 
     extra = {}
+    if cold:
+        extra["cfg2_single_launches_cold"] = cold
     if not args.quick:
         st, wu = max(20, args.steps // 4), 5
         cases = {

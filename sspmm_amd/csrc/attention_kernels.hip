@@ -197,9 +197,17 @@ struct VecLoad<16> {
 
 // One wave per (vector-row, batch element); lane l takes the stored vectors l, l + 64, ... of the
 // row, V dense rows at a time.  Three passes over the row's values (maximum, sum of exponentials,
-// result): the first comes from HBM, the other two hit the caches.
+// result).  The first kSoftmaxCached vectors of every lane (512 / 256 vectors of the row for V = 8 / 16) are
+// loaded once, all loads in flight together, and stay in registers for the three passes; only the
+// rest of a longer row is read again (from the caches).
+template <int V>
+struct SoftmaxCached {
+  static constexpr int value = V == 8 ? 8 : 4;
+};
+
 template <int V>
 __global__ __launch_bounds__(64) void softmax_kernel(const SoftmaxArgs p) {
+  constexpr int KC = SoftmaxCached<V>::value;
   const uint32_t w = xcd_work_index(p.per_xcd);
   if (w >= p.total_work) return;
   const uint32_t r = w % (uint32_t)p.m_vec;
@@ -211,6 +219,19 @@ __global__ __launch_bounds__(64) void softmax_kernel(const SoftmaxArgs p) {
   const uint16_t *in = p.values + (int64_t)batch * p.stride;
   uint16_t *out = p.out + (int64_t)batch * p.stride;
   const float s = p.scaler;
+  const int tail = beg + lane + 64 * KC;  // the lane's first vector that is not held in registers
+
+  _Float16 cached[KC][V];
+#pragma unroll
+  for (int i = 0; i < KC; ++i) {
+    const int j = beg + lane + 64 * i;
+    if (j < end) {
+      VecLoad<V>::load(in + (int64_t)j * V, cached[i]);
+    } else {
+#pragma unroll
+      for (int v = 0; v < V; ++v) cached[i][v] = (_Float16)0;  // never used: the passes below skip these slots
+    }
+  }
 
   float mx[V], sum[V];
 #pragma unroll
@@ -218,7 +239,13 @@ __global__ __launch_bounds__(64) void softmax_kernel(const SoftmaxArgs p) {
     mx[v] = -INFINITY;
     sum[v] = 0.f;
   }
-  for (int j = beg + lane; j < end; j += 64) {
+#pragma unroll
+  for (int i = 0; i < KC; ++i)
+    if (beg + lane + 64 * i < end) {
+#pragma unroll
+      for (int v = 0; v < V; ++v) mx[v] = fmaxf(mx[v], (float)cached[i][v] * s);
+    }
+  for (int j = tail; j < end; j += 64) {
     _Float16 x[V];
     VecLoad<V>::load(in + (int64_t)j * V, x);
 #pragma unroll
@@ -226,7 +253,13 @@ __global__ __launch_bounds__(64) void softmax_kernel(const SoftmaxArgs p) {
   }
 #pragma unroll
   for (int v = 0; v < V; ++v) mx[v] = wave_max(mx[v]);
-  for (int j = beg + lane; j < end; j += 64) {
+#pragma unroll
+  for (int i = 0; i < KC; ++i)
+    if (beg + lane + 64 * i < end) {
+#pragma unroll
+      for (int v = 0; v < V; ++v) sum[v] += __expf((float)cached[i][v] * s - mx[v]);
+    }
+  for (int j = tail; j < end; j += 64) {
     _Float16 x[V];
     VecLoad<V>::load(in + (int64_t)j * V, x);
 #pragma unroll
@@ -234,7 +267,17 @@ __global__ __launch_bounds__(64) void softmax_kernel(const SoftmaxArgs p) {
   }
 #pragma unroll
   for (int v = 0; v < V; ++v) sum[v] = 1.0f / wave_sum(sum[v]);
-  for (int j = beg + lane; j < end; j += 64) {
+#pragma unroll
+  for (int i = 0; i < KC; ++i) {
+    const int j = beg + lane + 64 * i;
+    if (j < end) {
+      _Float16 y[V];
+#pragma unroll
+      for (int v = 0; v < V; ++v) y[v] = (_Float16)(__expf((float)cached[i][v] * s - mx[v]) * sum[v]);
+      VecLoad<V>::store(out + (int64_t)j * V, y);
+    }
+  }
+  for (int j = tail; j < end; j += 64) {
     _Float16 x[V], y[V];
     VecLoad<V>::load(in + (int64_t)j * V, x);
 #pragma unroll

@@ -59,7 +59,7 @@ def test_sddmm_row_length_tails_and_permutation(oracle, built_library, per_row):
 @pytest.mark.parametrize("V", [8, 16])
 def test_softmax_matches_oracle_and_rows_sum_to_one(oracle, built_library, V):
     rng = np.random.default_rng(7)
-    lens = np.array([0, 1, 5, 64, 65, 200, 0, 1000, 3])
+    lens = np.array([0, 1, 5, 64, 65, 200, 0, 1000, 3, 256, 257, 512, 513])  # around what a wave keeps in registers
     off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
     vals = (rng.standard_normal(off[-1] * V) * 4).astype(np.float16)
     scaler = 1.0 / math.sqrt(64)
@@ -72,6 +72,9 @@ def test_softmax_matches_oracle_and_rows_sum_to_one(oracle, built_library, V):
     for i, n in enumerate(lens):
         if n:
             assert np.all(np.abs(g[off[i]:off[i + 1]].sum(axis=0) - 1) < 1e-2)
+    # a negative scaler turns the row's minimum into the reference point
+    neg = sspmm_amd.csr_softmax(None, dev(off), dev(vals), -0.25, V).cpu().numpy()
+    assert np.abs(neg.astype(np.float64) - oracle.softmax(len(lens), V, off, vals, -0.25).astype(np.float64)).max() <= 2e-3
     # a large common offset must not overflow: softmax is shift invariant
     big = (vals.astype(np.float32) + 30000).astype(np.float16)
     shifted = sspmm_amd.csr_softmax(None, dev(off), dev(big), 1.0, V).cpu().numpy()

@@ -40,13 +40,20 @@ __device__ __forceinline__ uint32_t xcd_work_index(uint32_t per_xcd) {
 
 // ------------------------------------------------------------------------------------ sddmm
 // One wave per (vector-row, batch element).  The V rows of lhs are the MFMA's first operand and
-// stay in registers (lane (m, g) holds features 32c + 8g .. + 7 of row m, c = 0 .. NC-1); per
-// group of 16 stored vectors, lane (m, g) loads the same features of the row of rhs named by
-// vector m, 16 contiguous bytes per load with no shuffling, NC MFMAs contract the features, and
-// the lane ends up with rows 4g .. 4g+3 of vector m: eight contiguous bytes of the output.
-// The column indices run two groups ahead of the arithmetic and the rows of rhs one group.
+// stay in registers (lane (m, g) holds features 32c + 8g .. + 7 of row m, c = 0 .. NC-1).  Per
+// group of 16 stored vectors the 16 rows of rhs they name are needed in the same layout, lane
+// (m, g) holding features 32c + 8g .. of the row of vector m.  Loaded that way, neighbouring
+// lanes would read 16 bytes each of sixteen different rows; instead the rows are fetched with
+// neighbouring lanes on neighbouring 16-byte pieces of one row (whole 128-byte lines for 64
+// features), written to a small LDS stage, and read back in the operand layout.  Rows of the
+// stage are padded by 16 bytes so that the sixteen rows a read touches spread over the banks.
+// NC MFMAs contract the features, and the lane ends up with rows 4g .. 4g+3 of vector m: eight
+// contiguous bytes of the output.  The column indices run two groups ahead of the arithmetic, the
+// rows of rhs one group (two stages, used alternately).
 template <int V, int NC>
 __global__ __launch_bounds__(64) void sddmm_kernel(const SddmmArgs p) {
+  constexpr uint32_t kStageRow = NC * 64u + 16u;  // bytes: room for 32 * NC features, and the padding
+  __shared__ __align__(16) unsigned char stage[2][16 * kStageRow];
   const uint32_t w = xcd_work_index(p.per_xcd);
   if (w >= p.total_work) return;
   const uint32_t r = w % (uint32_t)p.m_vec;
@@ -64,56 +71,97 @@ __global__ __launch_bounds__(64) void sddmm_kernel(const SddmmArgs p) {
   const __amdgpu_buffer_rsrc_t srd_cols = make_srd(p.col_idx, (uint32_t)end * 4u);  // past the row: reads 0
   uint16_t *out = p.out + (int64_t)batch * p.stride_out;
 
-  // feature offsets of this lane's 16-byte pieces; pieces past F (or rows past V) read zeros
-  uint32_t foff[NC];
+  // operand side: feature offsets of this lane's 16-byte pieces; pieces past F (or rows past V) are zeros
+  uint32_t op_off[NC];
+  bool op_ok[NC];
   half8 a[NC];
 #pragma unroll
   for (int c = 0; c < NC; ++c) {
     const uint32_t f0 = 32u * c + 8u * g;
-    foff[c] = f0 < F ? f0 * 2u : 0xffffffffu;
+    op_ok[c] = f0 < F;
+    op_off[c] = (uint32_t)m * kStageRow + f0 * 2u;
     const uint32_t off = (m < V && f0 < F) ? ((uint32_t)m * F + f0) * 2u : 0xfffffff0u;
     a[c] = __builtin_bit_cast(half8, __builtin_amdgcn_raw_buffer_load_b128(srd_lhs, off, 0, 0));
   }
-
-  auto load_cols = [&](int kc) { return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(srd_cols, (kc + m) * 4, 0, 0); };
-  auto load_rows = [&](half8(&b)[NC], uint32_t col) {
+  // fetch side: piece lane + 64 i of the group's 16 * F / 8 pieces, row-major (piece = 8 features of one row)
+  const uint32_t chunks = F / 8u;
+  uint32_t ld_row[NC], ld_src[NC], ld_dst[NC];
+  bool ld_ok[NC];
 #pragma unroll
-    for (int c = 0; c < NC; ++c) {
-      const uint32_t off = foff[c] == 0xffffffffu ? 0xfffffff0u : __umul24(col, F * 2u) + foff[c];
-      b[c] = __builtin_bit_cast(half8, __builtin_amdgcn_raw_buffer_load_b128(srd_rhs, off, 0, 0));
+  for (int i = 0; i < NC; ++i) {
+    const uint32_t piece = (uint32_t)lane + 64u * i;
+    ld_row[i] = piece / chunks;
+    const uint32_t ch = piece - ld_row[i] * chunks;
+    ld_ok[i] = ld_row[i] < 16u;
+    ld_src[i] = ch * 16u;
+    ld_dst[i] = ld_row[i] * kStageRow + ch * 16u;
+  }
+
+  struct Cols {
+    uint32_t c[NC];
+  };
+  struct Pieces {
+    uintx4 d[NC];
+  };
+  auto load_cols = [&](int kc) {
+    Cols x;
+#pragma unroll
+    for (int i = 0; i < NC; ++i)
+      x.c[i] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(srd_cols, (kc + (int)ld_row[i]) * 4, 0, 0);
+    return x;
+  };
+  auto load_rows = [&](Pieces &b, const Cols &x) {
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      const uint32_t off = ld_ok[i] ? __umul24(x.c[i], F * 2u) + ld_src[i] : 0xfffffff0u;
+      b.d[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_rhs, off, 0, 0));
     }
   };
-  auto finish = [&](const half8(&b)[NC], int kc) {
+  auto to_stage = [&](const Pieces &b, unsigned char *st) {
+#pragma unroll
+    for (int i = 0; i < NC; ++i)
+      if (ld_ok[i]) *reinterpret_cast<uintx4 *>(st + ld_dst[i]) = b.d[i];
+  };
+  auto finish = [&](const unsigned char *st, int kc) {
     floatx4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int c = 0; c < NC; ++c) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[c], b[c], acc, 0, 0, 0);
+    for (int c = 0; c < NC; ++c) {
+      half8 b = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (op_ok[c]) b = *reinterpret_cast<const half8 *>(st + op_off[c]);
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[c], b, acc, 0, 0, 0);
+    }
     if (kc + m < end && 4 * g < V) {
       const half4 h = {(_Float16)acc[0], (_Float16)acc[1], (_Float16)acc[2], (_Float16)acc[3]};  // round to nearest even
       *reinterpret_cast<half4 *>(out + ((int64_t)(kc + m) * V + 4 * g)) = h;
     }
   };
 
-  half8 b0[NC], b1[NC];
-  uint32_t c_next = load_cols(beg + 16);
+  // The LDS operations of a wave execute in order, so a stage can be rewritten right after the reads of the group
+  // that used it have been issued; no barrier is involved (one wave per workgroup).
+  Pieces b0, b1;
+  Cols c_next = load_cols(beg + 16);
   load_rows(b0, load_cols(beg));
+  to_stage(b0, stage[0]);
   int kc = beg;
   for (;;) {
-    // b0 holds group kc; c_next the columns of group kc + 16
+    // stage[0] holds group kc; c_next the columns of group kc + 16
     if (kc + 16 >= end) {
-      finish(b0, kc);
+      finish(stage[0], kc);
       break;
     }
-    uint32_t c_after = load_cols(kc + 32);
+    Cols c_after = load_cols(kc + 32);
     load_rows(b1, c_next);
-    finish(b0, kc);
+    finish(stage[0], kc);
+    to_stage(b1, stage[1]);
     kc += 16;
     if (kc + 16 >= end) {
-      finish(b1, kc);
+      finish(stage[1], kc);
       break;
     }
     c_next = load_cols(kc + 32);
     load_rows(b0, c_after);
-    finish(b1, kc);
+    finish(stage[1], kc);
+    to_stage(b0, stage[0]);
     kc += 16;
   }
 }

@@ -816,6 +816,9 @@ struct SideStreams {
   bool ready = false;
   hipStream_t s[3];
   hipEvent_t fork, join[3];
+  // held while a call enqueues its fork .. join sequence: the events are re-recorded by every call, so two host
+  // threads must not interleave their sequences on one device
+  std::mutex in_use;
 };
 static SideStreams g_side[16];
 static std::mutex g_side_mutex;
@@ -878,6 +881,8 @@ hipError_t launch_svc_count(const SvcArgs &a, int order, hipStream_t stream) {
     // One pass over the groups per size class, each taking the groups of its class; a group's class
     // is decided from min(non-zeros of the group, K), an upper bound of its distinct columns.
     SideStreams *ss = side_streams();
+    std::unique_lock<std::mutex> sequence;
+    if (ss) sequence = std::unique_lock<std::mutex>(ss->in_use);
     hipStream_t st[4];
     if ((e = fork_streams(ss, stream, st)) != hipSuccess) return e;
     if ((e = launch_lds_class<64>(a, m_vec, -1, kSmallKeys, 512, st[0])) != hipSuccess) return e;
@@ -928,6 +933,8 @@ hipError_t launch_svc_fill(const SvcArgs &args, int order, const uint16_t *csr_v
   const uint32_t key_bits = bits_of(a.K);
   hipError_t e;
   SideStreams *ss = side_streams();
+  std::unique_lock<std::mutex> sequence;
+  if (ss) sequence = std::unique_lock<std::mutex>(ss->in_use);
   hipStream_t st[4];
   if ((e = fork_streams(ss, stream, st, 1)) != hipSuccess) return e;
   // Grids: what the chip holds at once for the class's workgroup size and LDS, at most one workgroup per group.

@@ -145,6 +145,39 @@ def test_a_row_that_repeats_a_column_stays_inside_its_group(built_library):
     assert ((vcol >= 0) & (vcol < K)).all() and np.isin(vval, [0.0, 1.0]).all()
 
 
+def test_calls_from_several_host_threads_on_their_own_streams(oracle, built_library):
+    """The helper streams and events of the merge are per device: concurrent callers must not mix their
+    fork / join sequences."""
+    import threading
+    rng = np.random.default_rng(79)
+    cases = [_random_csr(rng, 600 + 50 * t, 3000, 900) for t in range(4)]
+    want = [oracle.svc(c.M, c.K, 8, c.row_ptr, c.col_ind, c.values) for c in cases]
+    errors = []
+
+    def worker(t):
+        try:
+            c = cases[t]
+            with torch.cuda.stream(torch.cuda.Stream()):
+                args = (dev(c.row_ptr), dev(c.col_ind), dev(c.values), c.M, c.K, 8)
+                for _ in range(8):
+                    r = sspmm_amd.svc(*args)
+                    torch.cuda.current_stream().synchronize()
+                    ok = (np.array_equal(r.vec_row_ptr.cpu().numpy(), want[t][0]) and
+                          np.array_equal(r.vec_col.cpu().numpy(), want[t][1]) and
+                          np.array_equal(r.vec_val.cpu().numpy().view(np.uint16), want[t][2].view(np.uint16)))
+                    if not ok:
+                        errors.append("thread %d: mismatch" % t)
+        except Exception as e:  # noqa: BLE001
+            errors.append("thread %d: %r" % (t, e))
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(4)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
+
+
 def test_cfg1_rowmerge_returns_the_vector_pattern(oracle, built_library):
     vs = synth.vector_sparse(512, 512, 8, 0.9, seed=1)
     csr = synth.expand_to_csr(vs)

@@ -211,6 +211,10 @@ def main():
             "cfg2_single_launch": dict(M=2048, K=512, V=8, sparsity=0.9, N=256, batch=1, out_f32=True, std=0.02, seed=2),
             "cfg2_batched_fp16_out": dict(M=2048, K=512, V=8, sparsity=0.9, N=256, batch=args.batch, out_f32=False,
                                           std=0.02, seed=2),
+            "cfg2_shape_v16_batched": dict(M=2048, K=512, V=16, sparsity=0.9, N=256, batch=args.batch, out_f32=True,
+                                           std=0.02, seed=2),
+            "cfg2_shape_v16_batched_fp16_out": dict(M=2048, K=512, V=16, sparsity=0.9, N=256, batch=args.batch,
+                                                    out_f32=False, std=0.02, seed=2),
             "cfg3_1024x2304_v16_s0.8_n3136": dict(M=1024, K=2304, V=16, sparsity=0.8, N=3136, batch=1, out_f32=True,
                                                   std=0.05, seed=3),
             "cfg3_2048x1024_v16_s0.95_n3136": dict(M=2048, K=1024, V=16, sparsity=0.95, N=3136, batch=1,

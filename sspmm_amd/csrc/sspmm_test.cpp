@@ -99,6 +99,39 @@ float to_float<float>(float v) { return v; }
 template <>
 float to_float<__half>(__half v) { return __half2float(v); }
 
+// What this device sustains for a plain copy (reads + writes of 1 GiB each way), measured once per run: the
+// denominator beside the published HBM peak.
+double device_copy_gbs() {
+  static double gbs = 0;
+  if (gbs > 0) return gbs;
+  const size_t bytes = (size_t)1 << 30;
+  void *src = nullptr, *dst = nullptr;
+  if (hipMalloc(&src, bytes) != hipSuccess || hipMalloc(&dst, bytes) != hipSuccess) {
+    (void)hipFree(src);
+    (void)hipGetLastError();
+    return gbs = -1;
+  }
+  check(hipMemset(src, 1, bytes), "memset");
+  hipEvent_t a, b;
+  check(hipEventCreate(&a), "event");
+  check(hipEventCreate(&b), "event");
+  for (int i = 0; i < 3; ++i) check(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, nullptr), "copy");
+  check(hipEventRecord(a), "record");
+  const int reps = 20;
+  for (int i = 0; i < reps; ++i) check(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, nullptr), "copy");
+  check(hipEventRecord(b), "record");
+  check(hipEventSynchronize(b), "sync");
+  float ms = 0;
+  check(hipEventElapsedTime(&ms, a, b), "elapsed");
+  check(hipEventDestroy(a), "event");
+  check(hipEventDestroy(b), "event");
+  (void)hipFree(src);
+  (void)hipFree(dst);
+  gbs = 2.0 * bytes * reps / ms / 1e6;
+  std::printf("Device copy of 1 GiB: %.1f GB/s (reads + writes) = %.1f %% of the HBM peak\n", gbs, 100.0 * gbs / kHbmPeakGBs);
+  return gbs;
+}
+
 template <typename OutT>
 void bench(const Pattern &p, int N, int V, int kernel, bool sorted, bool func, bool record, bool reorder,
            const std::string &arch) {
@@ -170,9 +203,12 @@ void bench(const Pattern &p, int N, int V, int kernel, bool sorted, bool func, b
   const double bytes = 2.0 * V * nvec + 4.0 * nvec + 4.0 * (m_vec + 1) + 2.0 * K * N + sizeof(OutT) * (double)M * N;
   const double gbs = bytes / ms / 1e6;
   const double sp = M > 0 && K > 0 ? 100.0 - (double)p.nnz * 100 / M / K : 100.0;
+  const double copy_gbs = device_copy_gbs();  // (prints its own line the first time)
   std::printf("M = %d, K = %d, N = %d, NNZ = %lld, Sparsity = %lf%%\n", M, K, N, p.nnz, sp);
-  std::printf("Average Performance = %lf GFlops, %.3f us per launch, %.1f GB/s = %.1f %% of the HBM peak\n", gflops,
+  std::printf("Average Performance = %lf GFlops, %.3f us per launch, %.1f GB/s = %.1f %% of the HBM peak", gflops,
               ms * 1e3, gbs, 100.0 * gbs / kHbmPeakGBs);
+  if (copy_gbs > 0) std::printf(", %.1f %% of the device's copy rate", 100.0 * gbs / copy_gbs);
+  std::printf("\n");
   if (record) {
     const std::string path = "./data/" + arch + "_rospmm_" + std::to_string(V) + (reorder ? "_v1.csv" : "_v0.csv");
     std::ofstream out(path, std::ios::app);

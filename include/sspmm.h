@@ -147,7 +147,9 @@ int sspmm_softmax_batched_f16(int batch, int m_vec, int V, const int32_t *row_in
  * order: SVC_ORDER_CPYTHON reproduces the column order of the reference's output files (the
  * iteration order of CPython's set in `list(set(acc + row))`), bit for bit;
  * SVC_ORDER_SORTED stores each vector-row's columns ascending.
- * Column indices must lie in [0, K); a CSR row must not repeat a column.
+ * Column indices must lie in [0, K) and a CSR row must not repeat a column; a non-zero that breaks
+ * the first rule is ignored, rows that break the second give an unspecified column order, and
+ * neither makes the kernels touch memory outside the arrays named here.
  * ---------------------------------------------------------------------------------------- */
 #define SVC_ORDER_CPYTHON 0
 #define SVC_ORDER_SORTED 1

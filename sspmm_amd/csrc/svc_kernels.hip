@@ -215,7 +215,7 @@ __global__ __launch_bounds__(THREADS) void svc_count_distinct_kernel(const SvcAr
   int mine = 0;
   for (int idx = e0 + (int)threadIdx.x; idx < e1; idx += THREADS) {
     const uint32_t c = (uint32_t)a.col_ind[idx], bit = 1u << (c & 31u);
-    mine += (atomicOr(&bits[c >> 5], bit) & bit) ? 0 : 1;
+    if (c < (uint32_t)a.K) mine += (atomicOr(&bits[c >> 5], bit) & bit) ? 0 : 1;  // (a column outside [0, K) is ignored)
   }
   int total;
   block_exclusive_scan<THREADS>(mine, &total, scratch);
@@ -251,7 +251,8 @@ __device__ __forceinline__ void write_group_output(const SvcArgs &a, int grp, in
   for (int r = r0; r < r1; ++r) {
     const int b = a.row_ptr[r], e = a.row_ptr[r + 1];
     for (int idx = b + (int)threadIdx.x; idx < e; idx += THREADS) {
-      const int p = position_of((uint32_t)a.col_ind[idx]);
+      const uint32_t c = (uint32_t)a.col_ind[idx];
+      const int p = c < (uint32_t)a.K ? position_of(c) : -1;
       if (p >= 0 && p < n_out) out[(int64_t)p * a.V + (r - r0)] = a.csr_val[idx];
     }
   }
@@ -296,7 +297,7 @@ __global__ __launch_bounds__(THREADS) void svc_merge_cpython_kernel(const SvcArg
       int key = 0;
       if (idx < e) {
         key = a.col_ind[idx];
-        is_new = (slots == 0) || find_slot(table, slots - 1u, (uint32_t)key) < 0;
+        is_new = (uint32_t)key < (uint32_t)a.K && ((slots == 0) || find_slot(table, slots - 1u, (uint32_t)key) < 0);
       }
       int total;
       const int rank = block_exclusive_scan<THREADS>(is_new ? 1 : 0, &total, scratch);
@@ -321,8 +322,9 @@ __global__ __launch_bounds__(THREADS) void svc_merge_cpython_kernel(const SvcArg
     for (int p = threadIdx.x; p < n; p += THREADS) a.tmp_cols[e0 + p] = list[p];
   if (n > 0)
     for (int idx = e0 + (int)threadIdx.x; idx < e1; idx += THREADS) {
-      const int s = find_slot(table, slots - 1u, (uint32_t)a.col_ind[idx]);
-      a.pos[idx] = s >= 0 ? (int)(table[s] >> 32) : 0;  // s < 0 only for invalid (capped) input
+      const uint32_t c = (uint32_t)a.col_ind[idx];
+      const int s = c < (uint32_t)a.K ? find_slot(table, slots - 1u, c) : -1;
+      a.pos[idx] = s >= 0 ? (int)(table[s] >> 32) : -1;  // s < 0 only for invalid input: the fill skips it
     }
   }
 }
@@ -616,7 +618,7 @@ __global__ __launch_bounds__(THREADS) void svc_merge_fast_kernel(const SvcArgs a
       uint32_t k = 0;
       if (idx < e) {
         k = (uint32_t)a.col_ind[idx];
-        is_new = (slots == 0) || find_slot32(t, slots - 1u, k) < 0;
+        is_new = k < (uint32_t)a.K && ((slots == 0) || find_slot32(t, slots - 1u, k) < 0);
       }
       int total;
       const int rank = block_exclusive_scan<THREADS>(is_new ? 1 : 0, &total, scratch);
@@ -651,7 +653,7 @@ __global__ __launch_bounds__(THREADS) void svc_merge_sorted_kernel(const SvcArgs
   __syncthreads();
   for (int idx = e0 + (int)threadIdx.x; idx < e1; idx += THREADS) {
     const uint32_t c = (uint32_t)a.col_ind[idx];
-    atomicOr(&bits[c >> 5], 1u << (c & 31u));
+    if (c < (uint32_t)a.K) atomicOr(&bits[c >> 5], 1u << (c & 31u));  // (a column outside [0, K) is ignored)
   }
   __syncthreads();
   const int per = (words + THREADS - 1) / THREADS;
@@ -673,7 +675,7 @@ __global__ __launch_bounds__(THREADS) void svc_merge_sorted_kernel(const SvcArgs
   __syncthreads();
   for (int idx = e0 + (int)threadIdx.x; idx < e1; idx += THREADS) {
     const uint32_t c = (uint32_t)a.col_ind[idx];
-    a.pos[idx] = prefix[c >> 5] + __popc(bits[c >> 5] & ((1u << (c & 31u)) - 1u));
+    a.pos[idx] = c < (uint32_t)a.K ? prefix[c >> 5] + __popc(bits[c >> 5] & ((1u << (c & 31u)) - 1u)) : -1;
   }
 }
 
@@ -755,8 +757,10 @@ __global__ __launch_bounds__(THREADS) void svc_fill_kernel(const SvcArgs a, cons
   __syncthreads();
   for (int r = r0; r < r1; ++r) {
     const int b = a.row_ptr[r], e = a.row_ptr[r + 1];
-    for (int idx = b + (int)threadIdx.x; idx < e; idx += THREADS)
-      out[(int64_t)a.pos[idx] * a.V + (r - r0)] = csr_val[idx];
+    for (int idx = b + (int)threadIdx.x; idx < e; idx += THREADS) {
+      const int ps = a.pos[idx];
+      if (ps >= 0 && ps < n) out[(int64_t)ps * a.V + (r - r0)] = csr_val[idx];  // (-1: a column outside [0, K))
+    }
   }
 }
 

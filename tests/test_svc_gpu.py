@@ -145,6 +145,31 @@ def test_a_row_that_repeats_a_column_stays_inside_its_group(built_library):
     assert ((vcol >= 0) & (vcol < K)).all() and np.isin(vval, [0.0, 1.0]).all()
 
 
+@pytest.mark.parametrize("K,order", [(4096, "cpython"), (4096, "sorted"), (300000, "cpython")])
+def test_columns_outside_the_matrix_are_ignored(oracle, built_library, K, order):
+    """Invalid input (the contract wants 0 <= column < K): such non-zeros are dropped, nothing else changes, and
+    no kernel indexes a table with them.  The result is that of the matrix without them."""
+    rng = np.random.default_rng(80)
+    clean = _random_csr(rng, 96, K, 400)
+    rows = []
+    for r in range(clean.M):
+        c = clean.col_ind[clean.row_ptr[r]:clean.row_ptr[r + 1]]
+        bad = rng.choice([-1, -7, K, K + 5, 2**31 - 1, -2**31], size=rng.integers(0, 4)).astype(np.int64)
+        merged = np.concatenate([c.astype(np.int64), bad])
+        rng.shuffle(merged)
+        rows.append(merged)
+    lens = np.array([len(x) for x in rows])
+    ptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cols = np.concatenate(rows).astype(np.int32)
+    vals = rng.standard_normal(cols.size).astype(np.float16)
+    keep = (cols >= 0) & (cols < K)
+    kept_ptr = np.concatenate([[0], np.cumsum([keep[ptr[r]:ptr[r + 1]].sum() for r in range(len(rows))])]).astype(np.int32)
+    want = oracle.svc(len(rows), K, 8, kept_ptr, cols[keep], vals[keep], order=order)
+    vrp, vcol, vval, _ = gpu_svc(len(rows), K, 8, ptr, cols, vals, order)
+    assert np.array_equal(vrp, want[0]) and np.array_equal(vcol, want[1])
+    assert np.array_equal(vval.view(np.uint16), want[2].view(np.uint16))
+
+
 def test_calls_from_several_host_threads_on_their_own_streams(oracle, built_library):
     """The helper streams and events of the merge are per device: concurrent callers must not mix their
     fork / join sequences."""

@@ -271,6 +271,27 @@ def main():
             "alg_bytes": svc_bytes, "hbm_gbps": svc_bytes / svc_k_ms / 1e6,
         }
 
+        # the same pass on the shape of the matrices the reference's RowMerge is run on (its dataset of pruned
+        # transformer weights): 2048 x 2048, 90 % of the entries zero at random, V = 8 and 16
+        rng_d = np.random.default_rng(7)
+        mask_d = rng_d.random((2048, 2048)) < 0.1
+        d_ptr = np.concatenate([[0], np.cumsum(mask_d.sum(axis=1))]).astype(np.int32)
+        d_col = np.nonzero(mask_d)[1].astype(np.int32)
+        d_rp, d_ci = torch.from_numpy(d_ptr).cuda(), torch.from_numpy(d_col).cuda()
+        d_lists = O.csr_col_lists(2048, d_ptr, d_col)
+        for Vd in (8, 16):
+            rd = sspmm_amd.svc(d_rp, d_ci, None, 2048, 2048, Vd)
+            d_ms = time_launches(lambda: sspmm_amd.svc(d_rp, d_ci, None, 2048, 2048, Vd), 20, 3)
+            t0 = time.perf_counter()
+            d_want_ptr, d_want_cols = O.rowmerge_python(2048, Vd, d_lists)
+            d_py = (time.perf_counter() - t0) * 1e3
+            extra["svc_pruned_weight_2048x2048_s0.9_v%d" % Vd] = {
+                "gpu_ms_with_alloc_and_readback": d_ms, "python_rowmerge_ms": d_py, "speedup_vs_python": d_py / d_ms,
+                "bit_exact_vs_python": bool(rd.vec_row_ptr.cpu().numpy().tolist() == d_want_ptr and
+                                            rd.vec_col.cpu().numpy().tolist() == d_want_cols),
+                "nnz": int(d_col.size), "nvec": int(rd.num_vec),
+            }
+
         # ... and the SpMM that consumes it: the skewed pattern straight from the SVC, B 16384 x 256
         N4 = 256
         B4 = torch.from_numpy(synth.dense_rhs(csr.K, N4, seed=14)).cuda()

@@ -503,6 +503,24 @@ static constexpr int kSlabThreads = kSlabWaves * 64;
 // A slab is NQ tiles of 16 columns wide: 4 (64 columns, 128-byte rows) where K lets it fit in LDS, 2 (32 columns,
 // 64-byte rows) for matrices up to twice as tall.
 static constexpr int slab_row_bytes(int NQ) { return 32 * NQ; }
+// How a 64-column slab lies in LDS.  With 128-byte rows the 32-byte segments of a row are XOR-swizzled (see
+// slab_unit_dst) and every read address needs the swizzle applied in registers; where LDS allows, rows are padded
+// instead, which spreads the banks the same way and leaves the four tiles of a row at the immediate offsets
+// 0 / 32 / 64 / 96 of one address: a dozen vector-ALU instructions fewer per step, in a loop whose speed follows
+// its instruction count.  Padded and double-buffered, the rows of the two slabs alternate (A, B, 32 bytes of
+// padding: 288 bytes per row pair), which costs no more LDS than two unpadded slabs plus the padding.
+enum SlabLayout { kXorSingle = 0, kXorDouble = 1, kPadSingle = 2, kPadDouble = 3 };
+static constexpr bool layout_double(int L) { return L == kXorDouble || L == kPadDouble; }
+static constexpr bool layout_pad(int L) { return L == kPadSingle || L == kPadDouble; }
+static constexpr uint32_t layout_row_bytes(int L, int NQ) { return L == kPadSingle ? 160u : L == kPadDouble ? 288u : 32u * NQ; }
+// bytes of LDS taken by the slab(s), K rows and the zero row
+static constexpr uint32_t layout_slab_region(int L, int NQ, uint32_t rows) {
+  return rows * layout_row_bytes(L, NQ) * (L == kXorDouble ? 2u : 1u);
+}
+// offset of buffer `sel` (0 / 1) inside the region
+static constexpr uint32_t layout_buffer_off(int L, int NQ, uint32_t rows, uint32_t sel) {
+  return L == kPadDouble ? sel * 128u : sel * rows * layout_row_bytes(L, NQ);
+}
 // Per-wave LDS: the value tile of a step (32 vectors x V halfs; the V = 8 transpose read touches 16
 // bytes past its 512).
 static constexpr int wave_lds_bytes(int V) { return val_tile_bytes(V); }
@@ -738,7 +756,7 @@ struct SlabCtx {
 
 // One wave's share of a work item: the vector-rows wave, wave + 16, ... of the item's row table
 // against the slab at byte offset slab_base of LDS.
-template <int V, typename OutT, int NQ>
+template <int V, typename OutT, int NQ, int L>
 __device__ __forceinline__ void slab_process_item(const SlabCtx<V, OutT> &x, unsigned char *lds, uint32_t slab_base,
                                                   const SlabRows &rows, const uint16_t *vals,
                                                   __amdgpu_buffer_rsrc_t srd_c, const SlabStore<V, OutT, NQ> &out) {
@@ -761,7 +779,7 @@ __device__ __forceinline__ void slab_process_item(const SlabCtx<V, OutT> &x, uns
   // the value tile of the first step
   *reinterpret_cast<typename SlabVals<V>::type *>(x.val_dst) = ld[0].vraw;
 
-  const uint32_t lane_base = x.b_lane_off + slab_base + lds_address(lds);  // slab_base is a multiple of 128, and so is the LDS base
+  const uint32_t lane_base = x.b_lane_off + slab_base + lds_address(lds);  // slab_base is a multiple of 32 (128 for swizzled rows), the LDS base of 128
   // Accumulators are cleared by an MFMA of two zero operands: four instructions on the otherwise
   // idle matrix pipe instead of sixteen register moves on the vector ALU, which the loop saturates.
   Half8Bits zero_op;
@@ -792,13 +810,16 @@ __device__ __forceinline__ void slab_process_item(const SlabCtx<V, OutT> &x, uns
       for (int h = 0; h < 2; ++h) {
         const uint32_t c = ((int)x.slot0 + 4 * h < left) ? ld[cur].col[h] : x.zero_row;
         // row c of the slab, and the swizzle of its 32-byte segments (see slab_unit_dst)
-        addr[h] = NQ == 4 ? (((c << 7) + lane_base) | ((c << 4) & 0x60u)) : (((c << 6) + lane_base) | ((c << 3) & 0x20u));
+        addr[h] = layout_pad(L) ? __umul24(c, layout_row_bytes(L, NQ)) + lane_base
+                  : NQ == 4     ? (((c << 7) + lane_base) | ((c << 4) & 0x60u))
+                                : (((c << 6) + lane_base) | ((c << 3) & 0x20u));
       }
       Half8Bits b[NQ];
 #pragma unroll
       for (int q = 0; q < NQ; ++q) {
-        const uintx2 lo = lds_read_tr_abs(addr[0] ^ ((uint32_t)q << 5));
-        const uintx2 hi = lds_read_tr_abs(addr[1] ^ ((uint32_t)q << 5));
+        // (padded rows: an immediate offset of the read; swizzled rows: the segment index XORed in)
+        const uintx2 lo = layout_pad(L) ? lds_read_tr_abs(addr[0] + ((uint32_t)q << 5)) : lds_read_tr_abs(addr[0] ^ ((uint32_t)q << 5));
+        const uintx2 hi = layout_pad(L) ? lds_read_tr_abs(addr[1] + ((uint32_t)q << 5)) : lds_read_tr_abs(addr[1] ^ ((uint32_t)q << 5));
         b[q].u[0] = lo[0]; b[q].u[1] = lo[1]; b[q].u[2] = hi[0]; b[q].u[3] = hi[1];
       }
       // the next step's value tile goes to LDS behind the reads above (LDS operations of a wave
@@ -859,10 +880,11 @@ __device__ __forceinline__ uint32_t slab_unit_src(const SpmmArgs &p, uint32_t u,
 // A 16-lane group of a slab read touches four rows at the same segment; rows 256 bytes apart share banks, so the
 // segment index is XORed with the row bits above that distance: (c >> 1) & 3 for 128-byte rows, (c >> 2) & 1 for
 // 64-byte rows.  Rows then collide only when they agree modulo 8.
-template <int NQ>
+template <int NQ, int L>
 __device__ __forceinline__ uint32_t slab_unit_dst(uint32_t u) {
   constexpr uint32_t kPerRow = 2u * NQ;
   const uint32_t c = u / kPerRow;
+  if (layout_pad(L)) return c * layout_row_bytes(L, NQ) + (u % kPerRow) * 16u;
   const uint32_t swz = NQ == 4 ? ((c >> 1) & 3u) : ((c >> 2) & 1u);
   return c * slab_row_bytes(NQ) + (((u % kPerRow) * 16u) ^ (swz << 5));
 }
@@ -880,7 +902,7 @@ __device__ __forceinline__ intx4 slab_table_fetch(const SpmmArgs &p, const int32
   return e;
 }
 
-template <int V, typename OutT, bool DOUBLE, int NQ>
+template <int V, typename OutT, int L, int NQ>
 __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs p,
                                                                  const int32_t *__restrict__ row_offsets,
                                                                  const int32_t *__restrict__ row_indices) {
@@ -896,18 +918,22 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
   const int tid = threadIdx.x, lane = tid & 63, m = lane & 15, g = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // tell the compiler it is wave-uniform
   const uint32_t b_bytes = (uint32_t)p.K * (uint32_t)p.N * 2u;
-  constexpr uint32_t kSlabRowBytes = slab_row_bytes(NQ);
+  constexpr bool DOUBLE = layout_double(L);
+  constexpr bool ONE_TABLE = L == kPadDouble;  // (what fits beside the padded pair of slabs)
+  static_assert(!layout_pad(L) || NQ == 4, "padded rows are for the 64-column slab");
+  constexpr uint32_t kSlabRowBytes = layout_row_bytes(L, NQ);
   const uint32_t units = (uint32_t)p.K * (2u * NQ);
 
-  // ---- LDS: slab 0, [slab 1], value tiles, row table 0, row table 1
+  // ---- LDS: slab 0, [slab 1] (their rows alternating when padded), value tiles, row table 0, [row table 1]
   const uint32_t zero_row = (uint32_t)p.K;
-  const uint32_t slab_bytes = (zero_row + 1u) * kSlabRowBytes;
-  const uint32_t tiles_off = slab_bytes * (DOUBLE ? 2u : 1u);
+  const uint32_t tiles_off = layout_slab_region(L, NQ, zero_row + 1u);
   const uint32_t table_off = tiles_off + kSlabWaves * wave_lds_bytes(V);
   const uint32_t table_bytes = (p.rows_per_block + 1u) * 16u;
   if (tid < 2 * NQ) {
     *reinterpret_cast<uintx4 *>(lds + zero_row * kSlabRowBytes + tid * 16) = uintx4{0u, 0u, 0u, 0u};
-    if (DOUBLE) *reinterpret_cast<uintx4 *>(lds + slab_bytes + zero_row * kSlabRowBytes + tid * 16) = uintx4{0u, 0u, 0u, 0u};
+    if (DOUBLE)
+      *reinterpret_cast<uintx4 *>(lds + layout_buffer_off(L, NQ, zero_row + 1u, 1u) + zero_row * kSlabRowBytes + tid * 16) =
+          uintx4{0u, 0u, 0u, 0u};
   }
 
   SlabCtx<V, OutT> x;
@@ -939,7 +965,7 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const uint32_t u = u0 + i * kSlabThreads + tid;
-        if (u < units) *reinterpret_cast<uintx4 *>(lds + slab_unit_dst<NQ>(u)) = d[i];
+        if (u < units) *reinterpret_cast<uintx4 *>(lds + slab_unit_dst<NQ, L>(u)) = d[i];
       }
     }
     if ((uint32_t)tid <= p.rows_per_block) *reinterpret_cast<intx4 *>(lds + table_off + tid * 16) = e;
@@ -980,7 +1006,7 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
       // One buffer descriptor spans this batch element's C (the launcher checks it is below 4 GiB).
       const __amdgpu_buffer_rsrc_t srd_c = make_srd(reinterpret_cast<OutT *>(p.C) + (int64_t)cur.batch * p.stride_C,
                                                     (uint32_t)p.m_vec * x.c_vrow_bytes);
-      slab_process_item<V, OutT, NQ>(x, lds, slab_sel * slab_bytes, rows, p.values + (int64_t)cur.batch * p.stride_values,
+      slab_process_item<V, OutT, NQ, L>(x, lds, layout_buffer_off(L, NQ, zero_row + 1u, slab_sel), rows, p.values + (int64_t)cur.batch * p.stride_values,
                                  srd_c, out);
     }
     if (!has_next) break;
@@ -994,10 +1020,15 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
 #pragma unroll
         for (int i = 0; i < kSlabFetchUnits; ++i) {
           const uint32_t u = i * kSlabThreads + ctid;
-          if (u < units) *reinterpret_cast<uintx4 *>(lds + slab_sel * slab_bytes + slab_unit_dst<NQ>(u)) = f.d[i];
+          if (u < units)
+            *reinterpret_cast<uintx4 *>(lds + layout_buffer_off(L, NQ, zero_row + 1u, slab_sel) + slab_unit_dst<NQ, L>(u)) = f.d[i];
         }
       }
-      table_sel ^= 1u;
+      if (ONE_TABLE) {
+        __syncthreads();  // every wave is done with the table
+      } else {
+        table_sel ^= 1u;
+      }
       if ((uint32_t)ctid <= p.rows_per_block) *reinterpret_cast<intx4 *>(lds + table_off + table_sel * table_bytes + ctid * 16) = f.entry;
       __syncthreads();
     } else {
@@ -1014,7 +1045,7 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const uint32_t u = u0 + i * kSlabThreads + ctid;
-            if (u < units) *reinterpret_cast<uintx4 *>(lds + slab_unit_dst<NQ>(u)) = d[i];
+            if (u < units) *reinterpret_cast<uintx4 *>(lds + slab_unit_dst<NQ, L>(u)) = d[i];
           }
         }
       }
@@ -1071,11 +1102,12 @@ static constexpr uint32_t kSlabMaxRows = 512;  // vector-rows per work item (one
 static constexpr uint32_t kSlabMinRows = 32;   // keeps the copy of the slab a small part of an item's traffic
 
 // LDS bytes of a workgroup: slabs (+ zero rows), value tiles, two row tables.
-static uint32_t slab_lds_bytes(int K, int V, uint32_t rows, bool dbl, int NQ) {
-  return (uint32_t)(K + 1) * slab_row_bytes(NQ) * (dbl ? 2u : 1u) + kSlabWaves * wave_lds_bytes(V) + 2u * 16u * (rows + 1u);
+static uint32_t slab_lds_bytes(int K, int V, uint32_t rows, int layout, int NQ) {
+  return layout_slab_region(layout, NQ, (uint32_t)K + 1u) + kSlabWaves * wave_lds_bytes(V) +
+         (layout == kPadDouble ? 1u : 2u) * 16u * (rows + 1u);
 }
 // Largest K the slab kernel takes (one slab, smallest row tables).
-static bool slab_fits(int K, int V, int NQ) { return slab_lds_bytes(K, V, kSlabMinRows, false, NQ) <= kSlabLds; }
+static bool slab_fits(int K, int V, int NQ) { return slab_lds_bytes(K, V, kSlabMinRows, kXorSingle, NQ) <= kSlabLds; }
 
 static constexpr int kMaxDevices = 64;
 static int current_device() {
@@ -1095,9 +1127,9 @@ static uint32_t device_cus() {  // of the current device
   return cus[dev];
 }
 
-template <int V, typename OutT, bool DOUBLE, int NQ>
+template <int V, typename OutT, int L, int NQ>
 static hipError_t launch_slab_kernel(const SpmmArgs &p, uint32_t grid, uint32_t lds, hipStream_t stream) {
-  auto kern = spmm_slab_kernel<V, OutT, DOUBLE, NQ>;
+  auto kern = spmm_slab_kernel<V, OutT, L, NQ>;
   static bool raised[kMaxDevices] = {};  // per instantiation and device
   const int dev = current_device();
   if (!raised[dev]) {
@@ -1125,13 +1157,25 @@ static hipError_t launch_slab(const SpmmArgs &a, hipStream_t stream) {
   if (row_blocks > max_blocks) row_blocks = max_blocks;
   if (row_blocks < min_blocks) row_blocks = min_blocks;
   uint32_t rows = ((uint32_t)a.m_vec + row_blocks - 1u) / row_blocks;
-  bool dbl = (uint32_t)a.K * (2u * NQ) <= (uint32_t)kSlabFetchUnits * kSlabThreads && slab_lds_bytes(a.K, V, rows, true, NQ) <= kSlabLds;
-  while (!dbl && slab_lds_bytes(a.K, V, rows, false, NQ) > kSlabLds && rows > kSlabMinRows) rows = (rows + 1u) / 2u;  // smaller tables for a tall slab
+  // Layout: double-buffered where the next slab fits into the registers of one fetch and both slabs into LDS,
+  // padded rows where they fit (64-column slabs only).
+  const bool can_dbl = (uint32_t)a.K * (2u * NQ) <= (uint32_t)kSlabFetchUnits * kSlabThreads;
+  int layout = kXorSingle;
+  if (NQ == 4 && can_dbl && slab_lds_bytes(a.K, V, rows, kPadDouble, NQ) <= kSlabLds) layout = kPadDouble;
+  else if (can_dbl && slab_lds_bytes(a.K, V, rows, kXorDouble, NQ) <= kSlabLds) layout = kXorDouble;
+  else if (NQ == 4 && slab_lds_bytes(a.K, V, rows, kPadSingle, NQ) <= kSlabLds) layout = kPadSingle;
+  while (layout == kXorSingle && slab_lds_bytes(a.K, V, rows, kXorSingle, NQ) > kSlabLds && rows > kSlabMinRows)
+    rows = (rows + 1u) / 2u;  // smaller tables for a tall slab
   p.rows_per_block = rows;
   p.row_blocks = ((uint32_t)a.m_vec + rows - 1u) / rows;
-  const uint32_t lds = slab_lds_bytes(a.K, V, rows, dbl, NQ);
+  const uint32_t lds = slab_lds_bytes(a.K, V, rows, layout, NQ);
   const uint32_t grid = 8u * wgs_per_xcd;
-  return dbl ? launch_slab_kernel<V, OutT, true, NQ>(p, grid, lds, stream) : launch_slab_kernel<V, OutT, false, NQ>(p, grid, lds, stream);
+  if (NQ == 4) {
+    if (layout == kPadDouble) return launch_slab_kernel<V, OutT, kPadDouble, 4>(p, grid, lds, stream);
+    if (layout == kPadSingle) return launch_slab_kernel<V, OutT, kPadSingle, 4>(p, grid, lds, stream);
+  }
+  return layout == kXorDouble ? launch_slab_kernel<V, OutT, kXorDouble, NQ>(p, grid, lds, stream)
+                              : launch_slab_kernel<V, OutT, kXorSingle, NQ>(p, grid, lds, stream);
 }
 
 template <int V, typename OutT>

@@ -301,10 +301,14 @@ def test_slab_kernel_work_item_lists(oracle, built_library, V, batch, m_rows, K,
 
 @pytest.mark.parametrize("V,K,expect", [(8, 574, 3), (8, 575, 3), (16, 512, 3), (16, 543, 3), (16, 544, 3), (8, 1150, 3),
                                         (16, 1100, 3), (8, 1300, 5), (16, 1024, 3), (8, 1025, 3), (16, 2286, 5),
-                                        (16, 2287, 2), (8, 2410, 5), (8, 2411, 2)])
+                                        (16, 2287, 2), (8, 2410, 5), (8, 2411, 2),
+                                        # padded rows: both slabs (K <= 512, and <= 506 for V = 16), one slab (to about 950 / 900)
+                                        (8, 512, 3), (8, 513, 3), (16, 506, 3), (16, 507, 3), (8, 950, 3), (8, 960, 3),
+                                        (16, 900, 3), (16, 910, 3)])
 def test_slab_kernel_around_its_lds_limits(oracle, built_library, V, K, expect):
-    """K just below and above what two slabs (then one slab) leave room for in LDS, for the 64-column slab and,
-    above its limit, for the 32-column one; beyond that the forced choice falls back to the gather kernel."""
+    """K just below and above what two slabs (then one slab) leave room for in LDS, with padded and with swizzled
+    rows, for the 64-column slab and, above its limit, for the 32-column one; beyond that the forced choice falls
+    back to the gather kernel."""
     from sspmm_amd import _lib
     vs = synth.vector_sparse(80 * V, K, V, 0.95, seed=K)
     B = synth.dense_rhs(K, 192, seed=K + 1)

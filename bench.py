@@ -29,7 +29,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch of the headline workload at the default batch of 128, from hardware counters
 # (FETCH_SIZE and WRITE_SIZE, each scaled by its reading for a 256 MiB device copy): see
 # profiles/spmm_slab_v8_f32_cfg2_batch128_hbm_traffic.txt.  Other batch sizes report null.
-MEASURED_TRAFFIC_BYTES = {128: 66.5e6 + 268.4e6}
+MEASURED_TRAFFIC_BYTES = {128: 66.3e6 + 268.4e6}
 
 
 def parse_args():

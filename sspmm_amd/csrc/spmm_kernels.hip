@@ -632,8 +632,10 @@ template <int V, int NQ>
 struct SlabStore<V, float, NQ> {
   uint32_t voff[V / 8];                 // byte offset of the lane's 16 bytes for tile pair 0, per row half
   int col[V / 8];                       // its first column
+  bool full;                            // (wave-uniform) the whole tile lies inside N: no lane needs masking
   __device__ __forceinline__ void init(int lane, int n0, int N) {
     const int m = lane & 15, g = lane >> 4;
+    full = n0 + 16 * NQ <= N;
 #pragma unroll
     for (int h = 0; h < V / 8; ++h) {
       const int row = 8 * h + (m & 7);
@@ -655,7 +657,9 @@ struct SlabStore<V, float, NQ> {
           const uint32_t x = __builtin_bit_cast(uint32_t, fx), y = __builtin_bit_cast(uint32_t, fy);
           line[r] = h == 0 ? dpp_from_m_minus_8(x, y) : dpp_from_m_plus_8(x, y);
         }
-        if (col[h] + 32 * qp < N) slab_store_line(line, srd, voff[h] + 128u * qp, crow);
+        // (the common case without the save / restore of the execution mask that a per-lane condition costs)
+        if (full) slab_store_line(line, srd, voff[h] + 128u * qp, crow);
+        else if (col[h] + 32 * qp < N) slab_store_line(line, srd, voff[h] + 128u * qp, crow);
       }
     }
   }
@@ -665,8 +669,10 @@ template <int V>
 struct SlabStore<V, _Float16, 4> {
   uint32_t voff[V / 8];
   int col[V / 8];
+  bool full;
   __device__ __forceinline__ void init(int lane, int n0, int N) {
     const int m = lane & 15, g = lane >> 4;
+    full = n0 + 64 <= N;
 #pragma unroll
     for (int h = 0; h < V / 8; ++h) {
       const int row = 8 * h + (m & 7);
@@ -704,7 +710,8 @@ struct SlabStore<V, _Float16, 4> {
 #pragma unroll
       for (int r = 0; r < 4; ++r)
         line[r] = h == 0 ? dpp_from_m_minus_8(pr[0][r], pr[1][r]) : dpp_from_m_plus_8(pr[0][r], pr[1][r]);
-      if (col[h] < N) slab_store_line(line, srd, voff[h], crow);
+      if (full) slab_store_line(line, srd, voff[h], crow);
+      else if (col[h] < N) slab_store_line(line, srd, voff[h], crow);
     }
   }
 };
@@ -823,8 +830,8 @@ __device__ __forceinline__ void slab_process_item(const SlabCtx<V, OutT> &x, uns
         b[q].u[0] = lo[0]; b[q].u[1] = lo[1]; b[q].u[2] = hi[0]; b[q].u[3] = hi[1];
       }
       // the next step's value tile goes to LDS behind the reads above (LDS operations of a wave
-      // execute in order)
-      if (ld[nxt].valid) *reinterpret_cast<typename SlabVals<V>::type *>(x.val_dst) = ld[nxt].vraw;
+      // execute in order; unconditionally: after the last step it is zeros that nobody reads)
+      *reinterpret_cast<typename SlabVals<V>::type *>(x.val_dst) = ld[nxt].vraw;
 
 #pragma unroll
       for (int q = 0; q < NQ; ++q) acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[q].h, a.h, acc[q], 0, 0, 0);

@@ -495,7 +495,7 @@ __global__ __launch_bounds__(64 * kSplitWaves) void spmm_gather_split_kernel(con
 // and 4 MFMAs, with no byte shuffling in registers.  A 16-lane group of a slab read touches four
 // different rows of B at the same column offset; the 32-byte segments of slab row c are stored
 // XOR-swizzled by (c >> 1) & 3 so that those rows spread over the LDS banks.
-// The vector-rows of a row block are dealt to the waves round-robin, and the loads of a step are
+// The waves claim the vector-rows of a row block one at a time, and the loads of a step are
 // issued a few steps ahead (across vector-row boundaries).  Row K of the slab is all
 // zeros: unused k slots of a partial step point there.
 static constexpr int kSlabWaves = 16;
@@ -538,33 +538,44 @@ struct SlabLoads {    // what the head records for a step; the step consumes it 
 };
 
 // Walks one wave's sequence of steps.  The (vector-row, first vector, end vector) triples of the
-// row block are copied into a table in LDS when the workgroup starts; wave w takes the positions
-// w, w + 8, w + 16, ... of the block, so finding the next vector-row is one broadcast LDS read and
-// no scalar-memory or atomic round trip sits in the main loop.  A vector-row of n vectors is
-// ceil(n / 32) steps, and an empty vector-row is one step without vectors (its zeros still have
-// to be written).  The cursor runs slab_ring(V) - 1 steps ahead of the arithmetic: it issues the
-// loads of a step and records the step's vector-row and length in the ring slot that receives
-// them.  It reads the table entry of its following vector-row one row ahead, so that the LDS
-// latency is off the critical path.
+// row block are copied into a table in LDS when the workgroup starts, and the waves claim its
+// positions one at a time from a counter in LDS: the waves of a workgroup do not run at the same
+// speed (the older waves of a SIMD win the arbitration for the memory pipeline, and finish a
+// fixed share of rows a third sooner than the younger ones), so a fixed deal of rows would leave
+// the fast waves idle at the end of every item.  A vector-row of n vectors is ceil(n / 32) steps,
+// and an empty vector-row is one step without vectors (its zeros still have to be written).  The
+// cursor runs slab_ring(V) - 1 steps ahead of the arithmetic: it issues the loads of a step and
+// records the step's vector-row and length in the ring slot that receives them.  Both LDS round
+// trips behind a new row are off the critical path: the claim of a position is issued two rows
+// ahead and the read of its table entry one row ahead.
 typedef int intx4 __attribute__((ext_vector_type(4)));
 struct SlabCursor {
   int row, kc, end;  // current step: vectors [kc, min(kc + 32, end)) of vector-row `row`
   int valid;  // flags are ints: wave-uniform 0 / 1 that stay in scalar registers
   intx4 next;        // table entry of the following vector-row (still in vector registers)
   int next_valid;
-  int count;         // rows requested so far
+  int claim;         // what the counter returned for the row after that (still in a vector register)
 };
 
 struct SlabRows {      // what the cursors need to find rows
   const intx4 *table;  // LDS: n_rows entries (row, first vector, end vector, -) and an all-zero entry behind them
-  int n_rows, wave;
+  int *counter;        // LDS: the number of positions claimed so far (the spare word of the table's last entry)
+  int n_rows, lane;
 };
 
+// Lane 0 takes the next position (the append instruction that would do it for a whole wave addresses only the
+// first 64 KB of LDS, and the tables lie above that).
+__device__ __forceinline__ int cursor_claim(const SlabRows &rows) {
+  int t = 0;
+  if (rows.lane == 0) t = __hip_atomic_fetch_add(rows.counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  return t;
+}
+
 __device__ __forceinline__ void cursor_prefetch(SlabCursor &c, const SlabRows &rows) {
-  const int idx = rows.wave + kSlabWaves * c.count;
-  ++c.count;
+  const int idx = __builtin_amdgcn_readfirstlane(c.claim);
   c.next_valid = idx < rows.n_rows ? 1 : 0;
   c.next = rows.table[min(idx, rows.n_rows)];
+  c.claim = cursor_claim(rows);
 }
 
 __device__ __forceinline__ void cursor_take_next(SlabCursor &c, const SlabRows &rows) {
@@ -761,14 +772,14 @@ struct SlabCtx {
   uint32_t c_vrow_bytes;
 };
 
-// One wave's share of a work item: the vector-rows wave, wave + 16, ... of the item's row table
+// One wave's share of a work item: the vector-rows it claims from the item's row table,
 // against the slab at byte offset slab_base of LDS.
 template <int V, typename OutT, int NQ, int L>
 __device__ __forceinline__ void slab_process_item(const SlabCtx<V, OutT> &x, unsigned char *lds, uint32_t slab_base,
                                                   const SlabRows &rows, const uint16_t *vals,
                                                   __amdgpu_buffer_rsrc_t srd_c, const SlabStore<V, OutT, NQ> &out) {
   SlabCursor head;  // issues loads
-  head.count = 0;
+  head.claim = cursor_claim(rows);
   cursor_prefetch(head, rows);
   cursor_take_next(head, rows);
   if (!head.valid) return;
@@ -1007,7 +1018,9 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
       SlabRows rows;
       rows.table = reinterpret_cast<const intx4 *>(lds + table_off + table_sel * table_bytes);
       rows.n_rows = min(p.m_vec, row_lo + (int)p.rows_per_block) - row_lo;
-      rows.wave = wave;
+      // (the entry at rows_per_block is rewritten, all zeros, with every table)
+      rows.counter = reinterpret_cast<int *>(lds + table_off + table_sel * table_bytes + p.rows_per_block * 16u + 12u);
+      rows.lane = lane;
       SlabStore<V, OutT, NQ> out;
       out.init(lane, (int)cur.tile * (16 * NQ), p.N);
       // One buffer descriptor spans this batch element's C (the launcher checks it is below 4 GiB).

@@ -553,36 +553,35 @@ struct SlabCursor {
   int row, kc, end;  // current step: vectors [kc, min(kc + 32, end)) of vector-row `row`
   int valid;  // flags are ints: wave-uniform 0 / 1 that stay in scalar registers
   intx4 next;        // table entry of the following vector-row (still in vector registers)
-  int next_valid;
   int claim;         // what the counter returned for the row after that (still in a vector register)
 };
 
 struct SlabRows {      // what the cursors need to find rows
-  const intx4 *table;  // LDS: n_rows entries (row, first vector, end vector, -) and an all-zero entry behind them
-  int *counter;        // LDS: the number of positions claimed so far (the spare word of the table's last entry)
+  const intx4 *table;  // LDS: n_rows entries (row, first vector, end vector, 1) and an all-zero entry behind them
+  int *counter;        // LDS: the number of positions claimed so far (in the entry behind the table's last)
   int n_rows, lane;
 };
 
 // Lane 0 takes the next position (the append instruction that would do it for a whole wave addresses only the
 // first 64 KB of LDS, and the tables lie above that).
-__device__ __forceinline__ int cursor_claim(const SlabRows &rows) {
-  int t = 0;
+// (`spent` is a value the caller no longer needs: what the other lanes return, so that no register has to be cleared)
+__device__ __forceinline__ int cursor_claim(const SlabRows &rows, int spent) {
+  int t = spent;
   if (rows.lane == 0) t = __hip_atomic_fetch_add(rows.counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   return t;
 }
 
 __device__ __forceinline__ void cursor_prefetch(SlabCursor &c, const SlabRows &rows) {
   const int idx = __builtin_amdgcn_readfirstlane(c.claim);
-  c.next_valid = idx < rows.n_rows ? 1 : 0;
-  c.next = rows.table[min(idx, rows.n_rows)];
-  c.claim = cursor_claim(rows);
+  c.next = rows.table[min(idx, rows.n_rows)];  // positions beyond the block read the all-zero entry: not valid
+  c.claim = cursor_claim(rows, c.claim);
 }
 
 __device__ __forceinline__ void cursor_take_next(SlabCursor &c, const SlabRows &rows) {
   c.row = __builtin_amdgcn_readfirstlane(c.next[0]);
   c.kc = __builtin_amdgcn_readfirstlane(c.next[1]);
   c.end = __builtin_amdgcn_readfirstlane(c.next[2]);
-  c.valid = c.next_valid;
+  c.valid = __builtin_amdgcn_readfirstlane(c.next[3]);
   cursor_prefetch(c, rows);
 }
 
@@ -631,6 +630,10 @@ __device__ __forceinline__ void slab_store_line(uintx4 line, __amdgpu_buffer_rsr
 //     gathers all four tiles of a row into one instruction.
 template <int V, typename OutT, int NQ>
 struct SlabStore;
+// Lanes whose columns lie beyond N carry this offset instead of a mask: it is outside every buffer the kernel is
+// launched on (C of one batch element is at most 2 GiB), and the hardware drops stores outside the buffer.  The
+// stores of a tile then need no branch and no change of the execution mask.
+static constexpr uint32_t kSlabDropStore = 0x80000000u;
 
 __device__ __forceinline__ uint32_t dpp_from_m_minus_8(uint32_t keep, uint32_t src) {  // lanes m >= 8 take src of lane m - 8
   return (uint32_t)__builtin_amdgcn_update_dpp((int)keep, (int)src, 0x118, 0xf, 0xc, false);
@@ -641,21 +644,21 @@ __device__ __forceinline__ uint32_t dpp_from_m_plus_8(uint32_t keep, uint32_t sr
 
 template <int V, int NQ>
 struct SlabStore<V, float, NQ> {
-  uint32_t voff[V / 8];                 // byte offset of the lane's 16 bytes for tile pair 0, per row half
-  int col[V / 8];                       // its first column
-  bool full;                            // (wave-uniform) the whole tile lies inside N: no lane needs masking
+  uint32_t voff[V / 8][NQ / 2];         // byte offset of the lane's 16 bytes per row half and tile pair
   __device__ __forceinline__ void init(int lane, int n0, int N) {
     const int m = lane & 15, g = lane >> 4;
-    full = n0 + 16 * NQ <= N;
 #pragma unroll
     for (int h = 0; h < V / 8; ++h) {
       const int row = 8 * h + (m & 7);
       const int tile = h == 0 ? (m >> 3) : 1 - (m >> 3);
-      col[h] = n0 + 16 * tile + 4 * g;
-      voff[h] = ((uint32_t)row * (uint32_t)N + (uint32_t)col[h]) * 4u;
+#pragma unroll
+      for (int qp = 0; qp < NQ / 2; ++qp) {
+        const int col = n0 + 32 * qp + 16 * tile + 4 * g;
+        voff[h][qp] = col < N ? ((uint32_t)row * (uint32_t)N + (uint32_t)col) * 4u : kSlabDropStore;
+      }
     }
   }
-  __device__ __forceinline__ void store(const floatx4 (&acc)[NQ], __amdgpu_buffer_rsrc_t srd, uint32_t crow, int N) const {
+  __device__ __forceinline__ void store(const floatx4 (&acc)[NQ], __amdgpu_buffer_rsrc_t srd, uint32_t crow) const {
 #pragma unroll
     for (int qp = 0; qp < NQ / 2; ++qp) {
 #pragma unroll
@@ -668,9 +671,7 @@ struct SlabStore<V, float, NQ> {
           const uint32_t x = __builtin_bit_cast(uint32_t, fx), y = __builtin_bit_cast(uint32_t, fy);
           line[r] = h == 0 ? dpp_from_m_minus_8(x, y) : dpp_from_m_plus_8(x, y);
         }
-        // (the common case without the save / restore of the execution mask that a per-lane condition costs)
-        if (full) slab_store_line(line, srd, voff[h] + 128u * qp, crow);
-        else if (col[h] + 32 * qp < N) slab_store_line(line, srd, voff[h] + 128u * qp, crow);
+        slab_store_line(line, srd, voff[h][qp], crow);
       }
     }
   }
@@ -679,20 +680,17 @@ struct SlabStore<V, float, NQ> {
 template <int V>
 struct SlabStore<V, _Float16, 4> {
   uint32_t voff[V / 8];
-  int col[V / 8];
-  bool full;
   __device__ __forceinline__ void init(int lane, int n0, int N) {
     const int m = lane & 15, g = lane >> 4;
-    full = n0 + 64 <= N;
 #pragma unroll
     for (int h = 0; h < V / 8; ++h) {
       const int row = 8 * h + (m & 7);
       const int pair = h == 0 ? (m >> 3) : 1 - (m >> 3);
-      col[h] = n0 + 32 * pair + 16 * (g & 1) + 8 * (g >> 1);
-      voff[h] = ((uint32_t)row * (uint32_t)N + (uint32_t)col[h]) * 2u;
+      const int col = n0 + 32 * pair + 16 * (g & 1) + 8 * (g >> 1);
+      voff[h] = col < N ? ((uint32_t)row * (uint32_t)N + (uint32_t)col) * 2u : kSlabDropStore;
     }
   }
-  __device__ __forceinline__ void store(const floatx4 (&acc)[4], __amdgpu_buffer_rsrc_t srd, uint32_t crow, int N) const {
+  __device__ __forceinline__ void store(const floatx4 (&acc)[4], __amdgpu_buffer_rsrc_t srd, uint32_t crow) const {
     // pr[pair][0..3]: after the swaps, lane (m, g) holds columns 8 * (g >> 1) .. + 7 of tile
     // 2 * pair + (g & 1), row m
     uint32_t pr[2][4];
@@ -721,8 +719,7 @@ struct SlabStore<V, _Float16, 4> {
 #pragma unroll
       for (int r = 0; r < 4; ++r)
         line[r] = h == 0 ? dpp_from_m_minus_8(pr[0][r], pr[1][r]) : dpp_from_m_plus_8(pr[0][r], pr[1][r]);
-      if (full) slab_store_line(line, srd, voff[h], crow);
-      else if (col[h] < N) slab_store_line(line, srd, voff[h], crow);
+      slab_store_line(line, srd, voff[h], crow);
     }
   }
 };
@@ -732,15 +729,12 @@ struct SlabStore<V, _Float16, 4> {
 template <int V>
 struct SlabStore<V, _Float16, 2> {
   uint32_t voff;
-  int col;
-  bool row_ok;
   __device__ __forceinline__ void init(int lane, int n0, int N) {
     const int m = lane & 15, g = lane >> 4;
-    col = n0 + 16 * (g & 1) + 8 * (g >> 1);
-    voff = ((uint32_t)m * (uint32_t)N + (uint32_t)col) * 2u;
-    row_ok = m < V;
+    const int col = n0 + 16 * (g & 1) + 8 * (g >> 1);
+    voff = (m < V && col < N) ? ((uint32_t)m * (uint32_t)N + (uint32_t)col) * 2u : kSlabDropStore;
   }
-  __device__ __forceinline__ void store(const floatx4 (&acc)[2], __amdgpu_buffer_rsrc_t srd, uint32_t crow, int N) const {
+  __device__ __forceinline__ void store(const floatx4 (&acc)[2], __amdgpu_buffer_rsrc_t srd, uint32_t crow) const {
     uint32_t pk[2][2];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
@@ -757,7 +751,7 @@ struct SlabStore<V, _Float16, 2> {
       line[w] = sw[0];
       line[2 + w] = sw[1];
     }
-    if (row_ok && col < N) slab_store_line(line, srd, voff, crow);
+    slab_store_line(line, srd, voff, crow);
   }
 };
 
@@ -768,7 +762,6 @@ struct SlabCtx {
   uint32_t slot0, a_off, b_lane_off, zero_row;
   unsigned char *val_tile, *val_dst;
   __amdgpu_buffer_rsrc_t srd_cols;
-  int N;
   uint32_t c_vrow_bytes;
 };
 
@@ -779,7 +772,7 @@ __device__ __forceinline__ void slab_process_item(const SlabCtx<V, OutT> &x, uns
                                                   const SlabRows &rows, const uint16_t *vals,
                                                   __amdgpu_buffer_rsrc_t srd_c, const SlabStore<V, OutT, NQ> &out) {
   SlabCursor head;  // issues loads
-  head.claim = cursor_claim(rows);
+  head.claim = cursor_claim(rows, 0);
   cursor_prefetch(head, rows);
   cursor_take_next(head, rows);
   if (!head.valid) return;
@@ -847,7 +840,7 @@ __device__ __forceinline__ void slab_process_item(const SlabCtx<V, OutT> &x, uns
 #pragma unroll
       for (int q = 0; q < NQ; ++q) acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b[q].h, a.h, acc[q], 0, 0, 0);
       if (left <= 32) {  // last step of the vector-row: write its V x 64 tile of C and start over from zero
-        out.store(acc, srd_c, (uint32_t)ld[cur].row * x.c_vrow_bytes, x.N);
+        out.store(acc, srd_c, (uint32_t)ld[cur].row * x.c_vrow_bytes);
 #pragma unroll
         for (int q = 0; q < NQ; ++q) acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(zero_op.h, zero_op.h, zero_c, 0, 0, 0);
       }
@@ -916,6 +909,7 @@ __device__ __forceinline__ intx4 slab_table_fetch(const SpmmArgs &p, const int32
     e[0] = row_indices ? row_indices[row_lo + tid] : row_lo + tid;
     e[1] = row_offsets[e[0]];
     e[2] = row_offsets[e[0] + 1];
+    e[3] = 1;
   }
   return e;
 }
@@ -946,7 +940,7 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
   const uint32_t zero_row = (uint32_t)p.K;
   const uint32_t tiles_off = layout_slab_region(L, NQ, zero_row + 1u);
   const uint32_t table_off = tiles_off + kSlabWaves * wave_lds_bytes(V);
-  const uint32_t table_bytes = (p.rows_per_block + 1u) * 16u;
+  const uint32_t table_bytes = (p.rows_per_block + 2u) * 16u;
   if (tid < 2 * NQ) {
     *reinterpret_cast<uintx4 *>(lds + zero_row * kSlabRowBytes + tid * 16) = uintx4{0u, 0u, 0u, 0u};
     if (DOUBLE)
@@ -964,7 +958,6 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
   x.slot0 = (uint32_t)(8 * g + (m >> 2));
   x.b_lane_off = (uint32_t)(m & 3) * 8u;
   x.zero_row = zero_row;
-  x.N = p.N;
   x.c_vrow_bytes = (uint32_t)V * (uint32_t)p.N * (uint32_t)sizeof(OutT);
   const uint32_t nvec = (uint32_t)row_offsets[p.m_vec];
   x.srd_cols = make_srd(p.col_idx, nvec * 4u);
@@ -986,7 +979,7 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
         if (u < units) *reinterpret_cast<uintx4 *>(lds + slab_unit_dst<NQ, L>(u)) = d[i];
       }
     }
-    if ((uint32_t)tid <= p.rows_per_block) *reinterpret_cast<intx4 *>(lds + table_off + tid * 16) = e;
+    if ((uint32_t)tid <= p.rows_per_block + 1u) *reinterpret_cast<intx4 *>(lds + table_off + tid * 16) = e;
   }
   __syncthreads();
 
@@ -1018,12 +1011,12 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
       SlabRows rows;
       rows.table = reinterpret_cast<const intx4 *>(lds + table_off + table_sel * table_bytes);
       rows.n_rows = min(p.m_vec, row_lo + (int)p.rows_per_block) - row_lo;
-      // (the entry at rows_per_block is rewritten, all zeros, with every table)
-      rows.counter = reinterpret_cast<int *>(lds + table_off + table_sel * table_bytes + p.rows_per_block * 16u + 12u);
+      // (the entries at rows_per_block and behind it are rewritten, all zeros, with every table)
+      rows.counter = reinterpret_cast<int *>(lds + table_off + table_sel * table_bytes + (p.rows_per_block + 1u) * 16u);
       rows.lane = lane;
       SlabStore<V, OutT, NQ> out;
       out.init(lane, (int)cur.tile * (16 * NQ), p.N);
-      // One buffer descriptor spans this batch element's C (the launcher checks it is below 4 GiB).
+      // One buffer descriptor spans this batch element's C (the launcher checks it is at most 2 GiB).
       const __amdgpu_buffer_rsrc_t srd_c = make_srd(reinterpret_cast<OutT *>(p.C) + (int64_t)cur.batch * p.stride_C,
                                                     (uint32_t)p.m_vec * x.c_vrow_bytes);
       slab_process_item<V, OutT, NQ, L>(x, lds, layout_buffer_off(L, NQ, zero_row + 1u, slab_sel), rows, p.values + (int64_t)cur.batch * p.stride_values,
@@ -1049,7 +1042,7 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
       } else {
         table_sel ^= 1u;
       }
-      if ((uint32_t)ctid <= p.rows_per_block) *reinterpret_cast<intx4 *>(lds + table_off + table_sel * table_bytes + ctid * 16) = f.entry;
+      if ((uint32_t)ctid <= p.rows_per_block + 1u) *reinterpret_cast<intx4 *>(lds + table_off + table_sel * table_bytes + ctid * 16) = f.entry;
       __syncthreads();
     } else {
       __syncthreads();  // every wave is done with the slab and the table
@@ -1069,7 +1062,7 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
           }
         }
       }
-      if ((uint32_t)ctid <= p.rows_per_block) *reinterpret_cast<intx4 *>(lds + table_off + ctid * 16) = e;
+      if ((uint32_t)ctid <= p.rows_per_block + 1u) *reinterpret_cast<intx4 *>(lds + table_off + ctid * 16) = e;
       __syncthreads();
     }
     cur = nxt;
@@ -1124,7 +1117,7 @@ static constexpr uint32_t kSlabMinRows = 32;   // keeps the copy of the slab a s
 // LDS bytes of a workgroup: slabs (+ zero rows), value tiles, two row tables.
 static uint32_t slab_lds_bytes(int K, int V, uint32_t rows, int layout, int NQ) {
   return layout_slab_region(layout, NQ, (uint32_t)K + 1u) + kSlabWaves * wave_lds_bytes(V) +
-         (layout == kPadDouble ? 1u : 2u) * 16u * (rows + 1u);
+         (layout == kPadDouble ? 1u : 2u) * 16u * (rows + 2u);
 }
 // Largest K the slab kernel takes (one slab, smallest row tables).
 static bool slab_fits(int K, int V, int NQ) { return slab_lds_bytes(K, V, kSlabMinRows, kXorSingle, NQ) <= kSlabLds; }
@@ -1245,8 +1238,9 @@ hipError_t launch_spmm(const SpmmArgs &a, int V, bool out_f16, hipStream_t strea
     // workgroups to fill the chip; otherwise one wave per (vector-row, 128 columns).
     const uint64_t slabs = (uint64_t)((a.N + 63) / 64) * (uint64_t)a.batch;
     const uint64_t blocks = slabs * (uint64_t)((a.m_vec + 31) / 32);
-    // The slab kernel addresses one batch element's C through a 32-bit buffer descriptor.
-    const bool c_ok = (uint64_t)a.m_vec * (V == 8 ? 8u : 16u) * (uint64_t)a.N * out_size < 0xffffffffull;
+    // The slab kernel addresses one batch element's C through a 32-bit buffer descriptor, and marks the lanes
+    // that must not store with an offset of 2 GiB.
+    const bool c_ok = (uint64_t)a.m_vec * (V == 8 ? 8u : 16u) * (uint64_t)a.N * out_size <= (uint64_t)kSlabDropStore;
     const bool slab_ok = slab_fits(a.K, V, 4) && c_ok;
     // Matrices too tall for a 64-column slab can take slabs 32 columns wide, twice as many.  A tall slab is not
     // double-buffered, so it pays only where many vector-rows share it, and only for V = 8: with V = 16 a

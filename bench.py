@@ -29,14 +29,18 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch of the headline workload at the default batch of 128, from hardware counters
 # (FETCH_SIZE and WRITE_SIZE, each scaled by its reading for a 256 MiB device copy): see
 # profiles/spmm_slab_v8_f32_cfg2_batch128_hbm_traffic.txt.  Other batch sizes report null.
-MEASURED_TRAFFIC_BYTES = {128: 66.3e6 + 268.4e6}
+MEASURED_TRAFFIC_BYTES = {128: 66.1e6 + 268.4e6}
 
 
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=10)
+    # The chip needs a few hundred launches (tens of milliseconds) under this load before its clocks settle: launch
+    # times start near 58 us, rise to 70-80 us and come back to 57-59 us after about 500 launches.  The default
+    # warm-up covers that transient, so that the timed steps measure the sustained rate; the series of chunk
+    # averages through warm-up and timed steps is reported as extra.headline_us_per_chunk.
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--batch", type=int, default=128, help="independent value/B/C sets per step")
     ap.add_argument("--quick", action="store_true", help="skip the extra configurations and CPU legs")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -47,23 +51,41 @@ def parse_args():
     return ap.parse_args()
 
 
-def time_launches(fn, steps, warmup):
+def time_launches(fn, steps, warmup, series=None):
     """Average milliseconds per call over `steps` calls, HIP events on the launch stream."""
     import torch
-    for _ in range(warmup):
-        fn()
+    chunk = 100
+    marks = []
+
+    def run(n):
+        for i in range(n):
+            if series is not None and i % chunk == 0:
+                ev = torch.cuda.Event(enable_timing=True)
+                ev.record()
+                marks.append((ev, min(chunk, n - i)))
+            fn()
+
+    run(warmup)
     torch.cuda.synchronize()
+    n_warm = len(marks)
     start = torch.cuda.Event(enable_timing=True)
     end = torch.cuda.Event(enable_timing=True)
     start.record()
-    for _ in range(steps):
-        fn()
+    run(steps)
     end.record()
     torch.cuda.synchronize()
+    if series is not None:
+        # (events on the launch stream; the chunk that ends the warm-up runs into the host synchronisation and is left out)
+        bounds = [m[0] for m in marks] + [end]
+        for i, (ev, n) in enumerate(marks):
+            if i != n_warm - 1:
+                series.append(round(ev.elapsed_time(bounds[i + 1]) / n * 1e3, 1))
+            else:
+                series.append(None)
     return start.elapsed_time(end) / steps
 
 
-def spmm_case(L, torch, synth, M, K, V, sparsity, N, batch, out_f32, std, seed, steps, warmup, dense=False):
+def spmm_case(L, torch, synth, M, K, V, sparsity, N, batch, out_f32, std, seed, steps, warmup, dense=False, series=None):
     """Times one SpMM configuration; returns a dict of figures."""
     vs = synth.vector_sparse(M, K, V, sparsity, seed=seed, std=std)
     g = torch.Generator(device="cuda").manual_seed(seed)
@@ -82,7 +104,7 @@ def spmm_case(L, torch, synth, M, K, V, sparsity, N, batch, out_f32, std, seed, 
         if rc:
             raise RuntimeError("sspmm failed: %d" % rc)
 
-    ms = time_launches(launch, steps, warmup)
+    ms = time_launches(launch, steps, warmup, series)
     bytes_alg = batch * synth.spmm_algorithmic_bytes(vs.m_vec, V, nv, K, N, 4 if out_f32 else 2) \
         - (batch - 1) * (4 * nv + 4 * (vs.m_vec + 1))  # the pattern is shared by the batch
     flops = 2.0 * vs.nnz * N * batch
@@ -131,10 +153,11 @@ def main():
         del src, dst
 
     M, K, V, sparsity, N = 2048, 512, 8, 0.9, 256
-    kernel_names = {1: "spmm_generic_kernel<8,float>", 2: "spmm_gather_kernel<8,float>", 3: "spmm_slab_kernel<8,float,true>",
+    kernel_names = {1: "spmm_generic_kernel<8,float>", 2: "spmm_gather_kernel<8,float>", 3: "spmm_slab_kernel<8,float,*,4>",
                     4: "spmm_gather_split_kernel<8,float>", 5: "spmm_slab_kernel<8,float,*,2>"}
+    series = []
     main_res, (vs, vals, B, C) = spmm_case(L, torch, synth, M, K, V, sparsity, N, args.batch, True, 0.02, 2,
-                                           args.steps, args.warmup, dense=not args.quick)
+                                           args.steps, args.warmup, dense=not args.quick, series=series)
     torch.cuda.synchronize()
     main_kernel = kernel_names.get(L.sspmm_last_kernel(), "unknown")
 
@@ -203,10 +226,12 @@ def main():
     del vals, B, C
 
     extra = {}
+    # launch time (us) averaged over chunks of 100 launches, from the first warm-up launch to the last timed one
+    extra["headline_us_per_chunk"] = {"chunk": 100, "warmup_chunks": (args.warmup + 99) // 100, "us": series}
     if cold:
         extra["cfg2_single_launches_cold"] = cold
     if not args.quick:
-        st, wu = max(20, args.steps // 4), 5
+        st, wu = max(20, args.steps // 4), max(5, args.warmup // 5)
         cases = {
             "cfg2_single_launch": dict(M=2048, K=512, V=8, sparsity=0.9, N=256, batch=1, out_f32=True, std=0.02, seed=2),
             "cfg2_batched_fp16_out": dict(M=2048, K=512, V=8, sparsity=0.9, N=256, batch=args.batch, out_f32=False,

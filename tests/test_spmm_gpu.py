@@ -323,6 +323,48 @@ def test_slab_kernel_around_its_lds_limits(oracle, built_library, V, K, expect):
 
 @pytest.mark.parametrize("V", [8, 16])
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("m_vec,N", [(1, 72), (5, 8), (16, 200), (17, 264), (33, 136), (70, 72)])
+def test_slab_kernel_writes_nothing_outside_its_columns(oracle, built_library, V, out_dtype, m_vec, N):
+    """Column tails of the slab kernel: lanes beyond N must not store.  C lies between two guard areas, a second
+    batch element follows it at a stride that leaves a gap, and the vector-rows are processed last to first, so a
+    store that strayed into the following row would survive there.  Fewer vector-rows than the workgroup has waves,
+    one more than it has, several row blocks."""
+    from sspmm_amd import _lib
+    L = _lib.lib()
+    batch, K, guard = 2, 96, 4096
+    vs = synth.vector_sparse(m_vec * V, K, V, 0.7, seed=900 + m_vec)
+    rng = np.random.default_rng(901 + N)
+    vals = rng.standard_normal((batch, vs.values.size)).astype(np.float16)
+    B = rng.standard_normal((batch, K, N)).astype(np.float16)
+    M = m_vec * V
+    stride_c = M * N + 64  # elements: a gap of 64 behind every batch element
+    np_dtype = np.float32 if out_dtype == torch.float32 else np.float16
+    sentinel = 12345.0
+    buf = torch.full((guard + batch * stride_c + guard,), sentinel, dtype=out_dtype, device="cuda")
+    ro, ci, dv, dB = dev(vs.row_offsets), dev(vs.col_idx), dev(vals), dev(B)
+    order = dev(np.arange(m_vec - 1, -1, -1, dtype=np.int32))
+    fn = L.sspmm_batched_f16_f32 if out_dtype == torch.float32 else L.sspmm_batched_f16_f16
+    L.sspmm_select_kernel(3)
+    try:
+        rc = fn(batch, m_vec, V, N, K, order.data_ptr(), ro.data_ptr(), ci.data_ptr(), dv.data_ptr(), vs.values.size,
+                dB.data_ptr(), K * N, buf.data_ptr() + guard * buf.element_size(), stride_c,
+                torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        ran = L.sspmm_last_kernel()
+    finally:
+        L.sspmm_select_kernel(0)
+    assert rc == 0 and ran == 3
+    got = buf.cpu().numpy().astype(np_dtype)
+    assert np.all(got[:guard] == sentinel) and np.all(got[guard + batch * stride_c:] == sentinel)
+    for b in range(batch):
+        lo = guard + b * stride_c
+        assert np.all(got[lo + M * N:lo + stride_c] == sentinel), b
+        want = oracle.spmm(m_vec, V, N, K, vs.row_offsets, vs.col_idx, vals[b], B[b])
+        assert max_rel_err(got[lo:lo + M * N].reshape(M, N), want) <= (TIGHT_F32 if out_dtype == torch.float32 else TIGHT_F16)
+
+
+@pytest.mark.parametrize("V", [8, 16])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("N", [32, 72, 200, 256])
 def test_narrow_slab_kernel(oracle, built_library, V, out_dtype, N):
     """The 32-column slab (K between the 64-column slab's limit and twice that): column tails, ragged and empty

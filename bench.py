@@ -43,6 +43,8 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--batch", type=int, default=128, help="independent value/B/C sets per step")
     ap.add_argument("--quick", action="store_true", help="skip the extra configurations and CPU legs")
+    ap.add_argument("--attention-only", action="store_true",
+                    help="run only the sparse attention block (bsddmm, bcsr_softmax, bspmm) and print its figures")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy (its hardware-counter readings calibrate FETCH_SIZE / "
                          "WRITE_SIZE when the run is profiled)")
@@ -125,6 +127,35 @@ def spmm_case(L, torch, synth, M, K, V, sparsity, N, batch, out_f32, std, seed, 
     return out, handles
 
 
+def attention_block(torch, synth, sspmm_amd, st, wu):
+    """Times the three steps of the reference's sparse attention block; returns a dict of figures."""
+    # the sparse attention block of the reference (bsddmm -> bcsr_softmax -> bspmm) on one mask shared by
+    # 48 heads: 4096 tokens, head size 64, V=8, 90 % of the vectors masked out
+    seqA, dA, VA, bA = 4096, 64, 8, 48
+    mk_a = synth.vector_sparse(seqA, seqA, VA, 0.9, seed=7)
+    offA, colA = torch.from_numpy(mk_a.row_offsets).cuda(), torch.from_numpy(mk_a.col_idx).cuda()
+    qA, kA, vA = (torch.randn(bA, seqA, dA, device="cuda").half() for _ in range(3))
+    nvA = mk_a.col_idx.size
+    wA = sspmm_amd.bsddmm(None, offA, colA, qA, kA, VA)
+    pA = sspmm_amd.bcsr_softmax(None, offA, wA, 0.125, VA, bA)
+    t_sddmm = time_launches(lambda: sspmm_amd.bsddmm(None, offA, colA, qA, kA, VA), st, wu)
+    t_soft = time_launches(lambda: sspmm_amd.bcsr_softmax(None, offA, wA, 0.125, VA, bA), st, wu)
+    t_av = time_launches(lambda: sspmm_amd.bspmm(None, offA, colA, pA, vA, VA), st, wu)
+    t_dense = time_launches(lambda: torch.nn.functional.scaled_dot_product_attention(qA, kA, vA), st, wu)
+    by_sddmm = bA * (2 * seqA * dA * 2 + 2 * nvA * VA) + 4 * nvA + 4 * (mk_a.m_vec + 1)
+    by_soft = bA * 2 * 2 * nvA * VA + 4 * (mk_a.m_vec + 1)
+    by_av = bA * (2 * nvA * VA + 2 * seqA * dA + 2 * seqA * dA) + 4 * nvA + 4 * (mk_a.m_vec + 1)
+    res = {
+        "bsddmm_ms": t_sddmm, "bsddmm_hbm_frac": by_sddmm / t_sddmm / 1e6 / HBM_PEAK_GBPS, "bsddmm_alg_bytes": by_sddmm,
+        "bcsr_softmax_ms": t_soft, "bcsr_softmax_hbm_frac": by_soft / t_soft / 1e6 / HBM_PEAK_GBPS,
+        "bcsr_softmax_alg_bytes": by_soft,
+        "bspmm_ms": t_av, "bspmm_hbm_frac": by_av / t_av / 1e6 / HBM_PEAK_GBPS, "bspmm_alg_bytes": by_av,
+        "block_ms": t_sddmm + t_soft + t_av, "dense_sdpa_ms": t_dense, "nvec": int(nvA),
+    }
+    del qA, kA, vA, wA, pA
+    return res
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -141,6 +172,10 @@ def main():
     L = _lib.lib()
     torch.cuda.set_device(0)
     L.sspmm_select_kernel({"auto": 0, "generic": 1, "gather": 2, "slab": 3}[args.kernel])
+    if args.attention_only:
+        print(json.dumps({"sparse_attention_seq4096_d64_v8_s0.9_heads48":
+                          attention_block(torch, synth, sspmm_amd, args.steps, args.warmup)}))
+        return
 
     if args.calibrate_copy:
         src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device="cuda")
@@ -152,7 +187,7 @@ def main():
 
     M, K, V, sparsity, N = 2048, 512, 8, 0.9, 256
     kernel_names = {1: "spmm_generic_kernel<8,float>", 2: "spmm_gather_kernel<8,float>", 3: "spmm_slab_kernel<8,float,*,4>",
-                    4: "spmm_gather_split_kernel<8,float>", 5: "spmm_slab_kernel<8,float,*,2>"}
+                    4: "spmm_gather_split_kernel<8,float>", 5: "spmm_slab_kernel<8,float,*,2>", 6: "spmm_stage_kernel<8,float>"}
     series = []
     main_res, (vs, vals, B, C) = spmm_case(L, torch, synth, M, K, V, sparsity, N, args.batch, True, 0.02, 2,
                                            args.steps, args.warmup, dense=not args.quick, series=series)
@@ -380,30 +415,7 @@ def main():
             "projections": per,
         }
 
-        # the sparse attention block of the reference (bsddmm -> bcsr_softmax -> bspmm) on one mask shared by
-        # 48 heads: 4096 tokens, head size 64, V=8, 90 % of the vectors masked out
-        seqA, dA, VA, bA = 4096, 64, 8, 48
-        mk_a = synth.vector_sparse(seqA, seqA, VA, 0.9, seed=7)
-        offA, colA = torch.from_numpy(mk_a.row_offsets).cuda(), torch.from_numpy(mk_a.col_idx).cuda()
-        qA, kA, vA = (torch.randn(bA, seqA, dA, device="cuda").half() for _ in range(3))
-        nvA = mk_a.col_idx.size
-        wA = sspmm_amd.bsddmm(None, offA, colA, qA, kA, VA)
-        pA = sspmm_amd.bcsr_softmax(None, offA, wA, 0.125, VA, bA)
-        t_sddmm = time_launches(lambda: sspmm_amd.bsddmm(None, offA, colA, qA, kA, VA), st, wu)
-        t_soft = time_launches(lambda: sspmm_amd.bcsr_softmax(None, offA, wA, 0.125, VA, bA), st, wu)
-        t_av = time_launches(lambda: sspmm_amd.bspmm(None, offA, colA, pA, vA, VA), st, wu)
-        t_dense = time_launches(lambda: torch.nn.functional.scaled_dot_product_attention(qA, kA, vA), st, wu)
-        by_sddmm = bA * (2 * seqA * dA * 2 + 2 * nvA * VA) + 4 * nvA + 4 * (mk_a.m_vec + 1)
-        by_soft = bA * 2 * 2 * nvA * VA + 4 * (mk_a.m_vec + 1)
-        by_av = bA * (2 * nvA * VA + 2 * seqA * dA + 2 * seqA * dA) + 4 * nvA + 4 * (mk_a.m_vec + 1)
-        extra["sparse_attention_seq4096_d64_v8_s0.9_heads48"] = {
-            "bsddmm_ms": t_sddmm, "bsddmm_hbm_frac": by_sddmm / t_sddmm / 1e6 / HBM_PEAK_GBPS, "bsddmm_alg_bytes": by_sddmm,
-            "bcsr_softmax_ms": t_soft, "bcsr_softmax_hbm_frac": by_soft / t_soft / 1e6 / HBM_PEAK_GBPS,
-            "bcsr_softmax_alg_bytes": by_soft,
-            "bspmm_ms": t_av, "bspmm_hbm_frac": by_av / t_av / 1e6 / HBM_PEAK_GBPS, "bspmm_alg_bytes": by_av,
-            "block_ms": t_sddmm + t_soft + t_av, "dense_sdpa_ms": t_dense, "nvec": int(nvA),
-        }
-        del qA, kA, vA, wA, pA
+        extra["sparse_attention_seq4096_d64_v8_s0.9_heads48"] = attention_block(torch, synth, sspmm_amd, st, wu)
 
         # row reordering ahead of the SVC: 16384 rows that are noisy copies of 256 prototype rows, shuffled
         rc_csr = synth.clustered_csr(16384, 16384, 256, 128, seed=6, keep=0.9, extras=1)

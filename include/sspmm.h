@@ -32,8 +32,9 @@ int sspmm_version(void);
 /*
  * Testing and tuning hook without a counterpart in the reference: forces one SpMM kernel wherever
  * its preconditions hold.  0 = automatic choice (default), 1 = scalar kernel (any shape),
- * 2 = one-wave gather kernel, 3 = LDS-slab kernel.  Process-wide, not thread-safe.  Returns the
- * previous setting, or -1 for an unknown value.
+ * 2 = one-wave gather kernel, 3 = LDS-slab kernel, 6 = the gather kernel's staged form (rows of B
+ * fetched whole and passed through LDS; the automatic choice takes it for N <= 64 only) on any
+ * width.  Process-wide, not thread-safe.  Returns the previous setting, or -1 for an unknown value.
  */
 int sspmm_select_kernel(int which);
 
@@ -41,7 +42,8 @@ int sspmm_select_kernel(int which);
  * SpMM call of this process ran, numbered as above, with 4 = the gather kernel's variant for
  * K > 4096 that splits long vector-rows over the waves of a workgroup (selected as 2) and
  * 5 = the LDS-slab kernel with 32-column slabs, for K too tall for 64-column ones (selected
- * as 3); 0 before any call.  Not thread-safe. */
+ * as 3); the staged gather kernel reports 6 also where it was chosen automatically; 0 before any
+ * call.  Not thread-safe. */
 int sspmm_last_kernel(void);
 
 /* Static text for a return code of this library. */

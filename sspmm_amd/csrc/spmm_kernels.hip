@@ -1070,6 +1070,148 @@ __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs 
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// Gather kernel for right-hand sides of at most 64 columns (an attention head's features), where a
+// row of B is 128 bytes or less.  Fetching such rows in the MFMA's operand layout means 8 bytes per
+// lane, and the vector memory pipeline works through a wave's load four lanes at a time whatever
+// their width: half of its byte rate.  Here eight neighbouring lanes fetch the eight 16-byte pieces
+// of one row (a load instruction brings 8 whole rows, a step's 32 rows take 4 of them instead of 8),
+// the rows are staged in a per-wave tile in LDS and come back as MFMA operands through the
+// transpose reads of the slab kernel, whose accumulator layout and store of C are shared too.  No
+// byte shuffling in registers.  Rows of the tile are 144 bytes apart so that the four consecutive
+// rows a 16-lane group reads fall into different banks.
+static constexpr uint32_t kStagePitch = 144;
+
+template <int V>
+struct StageHead {  // what does not depend on other loads
+  uintx4 cols;      // column indices of k slots 4j .. 4j+3, j = lane / 8
+  typename SlabVals<V>::type vraw;
+  int kc;
+};
+template <int V>
+struct StageBody {
+  uintx4 piece[4];  // piece[i] = 16 bytes (columns 8 * (lane % 8) ..) of the row of B named by k slot 4j + i
+  typename SlabVals<V>::type vraw;
+};
+
+template <int V, typename OutT>
+__global__ __launch_bounds__(64) void spmm_stage_kernel(const SpmmArgs p) {
+  __shared__ __align__(16) unsigned char stage[32 * kStagePitch];
+  __shared__ __align__(16) unsigned char val_tile[val_tile_bytes(V)];
+  const uint32_t id = blockIdx.x;
+  const uint32_t w = (id & 7u) * p.per_xcd + (id >> 3);
+  if (w >= p.total_work) return;
+  const uint32_t r = w % (uint32_t)p.m_vec;
+  const uint32_t t = w / (uint32_t)p.m_vec;
+  const uint32_t tile = t % p.n_tiles;  // 64 columns
+  const uint32_t batch = t / p.n_tiles;
+  const int row = __builtin_amdgcn_readfirstlane(p.row_indices ? p.row_indices[r] : (int)r);
+
+  const int lane = threadIdx.x;
+  const int m = lane & 15, g = lane >> 4, j = lane >> 3, pc = lane & 7;
+  const int beg = p.row_offsets[row], end = p.row_offsets[row + 1];
+
+  const uint16_t *vals = p.values + (int64_t)batch * p.stride_values;
+  const uint32_t b_bytes = (uint32_t)p.K * (uint32_t)p.N * 2u;
+  // the descriptors of the pattern and the values end at this vector-row's last vector: slots past it read as zero
+  const __amdgpu_buffer_rsrc_t srd_cols = make_srd(p.col_idx, (uint32_t)end * 4u);
+  const __amdgpu_buffer_rsrc_t srd_vals = make_srd(vals, (uint32_t)end * (V * 2u));
+  const __amdgpu_buffer_rsrc_t srd_b = make_srd(p.B + (int64_t)batch * p.stride_B, b_bytes);
+
+  // Lanes whose columns lie beyond N aim every gather at the first byte past B, where loads return zero.
+  const int ncol = (int)tile * 64 + 8 * pc;
+  const bool col_ok = ncol < p.N;
+  const uint32_t lane_n2 = col_ok ? (uint32_t)p.N * 2u : 0u;
+  const uint32_t lane_col_off = col_ok ? (uint32_t)ncol * 2u : b_bytes;
+  constexpr uint32_t kLaneBytes = V * 2u * 32u / 64u;
+  const uint32_t vals_lane_off = (uint32_t)lane * kLaneBytes;
+  unsigned char *const tile_dst = val_tile + lane * kLaneBytes;
+  unsigned char *const stage_dst = stage + (uint32_t)(4 * j) * kStagePitch + (uint32_t)pc * 16u;
+  // transpose reads: k slots 8g + m/4 (and + 4) of the value tile and of the staged rows
+  const uint32_t a_off = (uint32_t)(8 * g + (m >> 2)) * (V * 2u) + (uint32_t)(m & 3) * 8u;
+  const uint32_t b_rd = lds_address(stage) + (uint32_t)(8 * g + (m >> 2)) * kStagePitch + (uint32_t)(m & 3) * 8u;
+
+  const auto load_head = [&](StageHead<V> &h, int kc) {
+    h.kc = kc;
+    h.cols = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_cols, (kc + 4 * j) * 4, 0, 0));
+    h.vraw = SlabVals<V>::load(srd_vals, (uint32_t)kc * (V * 2u) + vals_lane_off);
+  };
+  const auto load_body = [&](StageBody<V> &c, const StageHead<V> &h) {
+    uint32_t off[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) off[i] = __umul24(h.cols[i], lane_n2) + lane_col_off;
+    if (h.kc + 32 > end) {  // wave-uniform: only the last chunk of a vector-row can be partial
+#pragma unroll
+      for (int i = 0; i < 4; ++i) off[i] = (h.kc + 4 * j + i < end) ? off[i] : b_bytes;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      c.piece[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_b, off[i], 0, 0));
+    c.vraw = h.vraw;
+  };
+  floatx4 acc[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const auto contract = [&](const StageBody<V> &c) {
+    // (LDS operations of a wave execute in order: these writes land behind the previous chunk's reads)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<uintx4 *>(stage_dst + i * kStagePitch) = c.piece[i];
+    *reinterpret_cast<typename SlabVals<V>::type *>(tile_dst) = c.vraw;
+    Half8Bits a;
+    {
+      const uintx2 lo = lds_read_tr(val_tile, a_off);
+      const uintx2 hi = lds_read_tr(val_tile, a_off + 4u * (V * 2u));
+      a.u[0] = lo[0]; a.u[1] = lo[1]; a.u[2] = hi[0]; a.u[3] = hi[1];
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      Half8Bits b;
+      const uintx2 lo = lds_read_tr_abs(b_rd + 32u * q);
+      const uintx2 hi = lds_read_tr_abs(b_rd + 4u * kStagePitch + 32u * q);
+      b.u[0] = lo[0]; b.u[1] = lo[1]; b.u[2] = hi[0]; b.u[3] = hi[1];
+      // the staged rows are the first operand, as the slab is in the slab kernel: lane (m, g) ends up with
+      // columns 16q + 4g .. + 3 of output row m
+      acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b.h, a.h, acc[q], 0, 0, 0);
+    }
+  };
+
+  if (beg < end) {
+    // Heads run two chunks ahead of the arithmetic, bodies one (two of each, used alternately).
+    StageHead<V> h0, h1;
+    StageBody<V> c0, c1;
+    load_head(h0, beg);
+    load_head(h1, beg + 32);
+    load_body(c0, h0);
+    int kc = beg + 32;  // first vector of the chunk whose body is loaded next
+    for (;;) {
+      if (kc >= end) {
+        contract(c0);
+        break;
+      }
+      load_head(h0, kc + 32);
+      load_body(c1, h1);
+      contract(c0);
+      kc += 32;
+      if (kc >= end) {
+        contract(c1);
+        break;
+      }
+      load_head(h1, kc + 32);
+      load_body(c0, h0);
+      contract(c1);
+      kc += 32;
+    }
+  }
+
+  SlabStore<V, OutT, 4> out;
+  out.init(lane, (int)tile * 64, p.N);
+  const uint32_t c_vrow_bytes = (uint32_t)V * (uint32_t)p.N * (uint32_t)sizeof(OutT);
+  // One buffer descriptor spans this batch element's C (the launcher checks it is at most 2 GiB).
+  const __amdgpu_buffer_rsrc_t srd_c = make_srd(reinterpret_cast<OutT *>(p.C) + (int64_t)batch * p.stride_C,
+                                                (uint32_t)p.m_vec * c_vrow_bytes);
+  out.store(acc, srd_c, (uint32_t)row * c_vrow_bytes);
+}
+
 // Shape-agnostic kernel: any N, any alignment.  One thread per output column, scalar gathers,
 // accumulation in ascending vector order (the order of the reference's host check loop,
 // reference SSpMM/sspmm_test.cpp:82-94).
@@ -1200,7 +1342,15 @@ static hipError_t launch_v(const SpmmArgs &a, int which, hipStream_t stream) {
     p.n_tiles = (uint32_t)((a.N + 127) / 128);
     p.total_work = (uint32_t)a.m_vec * p.n_tiles * (uint32_t)a.batch;
     p.per_xcd = (p.total_work + 7u) / 8u;
-    if (a.K > kSplitMinK) {
+    // (the staged kernel addresses one batch element's C through a 32-bit buffer descriptor, as the slab kernel does)
+    const bool c_ok = (uint64_t)a.m_vec * V * (uint64_t)a.N * sizeof(OutT) <= (uint64_t)kSlabDropStore;
+    if (g_kernel_override == 6 && c_ok) {  // (tuning) the staged kernel on any width, 64 columns per wave
+      p.n_tiles = (uint32_t)((a.N + 63) / 64);
+      p.total_work = (uint32_t)a.m_vec * p.n_tiles * (uint32_t)a.batch;
+      p.per_xcd = (p.total_work + 7u) / 8u;
+      g_last_kernel = 6;
+      hipLaunchKernelGGL((spmm_stage_kernel<V, OutT>), dim3(p.per_xcd * 8u), dim3(64), 0, stream, p);
+    } else if (a.K > kSplitMinK) {
       g_last_kernel = 4;
       static_assert(kSplitWaves >= 4, "wave rr < 4 stores output row 4g + rr");
       p.total_work = (((uint32_t)a.m_vec + kSplitWaves - 1u) / kSplitWaves) * p.n_tiles * (uint32_t)a.batch;
@@ -1210,7 +1360,12 @@ static hipError_t launch_v(const SpmmArgs &a, int which, hipStream_t stream) {
       p.n_tiles = 1;
       p.total_work = (uint32_t)a.m_vec * (uint32_t)a.batch;
       p.per_xcd = (p.total_work + 7u) / 8u;
-      hipLaunchKernelGGL((spmm_gather_kernel<V, OutT, 4>), dim3(p.per_xcd * 8u), dim3(64), 0, stream, p);
+      if (c_ok) {
+        g_last_kernel = 6;
+        hipLaunchKernelGGL((spmm_stage_kernel<V, OutT>), dim3(p.per_xcd * 8u), dim3(64), 0, stream, p);
+      } else {
+        hipLaunchKernelGGL((spmm_gather_kernel<V, OutT, 4>), dim3(p.per_xcd * 8u), dim3(64), 0, stream, p);
+      }
     } else {
       hipLaunchKernelGGL((spmm_gather_kernel<V, OutT, 8>), dim3(p.per_xcd * 8u), dim3(64), 0, stream, p);
     }
@@ -1249,7 +1404,7 @@ hipError_t launch_spmm(const SpmmArgs &a, int V, bool out_f16, hipStream_t strea
     const bool narrow_ok = !slab_ok && slab_fits(a.K, V, 2) && c_ok;
     which = (slab_ok && a.m_vec >= 64 && blocks >= 1024) ? 3 : 2;
     if (narrow_ok && V == 8 && a.m_vec >= 256 && 2u * blocks >= 1024) which = 5;
-    if (g_kernel_override == 2) which = 2;
+    if (g_kernel_override == 2 || g_kernel_override == 6) which = 2;
     if (g_kernel_override == 3 && slab_ok) which = 3;
     if (g_kernel_override == 3 && narrow_ok) which = 5;
   }

@@ -9,7 +9,7 @@ from gpu_util import PARITY_TOL, TIGHT_F16, TIGHT_F32, dev, max_rel_err
 
 pytestmark = pytest.mark.gpu
 
-KERNELS = {"auto": 0, "gather": 2, "slab": 3}
+KERNELS = {"auto": 0, "gather": 2, "slab": 3, "staged": 6}
 
 
 @pytest.fixture(params=sorted(KERNELS))
@@ -77,8 +77,8 @@ def test_column_tails(oracle, kernel, V, N):
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("N", [8, 40, 56, 64])
 def test_narrow_right_hand_sides(oracle, built_library, V, out_dtype, N):
-    """N <= 64 (an attention head's features) runs the gather kernel with four columns per lane: ragged rows
-    with partial last chunks, rows of several chunks, empty rows, a batch."""
+    """N <= 64 (an attention head's features) runs the staged gather kernel: ragged rows with partial last chunks,
+    rows of several chunks, empty rows, a batch."""
     from sspmm_amd import _lib
     rng = np.random.default_rng(700 + V + N)
     K, m_vec = 900, 37
@@ -90,7 +90,7 @@ def test_narrow_right_hand_sides(oracle, built_library, V, out_dtype, N):
                             (rng.standard_normal(cols.size * V) * 0.1).astype(np.float16), cols.size * V)
     B = synth.dense_rhs(K, N, seed=N)
     got, _ = check(oracle, vs, B, out_dtype)
-    assert _lib.lib().sspmm_last_kernel() == 2
+    assert _lib.lib().sspmm_last_kernel() == 6
     assert not got[:V].any()
     vals3 = (rng.standard_normal((3, cols.size * V)) * 0.1).astype(np.float16)
     B3 = np.stack([synth.dense_rhs(K, N, seed=60 + b) for b in range(3)])

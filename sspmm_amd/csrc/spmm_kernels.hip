@@ -76,7 +76,9 @@ struct Store8<_Float16> {
     half8 h;
 #pragma unroll
     for (int i = 0; i < 8; ++i) h[i] = (_Float16)v[i];  // v_cvt_f16_f32: round to nearest even
-    *reinterpret_cast<half8 *>(p) = h;
+    // (non-temporal: the rows of B the grid keeps gathering stay in the L2; measured 1-10 % on fp16 outputs, while
+    // fp32 outputs gain on some shapes and lose up to 23 % on others and keep ordinary stores)
+    __builtin_nontemporal_store(h, reinterpret_cast<half8 *>(p));
   }
 };
 

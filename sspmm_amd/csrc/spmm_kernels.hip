@@ -1346,7 +1346,9 @@ static hipError_t launch_v(const SpmmArgs &a, int which, hipStream_t stream) {
     p.per_xcd = (p.total_work + 7u) / 8u;
     // (the staged kernel addresses one batch element's C through a 32-bit buffer descriptor, as the slab kernel does)
     const bool c_ok = (uint64_t)a.m_vec * V * (uint64_t)a.N * sizeof(OutT) <= (uint64_t)kSlabDropStore;
-    if (g_kernel_override == 6 && c_ok) {  // (tuning) the staged kernel on any width, 64 columns per wave
+    // The staged kernel: forced (tuning) on any width, 64 columns per wave; chosen for N <= 64 whatever K is (rows of
+    // 64 columns leave half of the split-row kernel's lanes idle: measured 1.5-2x on 8192 and 16384 columns).
+    if ((g_kernel_override == 6 || a.N <= 64) && c_ok) {
       p.n_tiles = (uint32_t)((a.N + 63) / 64);
       p.total_work = (uint32_t)a.m_vec * p.n_tiles * (uint32_t)a.batch;
       p.per_xcd = (p.total_work + 7u) / 8u;

@@ -102,6 +102,25 @@ def test_narrow_right_hand_sides(oracle, built_library, V, out_dtype, N):
 
 
 @pytest.mark.parametrize("V", [8, 16])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
+def test_narrow_right_hand_side_on_a_wide_matrix(oracle, built_library, V, out_dtype):
+    """N <= 64 keeps the staged gather kernel above K = 4096 too (an attention mask over a long sequence), long and
+    empty vector-rows included."""
+    from sspmm_amd import _lib
+    rng = np.random.default_rng(750 + V)
+    K, N, m_vec = 6000, 64, 19
+    lens = rng.integers(0, 90, m_vec)
+    lens[[0, 3, 11]] = [4100, 0, 513]
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cols = np.concatenate([rng.permutation(K)[:n] for n in lens]).astype(np.int32)
+    vs = synth.VectorSparse(m_vec * V, K, V, m_vec, off, cols,
+                            (rng.standard_normal(cols.size * V) * 0.05).astype(np.float16), cols.size * V)
+    got, _ = check(oracle, vs, synth.dense_rhs(K, N, seed=17), out_dtype)
+    assert _lib.lib().sspmm_last_kernel() == 6
+    assert not got[3 * V:4 * V].any()
+
+
+@pytest.mark.parametrize("V", [8, 16])
 @pytest.mark.parametrize("N", [1, 3, 17, 66, 130])
 def test_odd_widths_take_the_generic_kernel_and_match_the_oracle_bit_for_bit(oracle, built_library, V, N):
     """N % 8 != 0 runs the scalar kernel, which adds in the oracle's order: fp32 results are identical."""

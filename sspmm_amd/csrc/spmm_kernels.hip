@@ -1348,7 +1348,10 @@ static hipError_t launch_v(const SpmmArgs &a, int which, hipStream_t stream) {
     const bool c_ok = (uint64_t)a.m_vec * V * (uint64_t)a.N * sizeof(OutT) <= (uint64_t)kSlabDropStore;
     // The staged kernel: forced (tuning) on any width, 64 columns per wave; chosen for N <= 64 whatever K is (rows of
     // 64 columns leave half of the split-row kernel's lanes idle: measured 1.5-2x on 8192 and 16384 columns).
-    if ((g_kernel_override == 6 || a.N <= 64) && c_ok) {
+    // Also where the register-path kernel would start fewer than two waves per CU: 64 columns per wave make twice
+    // as many (about 10 % on launches of 4-5 us; from two to four waves per CU the register path is 10-20 % faster).
+    const bool few_waves = a.K <= kSplitMinK && p.total_work <= 2u * device_cus();
+    if ((g_kernel_override == 6 || a.N <= 64 || (few_waves && g_kernel_override == 0)) && c_ok) {
       p.n_tiles = (uint32_t)((a.N + 63) / 64);
       p.total_work = (uint32_t)a.m_vec * p.n_tiles * (uint32_t)a.batch;
       p.per_xcd = (p.total_work + 7u) / 8u;
@@ -1406,7 +1409,10 @@ hipError_t launch_spmm(const SpmmArgs &a, int V, bool out_f16, hipStream_t strea
     // gathered row of B already serves 16 output rows (measured: 1.2-1.3x over the gather kernel for V = 8 from
     // 256 vector-rows on, 0.8-0.9x for V = 16, 0.5-0.7x with 64 vector-rows at 90 % sparsity and above).
     const bool narrow_ok = !slab_ok && slab_fits(a.K, V, 2) && c_ok;
-    which = (slab_ok && a.m_vec >= 64 && blocks >= 1024) ? 3 : 2;
+    // (measured on a sweep of shapes at 90 % sparsity: with V = 8 the slab kernel is 1.15-1.4x faster than the gather
+    // kernel from 512 such blocks on, with V = 16 from 1024 (fp16 C) or 256 (fp32 C); below that the two tie or the
+    // gather kernel wins)
+    which = (slab_ok && a.m_vec >= 64 && blocks >= (V == 8 ? 512u : out_f16 ? 1024u : 256u)) ? 3 : 2;
     if (narrow_ok && V == 8 && a.m_vec >= 256 && 2u * blocks >= 1024) which = 5;
     if (g_kernel_override == 2 || g_kernel_override == 6) which = 2;
     if (g_kernel_override == 3 && slab_ok) which = 3;

@@ -299,7 +299,32 @@ __global__ __launch_bounds__(64) void spmm_gather_kernel(const SpmmArgs p) {
     }
   }
 
-  if (col_ok) {
+  if constexpr (std::is_same<OutT, float>::value && CPL == 8) {
+    // fp32 rows of 128 columns: a lane's eight columns are 32 bytes, so a store instruction of the layout the
+    // MFMAs leave would write 16-byte pieces 32 bytes apart.  The tile passes through LDS instead and goes out as
+    // whole lines, two rows of 512 bytes per instruction, non-temporal (launches of few vectors per row are
+    // mostly these stores: measured up to 1.5x at 95-98 % sparsity, nothing lost at 90 %).
+    __shared__ __align__(16) float ctile[V][128 + 4];
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+      const int v = 4 * g + rr;
+      if (v < V) {
+        *reinterpret_cast<floatx4 *>(&ctile[v][8 * m]) = floatx4{acc[0][rr], acc[1][rr], acc[2][rr], acc[3][rr]};
+        *reinterpret_cast<floatx4 *>(&ctile[v][8 * m + 4]) = floatx4{acc[4][rr], acc[5][rr], acc[6][rr], acc[7][rr]};
+      }
+    }
+    // (one wave per workgroup and LDS operations execute in order: no barrier)
+    float *cbase = reinterpret_cast<float *>(p.C) + (int64_t)batch * p.stride_C + (int64_t)row * V * p.N;
+    const int c4 = (lane & 31) * 4, gcol = (int)tile * 128 + c4;
+    if (gcol < p.N) {
+#pragma unroll
+      for (int i = 0; i < V / 2; ++i) {
+        const int v = 2 * i + (lane >> 5);
+        const floatx4 x = *reinterpret_cast<const floatx4 *>(&ctile[v][c4]);
+        __builtin_nontemporal_store(x, reinterpret_cast<floatx4 *>(cbase + (int64_t)v * p.N + gcol));
+      }
+    }
+  } else if (col_ok) {
     OutT *cbase = reinterpret_cast<OutT *>(p.C) + (int64_t)batch * p.stride_C;
 #pragma unroll
     for (int rr = 0; rr < 4; ++rr) {
@@ -1350,7 +1375,8 @@ static hipError_t launch_v(const SpmmArgs &a, int which, hipStream_t stream) {
     // 64 columns leave half of the split-row kernel's lanes idle: measured 1.5-2x on 8192 and 16384 columns).
     // Also where the register-path kernel would start fewer than two waves per CU: 64 columns per wave make twice
     // as many (about 10 % on launches of 4-5 us; from two to four waves per CU the register path is 10-20 % faster).
-    const bool few_waves = a.K <= kSplitMinK && p.total_work <= 2u * device_cus();
+    // (Not for K above 3072: where such a matrix is denser than 90 % its long rows cost the staged form 1.5x.)
+    const bool few_waves = a.K <= 3072 && p.total_work <= 2u * device_cus();
     if ((g_kernel_override == 6 || a.N <= 64 || (few_waves && g_kernel_override == 0)) && c_ok) {
       p.n_tiles = (uint32_t)((a.N + 63) / 64);
       p.total_work = (uint32_t)a.m_vec * p.n_tiles * (uint32_t)a.batch;
@@ -1410,9 +1436,10 @@ hipError_t launch_spmm(const SpmmArgs &a, int V, bool out_f16, hipStream_t strea
     // 256 vector-rows on, 0.8-0.9x for V = 16, 0.5-0.7x with 64 vector-rows at 90 % sparsity and above).
     const bool narrow_ok = !slab_ok && slab_fits(a.K, V, 2) && c_ok;
     // (measured on a sweep of shapes at 90 % sparsity: with V = 8 the slab kernel is 1.15-1.4x faster than the gather
-    // kernel from 512 such blocks on, with V = 16 from 1024 (fp16 C) or 256 (fp32 C); below that the two tie or the
-    // gather kernel wins)
-    which = (slab_ok && a.m_vec >= 64 && blocks >= (V == 8 ? 512u : out_f16 ? 1024u : 256u)) ? 3 : 2;
+    // kernel from 512 such blocks on, with V = 16 from 1024 (fp16 C) or 2048 (fp32 C, where the gather kernel's
+    // whole-line stores keep it level with the slab kernel for longer); below that the two tie or the gather kernel
+    // wins)
+    which = (slab_ok && a.m_vec >= 64 && blocks >= (V == 8 ? 512u : out_f16 ? 1024u : 2048u)) ? 3 : 2;
     if (narrow_ok && V == 8 && a.m_vec >= 256 && 2u * blocks >= 1024) which = 5;
     if (g_kernel_override == 2 || g_kernel_override == 6) which = 2;
     if (g_kernel_override == 3 && slab_ok) which = 3;

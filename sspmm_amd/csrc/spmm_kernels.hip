@@ -231,6 +231,35 @@ __device__ __forceinline__ void mac_chunk(const Chunk<CPL> &c, floatx4 (&acc)[CP
   }
 }
 
+// fp32 rows of 128 columns: a lane's eight columns are 32 bytes, so a store instruction of the layout the MFMAs
+// leave would write 16-byte pieces 32 bytes apart.  The V x 128 tile passes through LDS instead (`ctile`, private to
+// the wave: LDS operations of a wave execute in order, no barrier) and goes out as whole lines, two rows of 512
+// bytes per instruction, non-temporal.  Launches of few vectors per row are mostly these stores: measured up to
+// 2.2x at 95-98 % sparsity, 0.85-0.9x the time over a sweep of shapes at 90 %.
+// acc[q][rr] = C[row 4g + rr][column 8m + q] of the tile; crow = the tile's first row of C, at column 0.
+template <int V>
+__device__ __forceinline__ void store_tile_f32_lines(float (*ctile)[128 + 4], const floatx4 (&acc)[8], int lane, float *crow,
+                                                     int N, int tile) {
+  const int m = lane & 15, g = lane >> 4;
+#pragma unroll
+  for (int rr = 0; rr < 4; ++rr) {
+    const int v = 4 * g + rr;
+    if (v < V) {
+      *reinterpret_cast<floatx4 *>(&ctile[v][8 * m]) = floatx4{acc[0][rr], acc[1][rr], acc[2][rr], acc[3][rr]};
+      *reinterpret_cast<floatx4 *>(&ctile[v][8 * m + 4]) = floatx4{acc[4][rr], acc[5][rr], acc[6][rr], acc[7][rr]};
+    }
+  }
+  const int c4 = (lane & 31) * 4, gcol = tile * 128 + c4;
+  if (gcol < N) {
+#pragma unroll
+    for (int i = 0; i < V / 2; ++i) {
+      const int v = 2 * i + (lane >> 5);
+      const floatx4 x = *reinterpret_cast<const floatx4 *>(&ctile[v][c4]);
+      __builtin_nontemporal_store(x, reinterpret_cast<floatx4 *>(crow + (int64_t)v * N + gcol));
+    }
+  }
+}
+
 template <int V, typename OutT, int CPL>
 __global__ __launch_bounds__(64) void spmm_gather_kernel(const SpmmArgs p) {
   __shared__ __align__(16) unsigned char val_tiles[2][val_tile_bytes(V)];  // the value tiles of two chunks in turn
@@ -300,30 +329,9 @@ __global__ __launch_bounds__(64) void spmm_gather_kernel(const SpmmArgs p) {
   }
 
   if constexpr (std::is_same<OutT, float>::value && CPL == 8) {
-    // fp32 rows of 128 columns: a lane's eight columns are 32 bytes, so a store instruction of the layout the
-    // MFMAs leave would write 16-byte pieces 32 bytes apart.  The tile passes through LDS instead and goes out as
-    // whole lines, two rows of 512 bytes per instruction, non-temporal (launches of few vectors per row are
-    // mostly these stores: measured up to 1.5x at 95-98 % sparsity, nothing lost at 90 %).
     __shared__ __align__(16) float ctile[V][128 + 4];
-#pragma unroll
-    for (int rr = 0; rr < 4; ++rr) {
-      const int v = 4 * g + rr;
-      if (v < V) {
-        *reinterpret_cast<floatx4 *>(&ctile[v][8 * m]) = floatx4{acc[0][rr], acc[1][rr], acc[2][rr], acc[3][rr]};
-        *reinterpret_cast<floatx4 *>(&ctile[v][8 * m + 4]) = floatx4{acc[4][rr], acc[5][rr], acc[6][rr], acc[7][rr]};
-      }
-    }
-    // (one wave per workgroup and LDS operations execute in order: no barrier)
-    float *cbase = reinterpret_cast<float *>(p.C) + (int64_t)batch * p.stride_C + (int64_t)row * V * p.N;
-    const int c4 = (lane & 31) * 4, gcol = (int)tile * 128 + c4;
-    if (gcol < p.N) {
-#pragma unroll
-      for (int i = 0; i < V / 2; ++i) {
-        const int v = 2 * i + (lane >> 5);
-        const floatx4 x = *reinterpret_cast<const floatx4 *>(&ctile[v][c4]);
-        __builtin_nontemporal_store(x, reinterpret_cast<floatx4 *>(cbase + (int64_t)v * p.N + gcol));
-      }
-    }
+    store_tile_f32_lines<V>(ctile, acc, lane, reinterpret_cast<float *>(p.C) + (int64_t)batch * p.stride_C + (int64_t)row * V * p.N,
+                            p.N, (int)tile);
   } else if (col_ok) {
     OutT *cbase = reinterpret_cast<OutT *>(p.C) + (int64_t)batch * p.stride_C;
 #pragma unroll
@@ -445,7 +453,10 @@ __global__ __launch_bounds__(64 * kSplitWaves) void spmm_gather_split_kernel(con
   floatx4 acc[8];
   if (row >= 0 && !is_long) {
     gather_accumulate<V>(acc, p, batch, beg, end, end, lane, ncol, col_ok, val_tiles_all[wave]);
-    if (col_ok) {
+    if constexpr (std::is_same<OutT, float>::value) {
+      __shared__ __align__(16) float ctile_all[kSplitWaves][V][128 + 4];
+      store_tile_f32_lines<V>(ctile_all[wave], acc, lane, reinterpret_cast<float *>(cbase) + (int64_t)row * V * p.N, p.N, (int)tile);
+    } else if (col_ok) {
 #pragma unroll
       for (int rr = 0; rr < 4; ++rr) {
         const int v = 4 * g + rr;

@@ -1450,7 +1450,9 @@ hipError_t launch_spmm(const SpmmArgs &a, int V, bool out_f16, hipStream_t strea
     // kernel from 512 such blocks on, with V = 16 from 1024 (fp16 C) or 2048 (fp32 C, where the gather kernel's
     // whole-line stores keep it level with the slab kernel for longer); below that the two tie or the gather kernel
     // wins)
-    which = (slab_ok && a.m_vec >= 64 && blocks >= (V == 8 ? 512u : out_f16 ? 1024u : 2048u)) ? 3 : 2;
+    // (N <= 64: the alternative is the staged gather kernel, which the slab kernel beats by 1.2-1.3x from 512 on)
+    const uint32_t enough = (V == 8 || a.N <= 64) ? 512u : out_f16 ? 1024u : 2048u;
+    which = (slab_ok && a.m_vec >= 64 && blocks >= enough) ? 3 : 2;
     if (narrow_ok && V == 8 && a.m_vec >= 256 && 2u * blocks >= 1024) which = 5;
     if (g_kernel_override == 2 || g_kernel_override == 6) which = 2;
     if (g_kernel_override == 3 && slab_ok) which = 3;

@@ -34,16 +34,17 @@ int sspmm_version(void);
  * its preconditions hold.  0 = automatic choice (default), 1 = scalar kernel (any shape),
  * 2 = one-wave gather kernel, 3 = LDS-slab kernel, 6 = the gather kernel's staged form (rows of B
  * fetched whole and passed through LDS; the automatic choice takes it for N <= 64 only) on any
- * width.  Process-wide, not thread-safe.  Returns the previous setting, or -1 for an unknown value.
+ * width.  The setting belongs to the calling host thread (other threads keep the automatic choice).
+ * Returns the previous setting, or -1 for an unknown value.
  */
 int sspmm_select_kernel(int which);
 
 /* Companion of sspmm_select_kernel (no counterpart in the reference either): the kernel the latest
- * SpMM call of this process ran, numbered as above, with 4 = the gather kernel's variant for
+ * SpMM call of the calling host thread ran, numbered as above, with 4 = the gather kernel's variant for
  * K > 4096 that splits long vector-rows over the waves of a workgroup (selected as 2) and
  * 5 = the LDS-slab kernel with 32-column slabs, for K too tall for 64-column ones (selected
  * as 3); the staged gather kernel reports 6 also where it was chosen automatically; 0 before any
- * call.  Not thread-safe. */
+ * call of this thread. */
 int sspmm_last_kernel(void);
 
 /* Static text for a return code of this library. */
@@ -106,7 +107,7 @@ int sspmm_sorted_row_swizzle(int m_vec, const int32_t *row_offsets, int32_t *row
  * Replaces sddmm_cuda / batched_sddmm_cuda, reference end2end/sspmm_e2e/src/cuda/sddmm_kernel.cu:
  * 1161-1226 and 1228-1295 (batch strides m*k, n*k, nnz*V at :1244-1246).
  *   lhs [m_vec*V, F] and rhs [n_rhs, F] row-major, F a multiple of 8 up to 256, 16-byte aligned;
- *   column indices in [0, n_rhs); n_rhs*F below 2^31.
+ *   column indices in [0, n_rhs); n_rhs below 2^24 and n_rhs*F below 2^31.
  * ---------------------------------------------------------------------------------------- */
 int sspmm_sddmm_f16(int m_vec, int V, int F, int n_rhs, const int32_t *row_indices, const int32_t *row_offsets,
                     const int32_t *col_idx, const sspmm_half_t *lhs, const sspmm_half_t *rhs, sspmm_half_t *out_values,
@@ -178,7 +179,8 @@ int svc_fill(int M, int K, int V, const int32_t *row_ptr, const int32_t *col_ind
  *   svc_permute_csr      writes the reordered CSR arrays (out_row_ptr[M+1], out_col[nnz] and,
  *                        when csr_val != NULL, out_val[nnz]); feed them to svc_count / svc_fill.
  * Both take a workspace of svc_reorder_workspace_bytes(M) bytes (0 = no usable device).
- * perm must be a permutation of 0..M-1; entries outside that range give empty rows.
+ * perm must be a permutation of 0..M-1; entries outside that range give empty rows, and when an entry
+ * repeats, what would not fit into the nnz entries of the output arrays is dropped.
  * ---------------------------------------------------------------------------------------- */
 size_t svc_reorder_workspace_bytes(int M);
 

@@ -106,7 +106,8 @@ int sspmm_sddmm_batched_f16(int batch, int m_vec, int V, int F, int n_rhs, const
   if (F % 8 != 0 || F > 256) return kInvalid;
   if (batch == 0 || m_vec == 0) return 0;
   if (!row_offsets) return kInvalid;
-  if ((int64_t)n_rhs * F >= (1ll << 31) || (int64_t)m_vec * batch >= (1ll << 31) - 8) return kInvalid;
+  // (the kernel forms a row's byte offset with a 24-bit multiply of the column index)
+  if ((int64_t)n_rhs * F >= (1ll << 31) || n_rhs >= (1 << 24) || (int64_t)m_vec * batch >= (1ll << 31) - 8) return kInvalid;
   if (reinterpret_cast<uintptr_t>(lhs) % 16 || reinterpret_cast<uintptr_t>(rhs) % 16 ||
       reinterpret_cast<uintptr_t>(out_values) % 8 || stride_lhs % 8 || stride_rhs % 8 || stride_out % 4)
     return kInvalid;

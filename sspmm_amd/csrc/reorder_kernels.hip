@@ -75,7 +75,11 @@ __global__ __launch_bounds__(kReorderThreads) void permute_rows_kernel(int M, co
   if (i >= M) return;
   const int src = perm[i];
   if (src < 0 || src >= M) return;
-  const int s0 = row_ptr[src], n = row_ptr[src + 1] - s0, d0 = out_row_ptr[i];
+  // A permutation keeps the number of non-zeros; when `perm` repeats a row the lengths add up to more, and whatever
+  // would land beyond the source's non-zero count (the size of the output arrays) is dropped.
+  const int total = row_ptr[M];
+  const int s0 = row_ptr[src], d0 = out_row_ptr[i];
+  const int n = min(row_ptr[src + 1] - s0, total - d0);
   for (int e = lane; e < n; e += kRowLanes) {
     out_col[d0 + e] = col_ind[s0 + e];
     if (val) out_val[d0 + e] = val[s0 + e];

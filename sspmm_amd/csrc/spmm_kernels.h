@@ -27,9 +27,9 @@ struct SpmmArgs {
 hipError_t launch_spmm(const SpmmArgs &args, int V, bool out_f16, hipStream_t stream);
 
 // Forces a kernel where its preconditions hold: 0 automatic, 1 scalar, 2 gather, 3 LDS slab.
-// Process-wide and not thread-safe: meant for tests and tuning.  Returns the previous value.
+// Per host thread: meant for tests and tuning.  Returns the previous value.
 int set_kernel_override(int which);
-// Kernel the latest launch_spmm of this process used (1 scalar, 2 gather, 3 LDS slab; 0 before any launch).
+// Kernel the latest launch_spmm of the calling thread used (1 scalar, 2 gather, 3 LDS slab; 0 before any launch).
 int last_kernel();
 
 hipError_t launch_sorted_row_swizzle(int m_vec, const int32_t *row_offsets, int32_t *row_indices,

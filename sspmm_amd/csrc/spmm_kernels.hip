@@ -76,8 +76,8 @@ struct Store8<_Float16> {
     half8 h;
 #pragma unroll
     for (int i = 0; i < 8; ++i) h[i] = (_Float16)v[i];  // v_cvt_f16_f32: round to nearest even
-    // (non-temporal: the rows of B the grid keeps gathering stay in the L2; measured 1-10 % on fp16 outputs, while
-    // fp32 outputs gain on some shapes and lose up to 23 % on others and keep ordinary stores)
+    // (non-temporal: the rows of B the grid keeps gathering stay in the L2; measured 1-10 % on fp16 outputs.  fp32
+    // tiles of 128 columns do not come through here: they go out as whole lines, see store_tile_f32_lines)
     __builtin_nontemporal_store(h, reinterpret_cast<half8 *>(p));
   }
 };
@@ -1279,9 +1279,11 @@ __global__ __launch_bounds__(64) void spmm_generic_kernel(const SpmmArgs p) {
   for (int v = 0; v < V; ++v) cbase[((int64_t)row * V + v) * p.N + n] = (OutT)acc[v];
 }
 
-static int g_kernel_override = 0;  // 0 auto, 1 generic, 2 gather, 3 slab (tests and tuning)
+// Test and tuning hooks.  Both are per host thread: a thread that forces a kernel changes what its own calls
+// run and nobody else's, and the launch path shares no mutable state between threads.
+static thread_local int g_kernel_override = 0;  // 0 auto, 1 generic, 2 gather, 3 slab, 6 staged gather
 
-static int g_last_kernel = 0;  // kernel of the latest launch
+static thread_local int g_last_kernel = 0;  // kernel of this thread's latest launch
 int last_kernel() { return g_last_kernel; }
 
 int set_kernel_override(int which) {
@@ -1427,8 +1429,10 @@ hipError_t launch_spmm(const SpmmArgs &a, int V, bool out_f16, hipStream_t strea
   // 24-bit multiplies bound K and 2N; one buffer descriptor must span B.
   const uint64_t b_bytes = (uint64_t)a.K * (uint64_t)a.N * 2u;
   const int out_size = out_f16 ? 2 : 4;
+  // The value vectors are fetched with 8-byte (V = 8) or 16-byte (V = 16) loads per lane.
   const bool fast = (a.N % 8 == 0) && (reinterpret_cast<uintptr_t>(a.B) % 16 == 0) &&
                     (reinterpret_cast<uintptr_t>(a.C) % 16 == 0) && (a.stride_B % 8 == 0) &&
+                    (reinterpret_cast<uintptr_t>(a.values) % 16 == 0) && (a.stride_values % 8 == 0) &&
                     ((a.stride_C * out_size) % 16 == 0) && (a.K < (1 << 24)) && (a.N < (1 << 23)) &&
                     (b_bytes + 16 <= 0xffffffffull);
   int which = 1;

@@ -13,6 +13,10 @@
 //
 //   sspmm_test --synthetic <M> <K> <V> <sparsity> <N> [mixed] [func]
 // runs one seeded vector-sparse matrix without any file.
+//
+// With `func` the process exits with status 2 when any matrix disagrees with the host loop: an element
+// off by more than the reference's absolute 0.5 (reference SSpMM/sspmm_test.cpp:239), or a maximum
+// error above $SSPMM_REL_TOL (default 1e-2) of the largest reference magnitude.
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
 
@@ -132,8 +136,15 @@ double device_copy_gbs() {
   return gbs;
 }
 
+double relative_tolerance() {
+  const char *t = std::getenv("SSPMM_REL_TOL");
+  const double v = t ? std::atof(t) : 0.0;
+  return v > 0 ? v : 1e-2;
+}
+
+// Returns false when `func` is set and the result disagrees with the host loop.
 template <typename OutT>
-void bench(const Pattern &p, int N, int V, int kernel, bool sorted, bool func, bool record, bool reorder,
+bool bench(const Pattern &p, int N, int V, int kernel, bool sorted, bool func, bool record, bool reorder,
            const std::string &arch) {
   const int m_vec = p.m_vec, K = p.K, M = m_vec * V;
   const int nvec = p.row_offsets[m_vec];
@@ -216,6 +227,7 @@ void bench(const Pattern &p, int N, int V, int kernel, bool sorted, bool func, b
     out << p.nnz << ',' << m_vec << ',' << K << ',' << N << ',' << gflops << ',' << (long long)bytes << ',' << gbs
         << ',' << gbs / kHbmPeakGBs << std::endl;
   }
+  bool agrees = true;
   if (func) {
     std::vector<OutT> got((size_t)M * N);
     check(hipMemcpy(got.data(), d_out, got.size() * sizeof(OutT), hipMemcpyDeviceToHost), "copy");
@@ -227,11 +239,14 @@ void bench(const Pattern &p, int N, int V, int kernel, bool sorted, bool func, b
       max_ref = std::max(max_ref, std::fabs(host[j]));
       if (d > 0.5f) ++errors;  // the reference's threshold (sspmm_test.cpp:239)
     }
-    if (errors)
-      std::printf("SPMM does not agree with SEQUENTIAL! %d errors! max error: %f\n", errors, max_error);
-    else
-      std::printf("Results verified: they agree. max abs error %g, relative to max |ref| %g\n", max_error,
-                  max_ref > 0 ? max_error / max_ref : 0.0f);
+    const double rel = max_ref > 0 ? max_error / max_ref : max_error;
+    if (errors || rel > relative_tolerance()) {
+      std::printf("SPMM does not agree with SEQUENTIAL! %d errors! max error: %f (%g of max |ref|, tolerance %g)\n", errors,
+                  max_error, rel, relative_tolerance());
+      agrees = false;
+    } else {
+      std::printf("Results verified: they agree. max abs error %g, relative to max |ref| %g\n", max_error, rel);
+    }
   }
   (void)hipFree(d_off);
   (void)hipFree(d_col);
@@ -239,6 +254,7 @@ void bench(const Pattern &p, int N, int V, int kernel, bool sorted, bool func, b
   (void)hipFree(d_val);
   (void)hipFree(d_rhs);
   (void)hipFree(d_out);
+  return agrees;
 }
 
 void usage() {
@@ -257,9 +273,9 @@ int main(int argc, char **argv) {
     const int N = std::atoi(argv[6]);
     const int mixed = argc > 7 ? std::atoi(argv[7]) : 0, func = argc > 8 ? std::atoi(argv[8]) : 1;
     const Pattern p = synthetic_pattern(M, K, V, sparsity, 1);
-    if (mixed) bench<__half>(p, N, V, 1, false, func, false, false, "gfx950");
-    else bench<float>(p, N, V, 1, false, func, false, false, "gfx950");
-    return 0;
+    const bool ok = mixed ? bench<__half>(p, N, V, 1, false, func, false, false, "gfx950")
+                          : bench<float>(p, N, V, 1, false, func, false, false, "gfx950");
+    return ok ? 0 : 2;
   }
   if (argc != 11) usage();
   const std::string paths(argv[1]);
@@ -281,7 +297,7 @@ int main(int argc, char **argv) {
     return 1;
   }
   std::string line;
-  int count = 0;
+  int count = 0, failed = 0;
   while (std::getline(list, line)) {
     if (line.empty()) continue;
     std::cout << "NO." << count << "  matrix:" << std::endl;
@@ -290,10 +306,15 @@ int main(int argc, char **argv) {
       std::fprintf(stderr, "cannot read %s\n", (dir + line).c_str());
       return 1;
     }
-    if (mixed) bench<__half>(p, dimN, V, kernel, sorted, func, record, reorder, arch);
-    else bench<float>(p, dimN, V, kernel, sorted, func, record, reorder, arch);
+    const bool ok = mixed ? bench<__half>(p, dimN, V, kernel, sorted, func, record, reorder, arch)
+                          : bench<float>(p, dimN, V, kernel, sorted, func, record, reorder, arch);
+    if (!ok) ++failed;
     ++count;
   }
   std::printf("matrix num:%d\n", count);
+  if (failed) {
+    std::printf("%d of them disagree with the host loop\n", failed);
+    return 2;
+  }
   return 0;
 }

@@ -843,6 +843,18 @@ static SideStreams *side_streams() {
   return &ss;
 }
 
+// A call that is being recorded into a HIP graph stays on the caller's stream: the helper streams and their
+// events are shared by every call on the device, and pulling them into one stream's capture would tie any other
+// call that forks before the capture ends to that capture.
+static SideStreams *side_streams_for(hipStream_t stream) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+    (void)hipGetLastError();  // (the legacy default stream cannot be asked while another stream captures)
+    status = hipStreamCaptureStatusNone;
+  }
+  return status == hipStreamCaptureStatusNone ? side_streams() : nullptr;
+}
+
 static uint32_t bits_of(int K) {
   uint32_t key_bits = 1;
   while (key_bits < 31 && (1u << key_bits) < (uint32_t)K) ++key_bits;
@@ -877,25 +889,32 @@ static hipError_t join_streams(SideStreams *ss, hipStream_t stream, int helpers 
 hipError_t launch_svc_count(const SvcArgs &a, int order, hipStream_t stream) {
   const int m_vec = (a.M + a.V - 1) / a.V;
   hipError_t e;
-  if (svc_direct(order, a.K)) {
+  if (m_vec == 0) {
+    // no groups: only the scan runs, which writes vec_row_ptr[0] = 0 (and empty class lists)
+  } else if (svc_direct(order, a.K)) {
     const size_t lds = 128 + (size_t)((a.K + 31) / 32) * 4;  // at most 16 KB
     hipLaunchKernelGGL((svc_count_distinct_kernel<256>), dim3(m_vec), dim3(256), lds, stream, a);
     if ((e = hipGetLastError()) != hipSuccess) return e;
   } else if (order == 0) {
     // One pass over the groups per size class, each taking the groups of its class; a group's class
     // is decided from min(non-zeros of the group, K), an upper bound of its distinct columns.
-    SideStreams *ss = side_streams();
+    SideStreams *ss = side_streams_for(stream);
     std::unique_lock<std::mutex> sequence;
     if (ss) sequence = std::unique_lock<std::mutex>(ss->in_use);
     hipStream_t st[4];
     if ((e = fork_streams(ss, stream, st)) != hipSuccess) return e;
-    if ((e = launch_lds_class<64>(a, m_vec, -1, kSmallKeys, 512, st[0])) != hipSuccess) return e;
-    if ((e = launch_lds_class<256>(a, m_vec, kSmallKeys, kMediumKeys, 2048, st[1])) != hipSuccess) return e;
-    if ((e = launch_lds_class<1024>(a, m_vec, kMediumKeys, kLargeKeys, 8192, st[2])) != hipSuccess) return e;
-    hipLaunchKernelGGL((svc_merge_cpython_kernel<1024, false>), dim3(m_vec), dim3(1024), 128, st[3], a, kLargeKeys,
-                       0x7fffffff, 0);
-    if ((e = hipGetLastError()) != hipSuccess) return e;
-    if ((e = join_streams(ss, stream)) != hipSuccess) return e;
+    // (from here on the helpers are joined back into the caller's stream whatever happens)
+    e = launch_lds_class<64>(a, m_vec, -1, kSmallKeys, 512, st[0]);
+    if (e == hipSuccess) e = launch_lds_class<256>(a, m_vec, kSmallKeys, kMediumKeys, 2048, st[1]);
+    if (e == hipSuccess) e = launch_lds_class<1024>(a, m_vec, kMediumKeys, kLargeKeys, 8192, st[2]);
+    if (e == hipSuccess) {
+      hipLaunchKernelGGL((svc_merge_cpython_kernel<1024, false>), dim3(m_vec), dim3(1024), 128, st[3], a, kLargeKeys,
+                         0x7fffffff, 0);
+      e = hipGetLastError();
+    }
+    const hipError_t ej = join_streams(ss, stream);
+    if (e != hipSuccess) return e;
+    if (ej != hipSuccess) return ej;
   } else {
     const int words = (a.K + 31) / 32;
     const size_t lds = 128 + (size_t)words * 8;
@@ -936,11 +955,12 @@ hipError_t launch_svc_fill(const SvcArgs &args, int order, const uint16_t *csr_v
   a.csr_val = csr_val;
   const uint32_t key_bits = bits_of(a.K);
   hipError_t e;
-  SideStreams *ss = side_streams();
+  SideStreams *ss = side_streams_for(stream);
   std::unique_lock<std::mutex> sequence;
   if (ss) sequence = std::unique_lock<std::mutex>(ss->in_use);
   hipStream_t st[4];
   if ((e = fork_streams(ss, stream, st, 1)) != hipSuccess) return e;
+  // (from here on the helper is joined back into the caller's stream whatever happens)
   // Grids: what the chip holds at once for the class's workgroup size and LDS, at most one workgroup per group.
   // The two classes of 1229 .. 4914 and 307 .. 1228 columns share a launch on the caller's stream (1024 threads
   // and 8192-slot tables for both): with one such workgroup per CU resident every group (up to the number of CUs) of either
@@ -949,17 +969,16 @@ hipError_t launch_svc_fill(const SvcArgs &args, int order, const uint16_t *csr_v
   // The many small groups, and the two classes that are nearly always empty, follow each other on one helper
   // stream: one fork and one join.
   const int cus = 256;
-  if ((e = launch_fast_class<1024, true>(a, min(m_vec, cus), 2, 1, kLargeKeys, 8192, key_bits, st[0], 81 * 1024)) !=
-      hipSuccess)
-    return e;
-  if ((e = launch_fast_class<64, true>(a, min(m_vec, 32 * cus), 0, 0, kSmallKeys, 512, key_bits, st[1])) != hipSuccess)
-    return e;
-  if ((e = launch_fast_class<1024, false>(a, min(m_vec, cus), 3, 3, kXLargeKeys, 32768, key_bits, st[1])) != hipSuccess)
-    return e;
-  // more columns than a 32768-slot table takes: 64-bit entries in the workspace
-  hipLaunchKernelGGL((svc_merge_cpython_kernel<1024, false>), dim3(min(m_vec, cus)), dim3(1024), 128, st[1], a, 0, 0, 0);
-  if ((e = hipGetLastError()) != hipSuccess) return e;
-  return join_streams(ss, stream, 1);
+  e = launch_fast_class<1024, true>(a, min(m_vec, cus), 2, 1, kLargeKeys, 8192, key_bits, st[0], 81 * 1024);
+  if (e == hipSuccess) e = launch_fast_class<64, true>(a, min(m_vec, 32 * cus), 0, 0, kSmallKeys, 512, key_bits, st[1]);
+  if (e == hipSuccess) e = launch_fast_class<1024, false>(a, min(m_vec, cus), 3, 3, kXLargeKeys, 32768, key_bits, st[1]);
+  if (e == hipSuccess) {
+    // more columns than a 32768-slot table takes: 64-bit entries in the workspace
+    hipLaunchKernelGGL((svc_merge_cpython_kernel<1024, false>), dim3(min(m_vec, cus)), dim3(1024), 128, st[1], a, 0, 0, 0);
+    e = hipGetLastError();
+  }
+  const hipError_t ej = join_streams(ss, stream, 1);
+  return e != hipSuccess ? e : ej;
 }
 
 }  // namespace sspmm

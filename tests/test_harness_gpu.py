@@ -47,6 +47,13 @@ def test_reference_command_line_on_cvse_files(built_library, tmp_path, V):
     assert len(first) >= 5 and int(first[3]) == 128  # nnz, m_vec, K, N, GFLOP/s, ...
 
 
+def test_a_mismatch_fails_the_run(built_library, tmp_path):
+    """The verification decides the exit status: with a tolerance no fp16 result can meet, the run fails."""
+    r = run(["--synthetic", 256, 256, 8, 0.9, 128, 1, 1], tmp_path, {"SSPMM_REL_TOL": "1e-12"})
+    assert r.returncode == 2, r.stdout
+    assert "does not agree" in r.stdout
+
+
 def test_wrong_argument_count_prints_usage(built_library, tmp_path):
     r = run(["paths.txt", 128], tmp_path)
     assert r.returncode == 1 and "sspmm_test <paths.txt>" in r.stdout

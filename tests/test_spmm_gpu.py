@@ -57,12 +57,57 @@ def test_cfg2_ffn_v8(oracle, kernel, shape, sparsity):
         assert _lib.lib().sspmm_last_kernel() == (5 if kernel == "slab" and shape[1] == 2048 else KERNELS[kernel])
 
 
-@pytest.mark.parametrize("shape,sparsity,N", [((1024, 2304), 0.8, 256), ((2048, 1024), 0.95, 256),
-                                             ((1024, 2304), 0.95, 3136), ((2048, 1024), 0.8, 3136)])
+@pytest.mark.parametrize("shape", [(1024, 2304), (2048, 1024)])
+@pytest.mark.parametrize("sparsity", [0.8, 0.95])
+@pytest.mark.parametrize("N", [256, 3136])
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
 def test_cfg3_conv_v16(oracle, built_library, shape, sparsity, N, out_dtype):
+    """All eight (shape, sparsity, N) points of the im2col configuration."""
     vs = synth.vector_sparse(shape[0], shape[1], 16, sparsity, seed=3, std=0.05)
     check(oracle, vs, synth.dense_rhs(shape[1], N, seed=13), out_dtype)
+
+
+@pytest.mark.parametrize("shape", [(2048, 512), (512, 2048)])
+@pytest.mark.parametrize("sparsity", [0.7, 0.9, 0.98])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
+def test_cfg2_shapes_v16(oracle, built_library, shape, sparsity, out_dtype):
+    vs = synth.vector_sparse(shape[0], shape[1], 16, sparsity, seed=2, std=0.02)
+    check(oracle, vs, synth.dense_rhs(shape[1], 256, seed=12), out_dtype)
+
+
+# the six weights of the BERT-base shaped encoder layer: hidden 768, FFN 3072, 8 x 512 tokens
+CFG5_WEIGHTS = {"q": (768, 768, 51), "k": (768, 768, 52), "v": (768, 768, 53), "o": (768, 768, 54),
+                "ffn1": (3072, 768, 55), "ffn2": (768, 3072, 56)}
+
+
+@pytest.mark.parametrize("name", sorted(CFG5_WEIGHTS))
+@pytest.mark.parametrize("out_dtype", [torch.float16, torch.float32])
+def test_cfg5_encoder_weights_v16_n4096(oracle, built_library, name, out_dtype):
+    """Every weight of the encoder-layer configuration at its real shape: V = 16, 90 %, N = 8 x 512 tokens."""
+    out_f, in_f, seed = CFG5_WEIGHTS[name]
+    vs = synth.vector_sparse(out_f, in_f, 16, 0.9, seed=seed, std=0.02)
+    check(oracle, vs, synth.dense_rhs(in_f, 4096, seed=seed + 100), out_dtype)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
+def test_headline_batch_128_every_element(oracle, built_library, out_dtype):
+    """The launch the benchmark times (A 2048x512, V = 8, 90 %, B 512x256, 128 batch elements that share the
+    pattern, dealt to the XCDs by batch element): every element against the oracle."""
+    from sspmm_amd import _lib
+    V, K, N, batch = 8, 512, 256, 128
+    vs = synth.vector_sparse(2048, K, V, 0.9, seed=2, std=0.02)
+    g = torch.Generator(device="cuda").manual_seed(2)
+    vals = (torch.randn(batch, vs.col_idx.size * V, generator=g, device="cuda") * 0.02).half()
+    B = torch.randn(batch, K, N, generator=g, device="cuda").half()
+    print("headline batch %d out=%s" % (batch, out_dtype), flush=True)
+    out = sspmm_amd.bspmm(None, dev(vs.row_offsets), dev(vs.col_idx), vals, B, V, out_dtype=out_dtype)
+    torch.cuda.synchronize()
+    assert _lib.lib().sspmm_last_kernel() == 3
+    out, vals_h, B_h = out.cpu().numpy(), vals.cpu().numpy(), B.cpu().numpy()
+    tol = TIGHT_F32 if out_dtype == torch.float32 else TIGHT_F16
+    for b in range(batch):
+        want = oracle.spmm(vs.m_vec, V, N, K, vs.row_offsets, vs.col_idx, vals_h[b], B_h[b], threads=8)
+        assert max_rel_err(out[b], want) <= tol, b
 
 
 @pytest.mark.parametrize("V", [8, 16])

@@ -34,7 +34,7 @@ int sspmm_version(void);
  * its preconditions hold.  0 = automatic choice (default), 1 = scalar kernel (any shape),
  * 2 = one-wave gather kernel, 3 = LDS-slab kernel, 6 = the gather kernel's staged form (rows of B
  * fetched whole and passed through LDS; the automatic choice takes it for N <= 64 only) on any
- * width.  The setting belongs to the calling host thread (other threads keep the automatic choice).
+ * width, 7 = the load-balanced gather kernel (products with a plan only; others ignore it).  The setting belongs to the calling host thread (other threads keep the automatic choice).
  * Returns the previous setting, or -1 for an unknown value.
  */
 int sspmm_select_kernel(int which);
@@ -43,7 +43,8 @@ int sspmm_select_kernel(int which);
  * SpMM call of the calling host thread ran, numbered as above, with 4 = the gather kernel's variant for
  * K > 4096 that splits long vector-rows over the waves of a workgroup (selected as 2) and
  * 5 = the LDS-slab kernel with 32-column slabs, for K too tall for 64-column ones (selected
- * as 3); the staged gather kernel reports 6 also where it was chosen automatically; 0 before any
+ * as 3); the staged gather kernel reports 6 also where it was chosen automatically, the load-balanced
+ * kernel 7; 0 before any
  * call of this thread. */
 int sspmm_last_kernel(void);
 
@@ -90,6 +91,54 @@ int sspmm_batched_f16_f32(int batch, int m_vec, int V, int N, int K, const int32
                           const int32_t *row_offsets, const int32_t *col_idx, const sspmm_half_t *values,
                           int64_t stride_values, const sspmm_half_t *B, int64_t stride_B, float *C,
                           int64_t stride_C, void *hip_stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Plans: what the library can know about a sparsity pattern before its first product.
+ *
+ * The reference starts one thread block per vector-row whatever its length (reference
+ * SSpMM/src/sspmm.cu:558-559); its handle on uneven rows is the permutation of SortedRowSwizzle
+ * (reference SSpMM/include/bm_test_utils.h:210-225, applied at end2end/sspmm_e2e/src/cuda/
+ * spmm_kernel.cu:48 and commented out at SSpMM/src/sspmm.cu:248).  A plan replaces that
+ * permutation for callers that keep a pattern: sspmm_plan_create reads row_offsets on the
+ * device, records the number of stored vectors and the longest vector-row, and when some rows
+ * are much longer than the rest builds a schedule in which such rows are cut into panels of
+ * equal work, processed by different workgroups and added up in a fixed order.  Products with
+ * a plan allocate nothing and give the same bits from run to run; a vector-row that was cut
+ * may differ from the product without a plan by the re-association of its fp32 sum.
+ *
+ *   max_N, max_batch  the widest right-hand side and the largest batch the plan will be used
+ *                     with (they size its scratch memory; products beyond them run without the
+ *                     schedule).
+ *   panel_steps       0 lets the library choose; a positive value forces panels of that many
+ *                     steps of 32 vectors (tests and tuning).
+ * sspmm_plan_create synchronises the stream (it sizes its allocation from what the device
+ * found) and must not be called while the stream is being captured; the plan belongs to the
+ * device that was current.  One plan serves one product at a time: two products with the same
+ * plan must not overlap on the device (use one plan per stream).  The pattern handed to a
+ * product must be the one the plan was made from.
+ * ---------------------------------------------------------------------------------------- */
+typedef struct sspmm_plan sspmm_plan_t;
+
+int sspmm_plan_create(int m_vec, int V, int K, const int32_t *row_offsets, int max_N, int max_batch,
+                      int panel_steps, void *hip_stream, sspmm_plan_t **plan);
+
+int sspmm_plan_destroy(sspmm_plan_t *plan);
+
+/* Fills info[0..7] (host memory): stored vectors, steps of the longest vector-row, steps of all
+ * vector-rows, steps per panel, vector-rows that were cut, panels of cut rows, work items,
+ * bytes of device memory the plan holds. */
+int sspmm_plan_info(const sspmm_plan_t *plan, int64_t *info);
+
+/* sspmm_batched_f16_f32 / sspmm_batched_f16_f16 with a plan in place of row_indices (the plan
+ * supplies the processing order); batch = 1 with zero strides is the single product. */
+int sspmm_plan_batched_f16_f32(const sspmm_plan_t *plan, int batch, int N, const int32_t *row_offsets,
+                               const int32_t *col_idx, const sspmm_half_t *values, int64_t stride_values,
+                               const sspmm_half_t *B, int64_t stride_B, float *C, int64_t stride_C, void *hip_stream);
+
+int sspmm_plan_batched_f16_f16(const sspmm_plan_t *plan, int batch, int N, const int32_t *row_offsets,
+                               const int32_t *col_idx, const sspmm_half_t *values, int64_t stride_values,
+                               const sspmm_half_t *B, int64_t stride_B, sspmm_half_t *C, int64_t stride_C,
+                               void *hip_stream);
 
 /*
  * row_indices = vector-rows ordered by descending length (ties: ascending row).  Replaces

@@ -9,6 +9,7 @@ All compute runs in hand-written HIP kernels reached through the C ABI of libssp
 operator raises.
 """
 from .spmm import spmm, bspmm, sorted_row_swizzle  # noqa: F401
+from .plan import Plan, PlanInfo  # noqa: F401
 from .svc import svc, SvcResult  # noqa: F401
 from .attention import sddmm, bsddmm, csr_softmax, bcsr_softmax, sparse_attention  # noqa: F401
 from .reorder import minhash_order, permute_csr, svc_reordered  # noqa: F401

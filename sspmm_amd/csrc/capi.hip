@@ -4,6 +4,7 @@
 
 #include "../../include/sspmm.h"
 #include "attention_kernels.h"
+#include "plan.h"
 #include "reorder_kernels.h"
 #include "spmm_kernels.h"
 #include "svc_kernels.h"
@@ -14,7 +15,8 @@ constexpr int kInvalid = (int)hipErrorInvalidValue;
 
 int spmm_entry(int batch, int m_vec, int V, int N, int K, const int32_t *row_indices, const int32_t *row_offsets,
                const int32_t *col_idx, const sspmm_half_t *values, int64_t stride_values, const sspmm_half_t *B,
-               int64_t stride_B, void *C, int64_t stride_C, bool out_f16, void *stream) {
+               int64_t stride_B, void *C, int64_t stride_C, bool out_f16, void *stream,
+               const sspmm::Plan *plan = nullptr) {
   if (V != 8 && V != 16) return kInvalid;
   if (batch < 0 || m_vec < 0 || N < 0 || K < 0) return kInvalid;
   if (batch == 0 || m_vec == 0 || N == 0) return 0;  // nothing to write
@@ -40,7 +42,19 @@ int spmm_entry(int batch, int m_vec, int V, int N, int K, const int32_t *row_ind
   a.stride_values = stride_values;
   a.stride_B = stride_B;
   a.stride_C = stride_C;
+  if (plan) return (int)sspmm::launch_spmm_planned(*plan, a, out_f16, static_cast<hipStream_t>(stream));
   return (int)sspmm::launch_spmm(a, V, out_f16, static_cast<hipStream_t>(stream));
+}
+
+int plan_entry(const sspmm_plan_t *plan, int batch, int N, const int32_t *row_offsets, const int32_t *col_idx,
+               const sspmm_half_t *values, int64_t stride_values, const sspmm_half_t *B, int64_t stride_B, void *C,
+               int64_t stride_C, bool out_f16, void *stream) {
+  if (!plan) return kInvalid;
+  const sspmm::Plan *pl = reinterpret_cast<const sspmm::Plan *>(plan);
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev != pl->device) return kInvalid;  // the plan's memory lives on its device
+  return spmm_entry(batch, pl->m_vec, pl->V, N, pl->K, nullptr, row_offsets, col_idx, values, stride_values, B, stride_B,
+                    C, stride_C, out_f16, stream, pl);
 }
 
 }  // namespace
@@ -50,7 +64,7 @@ extern "C" {
 int sspmm_version(void) { return (0 << 16) | 1; }
 
 int sspmm_select_kernel(int which) {
-  if (which < 0 || (which > 3 && which != 6)) return -1;
+  if (which < 0 || (which > 3 && which != 6 && which != 7)) return -1;
   return sspmm::set_kernel_override(which);
 }
 
@@ -88,6 +102,55 @@ int sspmm_batched_f16_f32(int batch, int m_vec, int V, int N, int K, const int32
                           int64_t stride_C, void *hip_stream) {
   return spmm_entry(batch, m_vec, V, N, K, row_indices, row_offsets, col_idx, values, stride_values, B, stride_B, C,
                     stride_C, false, hip_stream);
+}
+
+int sspmm_plan_create(int m_vec, int V, int K, const int32_t *row_offsets, int max_N, int max_batch, int panel_steps,
+                      void *hip_stream, sspmm_plan_t **plan) {
+  if (!plan) return kInvalid;
+  *plan = nullptr;
+  if (V != 8 && V != 16) return kInvalid;
+  if (m_vec < 0 || K < 0 || max_N < 0 || max_batch < 0 || panel_steps < 0) return kInvalid;
+  if (m_vec > 0 && !row_offsets) return kInvalid;
+  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capturing) != hipSuccess) {
+    (void)hipGetLastError();
+    return kInvalid;
+  }
+  if (capturing != hipStreamCaptureStatusNone) return kInvalid;  // it allocates and synchronises
+  sspmm::Plan *pl = nullptr;
+  const hipError_t e = sspmm::plan_create(m_vec, V, K, row_offsets, max_N, max_batch, panel_steps, stream, &pl);
+  *plan = reinterpret_cast<sspmm_plan_t *>(pl);
+  return (int)e;
+}
+
+int sspmm_plan_destroy(sspmm_plan_t *plan) { return (int)sspmm::plan_destroy(reinterpret_cast<sspmm::Plan *>(plan)); }
+
+int sspmm_plan_info(const sspmm_plan_t *plan, int64_t *info) {
+  if (!plan || !info) return kInvalid;
+  const sspmm::Plan *pl = reinterpret_cast<const sspmm::Plan *>(plan);
+  info[0] = pl->header[sspmm::kHdrNvec];
+  info[1] = pl->header[sspmm::kHdrMaxSteps];
+  info[2] = pl->header[sspmm::kHdrTotalSteps];
+  info[3] = pl->header[sspmm::kHdrBudget];
+  info[4] = pl->header[sspmm::kHdrSplitRows];
+  info[5] = pl->header[sspmm::kHdrSlots];
+  info[6] = pl->header[sspmm::kHdrItems];
+  info[7] = (int64_t)pl->bytes;
+  return 0;
+}
+
+int sspmm_plan_batched_f16_f32(const sspmm_plan_t *plan, int batch, int N, const int32_t *row_offsets,
+                               const int32_t *col_idx, const sspmm_half_t *values, int64_t stride_values,
+                               const sspmm_half_t *B, int64_t stride_B, float *C, int64_t stride_C, void *hip_stream) {
+  return plan_entry(plan, batch, N, row_offsets, col_idx, values, stride_values, B, stride_B, C, stride_C, false, hip_stream);
+}
+
+int sspmm_plan_batched_f16_f16(const sspmm_plan_t *plan, int batch, int N, const int32_t *row_offsets,
+                               const int32_t *col_idx, const sspmm_half_t *values, int64_t stride_values,
+                               const sspmm_half_t *B, int64_t stride_B, sspmm_half_t *C, int64_t stride_C,
+                               void *hip_stream) {
+  return plan_entry(plan, batch, N, row_offsets, col_idx, values, stride_values, B, stride_B, C, stride_C, true, hip_stream);
 }
 
 int sspmm_sorted_row_swizzle(int m_vec, const int32_t *row_offsets, int32_t *row_indices, void *hip_stream) {

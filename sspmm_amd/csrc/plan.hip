@@ -1,0 +1,108 @@
+// The plan object of the SpMM: what is worth knowing about a sparsity pattern before its first
+// product, computed once (on the device, from the row offsets) and owned by the library.
+//
+// It holds the pattern's statistics (stored vectors, longest vector-row), which the asynchronous
+// entry points without a plan cannot see because the row offsets live in device memory, and the
+// row-panel schedule with its scratch memory (schedule.h), so that products with a plan allocate
+// nothing.
+#include "plan.h"
+
+#include <new>
+
+namespace sspmm {
+
+static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+// Scratch memory for partial tiles a plan may take; beyond it the budget is doubled until the panels fit.
+static constexpr size_t kPlanPartialCap = (size_t)64 << 20;
+
+int64_t schedule_slot_cap(size_t partial_bytes, int V, int N, int batch) {
+  const int64_t tiles = ((int64_t)N + 63) / 64;
+  const int64_t per_slot = (int64_t)partial_tile_bytes(V) * (tiles > 0 ? tiles : 1) * (batch > 0 ? batch : 1);
+  return (int64_t)partial_bytes / per_slot;
+}
+
+hipError_t plan_create(int m_vec, int V, int K, const int32_t *row_offsets, int max_N, int max_batch, int budget,
+                       hipStream_t stream, Plan **out) {
+  *out = nullptr;
+  Plan *pl = new (std::nothrow) Plan();
+  if (!pl) return hipErrorOutOfMemory;
+  hipError_t e = hipGetDevice(&pl->device);
+  if (e != hipSuccess) {
+    delete pl;
+    return e;
+  }
+  pl->m_vec = m_vec;
+  pl->V = V;
+  pl->K = K;
+  pl->max_N = max_N;
+  pl->max_batch = max_batch;
+  pl->tiles_max = (max_N + 63) / 64;
+  for (int i = 0; i < kHdrWords; ++i) pl->header[i] = 0;
+  if (m_vec == 0) {
+    *out = pl;
+    return hipSuccess;
+  }
+  int32_t *d_header = nullptr;
+  if ((e = hipMalloc(reinterpret_cast<void **>(&d_header), 256)) != hipSuccess) {
+    delete pl;
+    return e;
+  }
+  const int64_t slot_cap = schedule_slot_cap(kPlanPartialCap, V, max_N, max_batch);
+  e = launch_schedule_measure(m_vec, row_offsets, budget, slot_cap, d_header, stream);
+  if (e == hipSuccess) e = hipMemcpyAsync(pl->header, d_header, sizeof(pl->header), hipMemcpyDeviceToHost, stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(stream);
+  (void)hipFree(d_header);
+  if (e != hipSuccess) {
+    delete pl;
+    return e;
+  }
+  const size_t n_items = (size_t)pl->header[kHdrItems], n_split = (size_t)pl->header[kHdrSplitRows];
+  const size_t n_slots = (size_t)pl->header[kHdrSlots];
+  const size_t units = (size_t)(pl->tiles_max > 0 ? pl->tiles_max : 1) * (size_t)(max_batch > 0 ? max_batch : 1);
+  const size_t off_items = 256;
+  const size_t off_counters = off_items + align256(n_items * sizeof(ScheduleItem));
+  pl->counters = n_split * units;
+  const size_t off_partials = off_counters + align256(pl->counters * 4);
+  pl->bytes = off_partials + align256(n_slots * units * partial_tile_bytes(V));
+  if ((e = hipMalloc(&pl->memory, pl->bytes)) != hipSuccess) {
+    delete pl;
+    return e;
+  }
+  unsigned char *base = static_cast<unsigned char *>(pl->memory);
+  pl->view.header = reinterpret_cast<int32_t *>(base);
+  pl->view.items = reinterpret_cast<ScheduleItem *>(base + off_items);
+  pl->view.counters = reinterpret_cast<int32_t *>(base + off_counters);
+  pl->view.partials = base + off_partials;
+  e = hipMemcpyAsync(pl->view.header, pl->header, sizeof(pl->header), hipMemcpyHostToDevice, stream);
+  if (e == hipSuccess) e = launch_schedule_fill(m_vec, row_offsets, pl->view, (int64_t)n_items, (int64_t)pl->counters, stream);
+  if (e == hipSuccess) e = hipStreamSynchronize(stream);  // products with the plan may come on any stream
+  if (e != hipSuccess) {
+    (void)hipFree(pl->memory);
+    delete pl;
+    return e;
+  }
+  *out = pl;
+  return hipSuccess;
+}
+
+hipError_t plan_destroy(Plan *pl) {
+  if (!pl) return hipSuccess;
+  hipError_t e = hipSuccess;
+  if (pl->memory) e = hipFree(pl->memory);
+  delete pl;
+  return e;
+}
+
+hipError_t launch_spmm_planned(const Plan &pl, const SpmmArgs &a, bool out_f16, hipStream_t stream) {
+  const int forced = kernel_override();
+  const bool can_balance = balanced_kernel_applies(a, pl.V, out_f16) && a.N <= pl.max_N && a.batch <= pl.max_batch;
+  // Rows are cut only when some row is much longer than the rest (the budget is at least twice the mean row):
+  // an even pattern keeps the kernels chosen by shape.
+  const bool skewed = pl.header[kHdrSplitRows] > 0;
+  if (can_balance && (forced == 7 || (forced == 0 && skewed)))
+    return launch_spmm_balanced(a, pl.V, out_f16, pl.view, pl.header[kHdrItems], stream);
+  return launch_spmm(a, pl.V, out_f16, stream);
+}
+
+}  // namespace sspmm

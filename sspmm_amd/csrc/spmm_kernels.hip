@@ -27,6 +27,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "schedule.h"
 #include "spmm_kernels.h"
 
 namespace sspmm {
@@ -1132,6 +1133,102 @@ struct StageBody {
   typename SlabVals<V>::type vraw;
 };
 
+// Per-lane constants of the staged gather: where the lane writes its share of the staged rows and of the value
+// tile, and where its transpose reads start.
+template <int V>
+struct StageLane {
+  int j, pc;            // the lane fetches 16-byte piece pc of the rows named by k slots 4j .. 4j+3
+  uint32_t vals_lane_off, a_off, b_rd;
+  unsigned char *tile_dst, *stage_dst;
+  const unsigned char *val_tile;
+  __device__ __forceinline__ void init(int lane, unsigned char *stage, unsigned char *tile) {
+    const int m = lane & 15, g = lane >> 4;
+    j = lane >> 3;
+    pc = lane & 7;
+    constexpr uint32_t kLaneBytes = V * 2u * 32u / 64u;
+    vals_lane_off = (uint32_t)lane * kLaneBytes;
+    val_tile = tile;
+    tile_dst = tile + lane * kLaneBytes;
+    stage_dst = stage + (uint32_t)(4 * j) * kStagePitch + (uint32_t)pc * 16u;
+    // transpose reads: k slots 8g + m/4 (and + 4) of the value tile and of the staged rows
+    a_off = (uint32_t)(8 * g + (m >> 2)) * (V * 2u) + (uint32_t)(m & 3) * 8u;
+    b_rd = lds_address(stage) + (uint32_t)(8 * g + (m >> 2)) * kStagePitch + (uint32_t)(m & 3) * 8u;
+  }
+};
+
+// acc += the V x 64 tile of vectors [beg, end) of a vector-row against columns ncol0 .. of B.  srd_cols and
+// srd_vals end at vector `end`: slots past it read as zero.  Lane (m, g) ends up with columns 16q + 4g .. + 3 of
+// output row m in acc[q] (the staged rows are the MFMA's first operand, as the slab is in the slab kernel).
+template <int V>
+__device__ __forceinline__ void stage_accumulate(floatx4 (&acc)[4], const StageLane<V> &x, __amdgpu_buffer_rsrc_t srd_cols,
+                                                 __amdgpu_buffer_rsrc_t srd_vals, __amdgpu_buffer_rsrc_t srd_b, int beg,
+                                                 int end, uint32_t lane_n2, uint32_t lane_col_off, uint32_t b_bytes) {
+  const auto load_head = [&](StageHead<V> &h, int kc) {
+    h.kc = kc;
+    h.cols = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_cols, (kc + 4 * x.j) * 4, 0, 0));
+    h.vraw = SlabVals<V>::load(srd_vals, (uint32_t)kc * (V * 2u) + x.vals_lane_off);
+  };
+  const auto load_body = [&](StageBody<V> &c, const StageHead<V> &h) {
+    uint32_t off[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) off[i] = __umul24(h.cols[i], lane_n2) + lane_col_off;
+    if (h.kc + 32 > end) {  // wave-uniform: only the last chunk of a vector-row can be partial
+#pragma unroll
+      for (int i = 0; i < 4; ++i) off[i] = (h.kc + 4 * x.j + i < end) ? off[i] : b_bytes;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      c.piece[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_b, off[i], 0, 0));
+    c.vraw = h.vraw;
+  };
+  const auto contract = [&](const StageBody<V> &c) {
+    // (LDS operations of a wave execute in order: these writes land behind the previous chunk's reads)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<uintx4 *>(x.stage_dst + i * kStagePitch) = c.piece[i];
+    *reinterpret_cast<typename SlabVals<V>::type *>(x.tile_dst) = c.vraw;
+    Half8Bits a;
+    {
+      const uintx2 lo = lds_read_tr(x.val_tile, x.a_off);
+      const uintx2 hi = lds_read_tr(x.val_tile, x.a_off + 4u * (V * 2u));
+      a.u[0] = lo[0]; a.u[1] = lo[1]; a.u[2] = hi[0]; a.u[3] = hi[1];
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      Half8Bits b;
+      const uintx2 lo = lds_read_tr_abs(x.b_rd + 32u * q);
+      const uintx2 hi = lds_read_tr_abs(x.b_rd + 4u * kStagePitch + 32u * q);
+      b.u[0] = lo[0]; b.u[1] = lo[1]; b.u[2] = hi[0]; b.u[3] = hi[1];
+      acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b.h, a.h, acc[q], 0, 0, 0);
+    }
+  };
+  if (beg >= end) return;
+  // Heads run two chunks ahead of the arithmetic, bodies one (two of each, used alternately).
+  StageHead<V> h0, h1;
+  StageBody<V> c0, c1;
+  load_head(h0, beg);
+  load_head(h1, beg + 32);
+  load_body(c0, h0);
+  int kc = beg + 32;  // first vector of the chunk whose body is loaded next
+  for (;;) {
+    if (kc >= end) {
+      contract(c0);
+      break;
+    }
+    load_head(h0, kc + 32);
+    load_body(c1, h1);
+    contract(c0);
+    kc += 32;
+    if (kc >= end) {
+      contract(c1);
+      break;
+    }
+    load_head(h1, kc + 32);
+    load_body(c0, h0);
+    contract(c1);
+    kc += 32;
+  }
+}
+
 template <int V, typename OutT>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(V == 8 ? 5 : 4, V == 8 ? 5 : 4))) void spmm_stage_kernel(const SpmmArgs p) {
   __shared__ __align__(16) unsigned char stage[32 * kStagePitch];
@@ -1146,7 +1243,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(V == 8 ? 5 :
   const int row = __builtin_amdgcn_readfirstlane(p.row_indices ? p.row_indices[r] : (int)r);
 
   const int lane = threadIdx.x;
-  const int m = lane & 15, g = lane >> 4, j = lane >> 3, pc = lane & 7;
+  StageLane<V> x;
+  x.init(lane, stage, val_tile);
   const int beg = p.row_offsets[row], end = p.row_offsets[row + 1];
 
   const uint16_t *vals = p.values + (int64_t)batch * p.stride_values;
@@ -1157,89 +1255,14 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(V == 8 ? 5 :
   const __amdgpu_buffer_rsrc_t srd_b = make_srd(p.B + (int64_t)batch * p.stride_B, b_bytes);
 
   // Lanes whose columns lie beyond N aim every gather at the first byte past B, where loads return zero.
-  const int ncol = (int)tile * 64 + 8 * pc;
+  const int ncol = (int)tile * 64 + 8 * x.pc;
   const bool col_ok = ncol < p.N;
   const uint32_t lane_n2 = col_ok ? (uint32_t)p.N * 2u : 0u;
   const uint32_t lane_col_off = col_ok ? (uint32_t)ncol * 2u : b_bytes;
-  constexpr uint32_t kLaneBytes = V * 2u * 32u / 64u;
-  const uint32_t vals_lane_off = (uint32_t)lane * kLaneBytes;
-  unsigned char *const tile_dst = val_tile + lane * kLaneBytes;
-  unsigned char *const stage_dst = stage + (uint32_t)(4 * j) * kStagePitch + (uint32_t)pc * 16u;
-  // transpose reads: k slots 8g + m/4 (and + 4) of the value tile and of the staged rows
-  const uint32_t a_off = (uint32_t)(8 * g + (m >> 2)) * (V * 2u) + (uint32_t)(m & 3) * 8u;
-  const uint32_t b_rd = lds_address(stage) + (uint32_t)(8 * g + (m >> 2)) * kStagePitch + (uint32_t)(m & 3) * 8u;
-
-  const auto load_head = [&](StageHead<V> &h, int kc) {
-    h.kc = kc;
-    h.cols = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_cols, (kc + 4 * j) * 4, 0, 0));
-    h.vraw = SlabVals<V>::load(srd_vals, (uint32_t)kc * (V * 2u) + vals_lane_off);
-  };
-  const auto load_body = [&](StageBody<V> &c, const StageHead<V> &h) {
-    uint32_t off[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) off[i] = __umul24(h.cols[i], lane_n2) + lane_col_off;
-    if (h.kc + 32 > end) {  // wave-uniform: only the last chunk of a vector-row can be partial
-#pragma unroll
-      for (int i = 0; i < 4; ++i) off[i] = (h.kc + 4 * j + i < end) ? off[i] : b_bytes;
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      c.piece[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_b, off[i], 0, 0));
-    c.vraw = h.vraw;
-  };
   floatx4 acc[4];
 #pragma unroll
   for (int q = 0; q < 4; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
-  const auto contract = [&](const StageBody<V> &c) {
-    // (LDS operations of a wave execute in order: these writes land behind the previous chunk's reads)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) *reinterpret_cast<uintx4 *>(stage_dst + i * kStagePitch) = c.piece[i];
-    *reinterpret_cast<typename SlabVals<V>::type *>(tile_dst) = c.vraw;
-    Half8Bits a;
-    {
-      const uintx2 lo = lds_read_tr(val_tile, a_off);
-      const uintx2 hi = lds_read_tr(val_tile, a_off + 4u * (V * 2u));
-      a.u[0] = lo[0]; a.u[1] = lo[1]; a.u[2] = hi[0]; a.u[3] = hi[1];
-    }
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      Half8Bits b;
-      const uintx2 lo = lds_read_tr_abs(b_rd + 32u * q);
-      const uintx2 hi = lds_read_tr_abs(b_rd + 4u * kStagePitch + 32u * q);
-      b.u[0] = lo[0]; b.u[1] = lo[1]; b.u[2] = hi[0]; b.u[3] = hi[1];
-      // the staged rows are the first operand, as the slab is in the slab kernel: lane (m, g) ends up with
-      // columns 16q + 4g .. + 3 of output row m
-      acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b.h, a.h, acc[q], 0, 0, 0);
-    }
-  };
-
-  if (beg < end) {
-    // Heads run two chunks ahead of the arithmetic, bodies one (two of each, used alternately).
-    StageHead<V> h0, h1;
-    StageBody<V> c0, c1;
-    load_head(h0, beg);
-    load_head(h1, beg + 32);
-    load_body(c0, h0);
-    int kc = beg + 32;  // first vector of the chunk whose body is loaded next
-    for (;;) {
-      if (kc >= end) {
-        contract(c0);
-        break;
-      }
-      load_head(h0, kc + 32);
-      load_body(c1, h1);
-      contract(c0);
-      kc += 32;
-      if (kc >= end) {
-        contract(c1);
-        break;
-      }
-      load_head(h1, kc + 32);
-      load_body(c0, h0);
-      contract(c1);
-      kc += 32;
-    }
-  }
+  stage_accumulate<V>(acc, x, srd_cols, srd_vals, srd_b, beg, end, lane_n2, lane_col_off, b_bytes);
 
   SlabStore<V, OutT, 4> out;
   out.init(lane, (int)tile * 64, p.N);
@@ -1248,6 +1271,151 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(V == 8 ? 5 :
   const __amdgpu_buffer_rsrc_t srd_c = make_srd(reinterpret_cast<OutT *>(p.C) + (int64_t)batch * p.stride_C,
                                                 (uint32_t)p.m_vec * c_vrow_bytes);
   out.store(acc, srd_c, (uint32_t)row * c_vrow_bytes);
+}
+
+// ------------------------------------------------------------------------------------------
+// Load-balanced kernel: the work list is a schedule (schedule.h) instead of the vector-rows.
+//
+// One wave per (work item, 64-column tile).  An item is at most `budget` steps of one vector-row, so
+// every wave of the grid has about the same amount to do whatever the row lengths are, and the
+// hardware's workgroup dispatcher hands items to CUs as waves retire.  The panels of a cut row leave
+// their accumulators in scratch memory as they lie in registers; each then counts itself in on the
+// row's counter, and the wave that finds all the others counted adds the partial tiles up in panel
+// order (its own from memory too, so that the sum has one order whichever wave does it), stores the
+// row of C and puts the counter back to zero for the next launch.  No wave ever waits for another.
+//
+// The inner loop is the staged gather's (rows of B fetched as whole 128-byte lines by eight lanes each,
+// passed through a per-wave LDS tile to the transpose reads): its 100 registers instead of the
+// register-path kernel's 190 keep twice as many waves on a CU.  (Deeper prefetch was measured and
+// does not pay: a grid of panels is bound by the rate at which the CUs' address units take load
+// instructions, 16 cycles per 16-byte load of a wave, and every load issued past the end of a short
+// row costs that too.)
+//
+// Work id -> (batch element, item, column tile) with the tile index fastest and the tile count padded
+// to 1, 2, 4 or a multiple of 8 (padding tiles return at once): workgroup ids go round-robin to the 8
+// XCDs, so an XCD sees only the column tiles congruent to it and keeps their slab of B in its L2,
+// while the items are dealt evenly over the XCDs that share a tile.
+struct BalancedArgs {
+  const int32_t *header;
+  const ScheduleItem *items;
+  int32_t *counters;
+  unsigned char *partials;
+  int n_items;            // what the host knows the schedule to hold, or -1: read the header (grid-stride loop)
+  uint32_t tiles_padded;
+};
+
+// Partial tiles travel between workgroups that may sit on different XCDs, each with an L2 of its own.  They are
+// written and read with device-scope accesses (the sc1 bit, what a device-scope atomic store or load carries:
+// stores go through to memory and are complete when the wave's store counter says so, loads are served from
+// there), as the counter's atomics are.  Release and acquire fences in their place write back and invalidate a
+// whole L2 for every panel (measured on 2048 rows with 1000 panels: 35 us per launch for the former, 5 us for the
+// latter, in a kernel of 18 us).
+static constexpr int kDeviceScope = 16;  // cache-policy bit sc1 of the buffer instructions
+
+// acc[q] of lane (m, g) = columns 16q + 4g .. + 3 of output row m; with V = 8 the lanes m >= 8 hold nothing.
+template <int V>
+struct PartialTile {
+  static constexpr uint32_t kLanes = V == 8 ? 32u : 64u;
+  static __device__ __forceinline__ uint32_t lane_offset(int lane) {
+    const int m = lane & 15, g = lane >> 4;
+    if (V == 8) return m < 8 ? (uint32_t)(g * 8 + m) * 16u : 0x80000000u;  // (beyond the descriptor: dropped / zeros)
+    return (uint32_t)lane * 16u;
+  }
+  static __device__ __forceinline__ void store(__amdgpu_buffer_rsrc_t srd, uint32_t tile_off, const floatx4 (&acc)[4], int lane) {
+    const uint32_t off = tile_off + lane_offset(lane);
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uintx4, acc[q]), srd, off + (uint32_t)q * (kLanes * 16u), 0, kDeviceScope);
+  }
+  static __device__ __forceinline__ void add(__amdgpu_buffer_rsrc_t srd, uint32_t tile_off, floatx4 (&acc)[4], int lane) {
+    const uint32_t off = tile_off + lane_offset(lane);
+    floatx4 x[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      x[q] = __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(srd, off + (uint32_t)q * (kLanes * 16u), 0, kDeviceScope));
+#pragma unroll
+    for (int q = 0; q < 4; ++q) acc[q] += x[q];
+  }
+};
+static_assert(PartialTile<8>::kLanes * 64u == partial_tile_bytes(8) && PartialTile<16>::kLanes * 64u == partial_tile_bytes(16),
+              "a partial tile is four 16-byte pieces per lane that holds rows");
+
+// PERSISTENT: a fixed grid walks the work ids (the number of items is only known on the device).
+template <int V, typename OutT, bool PERSISTENT>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void spmm_balanced_kernel(const SpmmArgs p, const BalancedArgs s) {
+  __shared__ __align__(16) unsigned char stage[32 * kStagePitch];
+  __shared__ __align__(16) unsigned char val_tile[val_tile_bytes(V)];
+  const int lane = threadIdx.x;
+  StageLane<V> x;
+  x.init(lane, stage, val_tile);
+  const uint32_t n_items = PERSISTENT ? (uint32_t)s.header[kHdrItems] : (uint32_t)s.n_items;
+  const uint32_t per_batch = n_items * s.tiles_padded;
+  const uint32_t n_units = per_batch * (uint32_t)p.batch;  // (below 2^31: the launcher checks, or bounds, it)
+  const uint32_t b_bytes = (uint32_t)p.K * (uint32_t)p.N * 2u;
+  const uint32_t c_vrow_bytes = (uint32_t)V * (uint32_t)p.N * (uint32_t)sizeof(OutT);
+
+  for (uint32_t id = blockIdx.x; id < n_units; id += gridDim.x) {
+    const uint32_t batch = id / per_batch, rem = id % per_batch;
+    const uint32_t tile = rem % s.tiles_padded;
+    if (tile >= p.n_tiles) {
+      if (PERSISTENT) continue;
+      return;
+    }
+    const ScheduleItem *ip = s.items + rem / s.tiles_padded;
+    // (the item is the same for the whole wave: scalar registers)
+    const int row = __builtin_amdgcn_readfirstlane(ip->row), kbeg = __builtin_amdgcn_readfirstlane(ip->kbeg),
+              kend = __builtin_amdgcn_readfirstlane(ip->kend), split_id = __builtin_amdgcn_readfirstlane(ip->split_id);
+
+    // the descriptors of the pattern and the values end at the panel's last vector: slots past it read as zero
+    const __amdgpu_buffer_rsrc_t srd_cols = make_srd(p.col_idx, (uint32_t)kend * 4u);
+    const __amdgpu_buffer_rsrc_t srd_vals = make_srd(p.values + (int64_t)batch * p.stride_values, (uint32_t)kend * (V * 2u));
+    const __amdgpu_buffer_rsrc_t srd_b = make_srd(p.B + (int64_t)batch * p.stride_B, b_bytes);
+    // Lanes whose columns lie beyond N aim every gather at the first byte past B, where loads return zero.
+    const int ncol = (int)tile * 64 + 8 * x.pc;
+    const bool col_ok = ncol < p.N;
+    const uint32_t lane_n2 = col_ok ? (uint32_t)p.N * 2u : 0u;
+    const uint32_t lane_col_off = col_ok ? (uint32_t)ncol * 2u : b_bytes;
+    floatx4 acc[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
+    stage_accumulate<V>(acc, x, srd_cols, srd_vals, srd_b, kbeg, kend, lane_n2, lane_col_off, b_bytes);
+
+    if (split_id >= 0) {
+      const uint32_t n_slots = (uint32_t)s.header[kHdrSlots], n_split = (uint32_t)s.header[kHdrSplitRows];
+      const int first_slot = __builtin_amdgcn_readfirstlane(ip->first_slot), pieces = __builtin_amdgcn_readfirstlane(ip->pieces),
+                piece = __builtin_amdgcn_readfirstlane(ip->piece);
+      const size_t unit = (size_t)batch * p.n_tiles + tile;
+      // the partial tiles of this row for this column tile and batch element (one descriptor)
+      const __amdgpu_buffer_rsrc_t srd_part =
+          make_srd(s.partials + (unit * n_slots + (uint32_t)first_slot) * partial_tile_bytes(V),
+                   (uint32_t)pieces * (uint32_t)partial_tile_bytes(V));
+      PartialTile<V>::store(srd_part, (uint32_t)piece * (uint32_t)partial_tile_bytes(V), acc, lane);
+      // the tile has reached memory before the panel counts itself in
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      int32_t *counter = s.counters + unit * n_split + (uint32_t)split_id;
+      int seen = 0;
+      if (lane == 0) seen = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      seen = __builtin_amdgcn_readfirstlane(seen);
+      if (seen != pieces - 1) {  // other panels of the row are still out: the last one adds up
+        if (PERSISTENT) continue;
+        return;
+      }
+      asm volatile("" ::: "memory");  // the loads below stay behind the count
+      if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+      for (int pc = 0; pc < pieces; ++pc)
+        PartialTile<V>::add(srd_part, (uint32_t)pc * (uint32_t)partial_tile_bytes(V), acc, lane);
+    }
+    SlabStore<V, OutT, 4> out;
+    out.init(lane, (int)tile * 64, p.N);
+    // One buffer descriptor spans this batch element's C (the launcher checks it is at most 2 GiB).
+    const __amdgpu_buffer_rsrc_t srd_c = make_srd(reinterpret_cast<OutT *>(p.C) + (int64_t)batch * p.stride_C,
+                                                  (uint32_t)p.m_vec * c_vrow_bytes);
+    out.store(acc, srd_c, (uint32_t)row * c_vrow_bytes);
+    if (!PERSISTENT) return;
+  }
 }
 
 // Shape-agnostic kernel: any N, any alignment.  One thread per output column, scalar gathers,
@@ -1285,6 +1453,8 @@ static thread_local int g_kernel_override = 0;  // 0 auto, 1 generic, 2 gather, 
 
 static thread_local int g_last_kernel = 0;  // kernel of this thread's latest launch
 int last_kernel() { return g_last_kernel; }
+
+int kernel_override() { return g_kernel_override; }
 
 int set_kernel_override(int which) {
   const int old = g_kernel_override;
@@ -1424,17 +1594,67 @@ static hipError_t launch_v(const SpmmArgs &a, int which, hipStream_t stream) {
   return hipGetLastError();
 }
 
-hipError_t launch_spmm(const SpmmArgs &a, int V, bool out_f16, hipStream_t stream) {
-  // The MFMA kernels need 16-byte row segments of B and C: N % 8 == 0 and aligned bases/strides;
-  // 24-bit multiplies bound K and 2N; one buffer descriptor must span B.
+// The MFMA kernels need 16-byte row segments of B and C: N % 8 == 0 and aligned bases/strides;
+// 24-bit multiplies bound K and 2N; one buffer descriptor must span B.
+static bool mfma_kernels_apply(const SpmmArgs &a, bool out_f16) {
   const uint64_t b_bytes = (uint64_t)a.K * (uint64_t)a.N * 2u;
   const int out_size = out_f16 ? 2 : 4;
   // The value vectors are fetched with 8-byte (V = 8) or 16-byte (V = 16) loads per lane.
-  const bool fast = (a.N % 8 == 0) && (reinterpret_cast<uintptr_t>(a.B) % 16 == 0) &&
-                    (reinterpret_cast<uintptr_t>(a.C) % 16 == 0) && (a.stride_B % 8 == 0) &&
-                    (reinterpret_cast<uintptr_t>(a.values) % 16 == 0) && (a.stride_values % 8 == 0) &&
-                    ((a.stride_C * out_size) % 16 == 0) && (a.K < (1 << 24)) && (a.N < (1 << 23)) &&
-                    (b_bytes + 16 <= 0xffffffffull);
+  return (a.N % 8 == 0) && (reinterpret_cast<uintptr_t>(a.B) % 16 == 0) &&
+         (reinterpret_cast<uintptr_t>(a.C) % 16 == 0) && (a.stride_B % 8 == 0) &&
+         (reinterpret_cast<uintptr_t>(a.values) % 16 == 0) && (a.stride_values % 8 == 0) &&
+         ((a.stride_C * out_size) % 16 == 0) && (a.K < (1 << 24)) && (a.N < (1 << 23)) &&
+         (b_bytes + 16 <= 0xffffffffull);
+}
+
+static uint32_t padded_tiles(uint32_t t) { return t <= 1u ? 1u : t <= 2u ? 2u : t <= 4u ? 4u : (t + 7u) & ~7u; }
+
+bool balanced_kernel_applies(const SpmmArgs &a, int V, bool out_f16) {
+  // (one batch element's C is addressed through a 32-bit buffer descriptor, and lanes that must not store carry an
+  // offset of 2 GiB)
+  return mfma_kernels_apply(a, out_f16) && (uint64_t)a.m_vec * (uint64_t)V * (uint64_t)a.N * (out_f16 ? 2u : 4u) <= 0x80000000ull;
+}
+
+template <int V, typename OutT>
+static void launch_balanced_v(const SpmmArgs &p, const BalancedArgs &s, uint32_t grid, hipStream_t stream) {
+  if (s.n_items >= 0) hipLaunchKernelGGL((spmm_balanced_kernel<V, OutT, false>), dim3(grid), dim3(64), 0, stream, p, s);
+  else hipLaunchKernelGGL((spmm_balanced_kernel<V, OutT, true>), dim3(grid), dim3(64), 0, stream, p, s);
+}
+
+hipError_t launch_spmm_balanced(const SpmmArgs &a, int V, bool out_f16, const ScheduleView &sv, int n_items,
+                                hipStream_t stream) {
+  SpmmArgs p = a;
+  p.n_tiles = (uint32_t)((a.N + 63) / 64);
+  BalancedArgs s;
+  s.header = sv.header;
+  s.items = sv.items;
+  s.counters = sv.counters;
+  s.partials = sv.partials;
+  s.n_items = n_items;
+  s.tiles_padded = padded_tiles(p.n_tiles);
+  uint32_t grid;
+  if (n_items >= 0) {
+    const uint64_t units = (uint64_t)n_items * s.tiles_padded * (uint64_t)a.batch;
+    if (units >= (1ull << 31)) return hipErrorInvalidValue;
+    if (units == 0) return hipSuccess;
+    grid = (uint32_t)units;
+  } else {
+    grid = 32u * device_cus();  // a multiple of 8: a workgroup's ids stay on one XCD through the grid-stride loop
+  }
+  g_last_kernel = 7;
+  if (V == 8) {
+    if (out_f16) launch_balanced_v<8, _Float16>(p, s, grid, stream);
+    else launch_balanced_v<8, float>(p, s, grid, stream);
+  } else {
+    if (out_f16) launch_balanced_v<16, _Float16>(p, s, grid, stream);
+    else launch_balanced_v<16, float>(p, s, grid, stream);
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_spmm(const SpmmArgs &a, int V, bool out_f16, hipStream_t stream) {
+  const int out_size = out_f16 ? 2 : 4;
+  const bool fast = mfma_kernels_apply(a, out_f16);
   int which = 1;
   if (fast) {
     // The slab kernel pays off when enough vector-rows share a slab and there are enough

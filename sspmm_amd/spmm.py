@@ -33,12 +33,19 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
-def spmm(row_indices, row_offsets, column_indices, values, rhs_matrix, vec_length, out_dtype=torch.float16):
+def _check_plan(plan, m_vec, vec_length, K):
+    if (plan.m_vec, plan.vec_length, plan.K) != (m_vec, vec_length, K):
+        raise ValueError("the plan was made for m_vec=%d, V=%d, K=%d, the product has m_vec=%d, V=%d, K=%d"
+                         % (plan.m_vec, plan.vec_length, plan.K, m_vec, vec_length, K))
+
+
+def spmm(row_indices, row_offsets, column_indices, values, rhs_matrix, vec_length, out_dtype=torch.float16, plan=None):
     """C[m_vec*V, N] = A_cvse @ rhs_matrix[K, N].
 
     Same call as the reference's `spmm(row_indices, row_offsets, column_indices, values,
     rhs_matrix, vec_length)`; returns a new fp16 tensor like the reference, or fp32 when
     out_dtype=torch.float32 (the reference's C++ `float*` overload, SSpMM/include/sspmm.cuh:31-37).
+    With `plan` (a sspmm_amd.Plan of this pattern) the plan's schedule replaces row_indices.
     """
     _check_inputs(row_indices, row_offsets, column_indices, values, rhs_matrix, vec_length)
     if rhs_matrix.dim() != 2:
@@ -46,6 +53,15 @@ def spmm(row_indices, row_offsets, column_indices, values, rhs_matrix, vec_lengt
     m_vec = row_offsets.size(-1) - 1
     K, N = rhs_matrix.size(0), rhs_matrix.size(1)
     out = torch.empty((m_vec * vec_length, N), dtype=out_dtype, device=rhs_matrix.device)
+    if plan is not None:
+        _check_plan(plan, m_vec, vec_length, K)
+        fn = {torch.float16: _lib.lib().sspmm_plan_batched_f16_f16,
+              torch.float32: _lib.lib().sspmm_plan_batched_f16_f32}[out_dtype]
+        with torch.cuda.device(rhs_matrix.device):
+            rc = fn(plan.handle, 1, N, _ptr(row_offsets), _ptr(column_indices), _ptr(values), 0, _ptr(rhs_matrix), 0,
+                    _ptr(out), 0, _stream())
+        _lib.check(rc, "sspmm_plan")
+        return out
     fn = {torch.float16: _lib.lib().sspmm_f16_f16, torch.float32: _lib.lib().sspmm_f16_f32}[out_dtype]
     with torch.cuda.device(rhs_matrix.device):
         rc = fn(m_vec, vec_length, N, K, _ptr(row_indices), _ptr(row_offsets), _ptr(column_indices), _ptr(values),
@@ -54,7 +70,7 @@ def spmm(row_indices, row_offsets, column_indices, values, rhs_matrix, vec_lengt
     return out
 
 
-def bspmm(row_indices, row_offsets, column_indices, values, rhs_matrix, vec_length, out_dtype=torch.float16):
+def bspmm(row_indices, row_offsets, column_indices, values, rhs_matrix, vec_length, out_dtype=torch.float16, plan=None):
     """Batched SpMM with one pattern for the whole batch: values [batch, nvec*V],
     rhs_matrix [batch, K, N] -> [batch, m_vec*V, N] (reference batched_spmm_cuda,
     end2end/sspmm_e2e/src/cuda/spmm_kernel.cu:516-586)."""
@@ -68,6 +84,15 @@ def bspmm(row_indices, row_offsets, column_indices, values, rhs_matrix, vec_leng
                          % (batch * nvec * vec_length, values.numel()))
     M = m_vec * vec_length
     out = torch.empty((batch, M, N), dtype=out_dtype, device=rhs_matrix.device)
+    if plan is not None:
+        _check_plan(plan, m_vec, vec_length, K)
+        fn = {torch.float16: _lib.lib().sspmm_plan_batched_f16_f16,
+              torch.float32: _lib.lib().sspmm_plan_batched_f16_f32}[out_dtype]
+        with torch.cuda.device(rhs_matrix.device):
+            rc = fn(plan.handle, batch, N, _ptr(row_offsets), _ptr(column_indices), _ptr(values), nvec * vec_length,
+                    _ptr(rhs_matrix), K * N, _ptr(out), M * N, _stream())
+        _lib.check(rc, "sspmm_plan_batched")
+        return out
     fn = {torch.float16: _lib.lib().sspmm_batched_f16_f16,
           torch.float32: _lib.lib().sspmm_batched_f16_f32}[out_dtype]
     with torch.cuda.device(rhs_matrix.device):

@@ -50,6 +50,15 @@ def test_argument_errors_without_device_work(built_library):
     assert L.svc_count(8, 8, 0, one, one, 4, 0, one, one, None) == 1  # V < 1
     assert L.svc_count(8, 8, 8, one, one, 4, 0, one, None, None) == 1  # no workspace
     assert L.svc_fill(8, 8, 8, one, one, one, 4, 0, one, one, one, None, None) == 1  # values in, no values out
+    # plans: unsupported V, no place to put the handle, no pattern
+    import ctypes as C
+    handle = C.c_void_p()
+    assert L.sspmm_plan_create(4, 4, 64, one, 64, 1, 0, None, C.byref(handle)) == 1
+    assert L.sspmm_plan_create(4, 8, 64, one, 64, 1, 0, None, None) == 1
+    assert L.sspmm_plan_create(4, 8, 64, None, 64, 1, 0, None, C.byref(handle)) == 1
+    assert L.sspmm_plan_destroy(None) == 0
+    assert L.sspmm_plan_info(None, None) == 1
+    assert L.sspmm_plan_batched_f16_f32(None, 1, 64, one, one, one, 0, one, 0, one, 0, None) == 1
     assert L.svc_workspace_bytes(16, 100, 8) >= 100 * 8
     assert b"invalid" in L.sspmm_error_string(1)
     assert L.sspmm_error_string(0) == b"success"

@@ -141,6 +141,26 @@ int sspmm_plan_batched_f16_f16(const sspmm_plan_t *plan, int batch, int N, const
                                void *hip_stream);
 
 /*
+ * sspmm_plan_batched_f16_f32 for one product without a plan and without allocating.  No
+ * counterpart in the reference.  It is for callers that cannot allocate device memory and so
+ * cannot hold a plan either: code inside a HIP graph capture whose pattern changes from call to
+ * call, tight serving loops, harnesses that forbid hipMalloc.  The schedule, its counters and
+ * the partial tiles of cut rows live in an array of device memory that is part of the library
+ * (9.7 MB on every GPU the library is used on, held until the process ends); every call rebuilds
+ * the schedule there on the device from row_offsets, on the caller's stream, before the product.
+ *   Limits: m_vec <= 32768 and N <= 4096; beyond them the call returns
+ *   SSPMM_ERROR_STATIC_SCRATCH_TOO_SMALL and does nothing.  Other arguments as sspmm_f16_f32.
+ *   All calls on one GPU share the array: two calls that overlap on a GPU (different streams,
+ *   or threads) race and give wrong results; calls on one stream are safe.
+ *   The first call on a device looks the array's address up and should not be made inside a
+ *   capture.  Same results as sspmm_plan_batched_f16_f32 with a plan of the same pattern, bit
+ *   for bit, as long as the plan's panels also fit 8 MB of partial tiles.
+ */
+#define SSPMM_ERROR_STATIC_SCRATCH_TOO_SMALL 9001
+int sspmm_noalloc_f16_f32(int m_vec, int V, int N, int K, const int32_t *row_offsets, const int32_t *col_idx,
+                          const sspmm_half_t *values, const sspmm_half_t *B, float *C, void *hip_stream);
+
+/*
  * row_indices = vector-rows ordered by descending length (ties: ascending row).  Replaces
  * SortedRowSwizzle, reference SSpMM/include/bm_test_utils.h:210-225 (a host std::sort there).
  * No scratch memory is needed.

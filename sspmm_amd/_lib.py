@@ -22,6 +22,7 @@ SIGNATURES = {
     "sspmm_f16_f16": (_int, [_int] * 4 + [_vp] * 7),
     "sspmm_batched_f16_f16": (_int, [_int] * 5 + [_vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),
     "sspmm_batched_f16_f32": (_int, [_int] * 5 + [_vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),
+    "sspmm_noalloc_f16_f32": (_int, [_int] * 4 + [_vp] * 6),
     "sspmm_sorted_row_swizzle": (_int, [_int, _vp, _vp, _vp]),
     "sspmm_plan_create": (_int, [_int, _int, _int, _vp, _int, _int, _int, _vp, ctypes.POINTER(ctypes.c_void_p)]),
     "sspmm_plan_destroy": (_int, [_vp]),

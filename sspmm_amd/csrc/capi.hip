@@ -73,6 +73,8 @@ int sspmm_last_kernel(void) { return sspmm::last_kernel(); }
 const char *sspmm_error_string(int code) {
   if (code == 0) return "success";
   if (code == kInvalid) return "invalid argument (unsupported V, negative size, null pointer or index range)";
+  if (code == SSPMM_ERROR_STATIC_SCRATCH_TOO_SMALL)
+    return "the problem exceeds the static scratch memory of the allocation-free entry point (m_vec <= 32768, N <= 4096)";
   return hipGetErrorString(static_cast<hipError_t>(code));
 }
 
@@ -151,6 +153,27 @@ int sspmm_plan_batched_f16_f16(const sspmm_plan_t *plan, int batch, int N, const
                                const sspmm_half_t *B, int64_t stride_B, sspmm_half_t *C, int64_t stride_C,
                                void *hip_stream) {
   return plan_entry(plan, batch, N, row_offsets, col_idx, values, stride_values, B, stride_B, C, stride_C, true, hip_stream);
+}
+
+int sspmm_noalloc_f16_f32(int m_vec, int V, int N, int K, const int32_t *row_offsets, const int32_t *col_idx,
+                          const sspmm_half_t *values, const sspmm_half_t *B, float *C, void *hip_stream) {
+  if (V != 8 && V != 16) return kInvalid;
+  if (m_vec < 0 || N < 0 || K < 0) return kInvalid;
+  if (!sspmm::static_spmm_fits(m_vec, N)) return SSPMM_ERROR_STATIC_SCRATCH_TOO_SMALL;
+  if (m_vec == 0 || N == 0) return 0;  // nothing to write
+  if (!row_offsets || !C) return kInvalid;
+  if ((int64_t)K * N >= (1ll << 31)) return kInvalid;
+  sspmm::SpmmArgs a{};
+  a.m_vec = m_vec;
+  a.N = N;
+  a.K = K;
+  a.batch = 1;
+  a.row_offsets = row_offsets;
+  a.col_idx = col_idx;
+  a.values = values;
+  a.B = B;
+  a.C = C;
+  return (int)sspmm::launch_spmm_static(a, V, false, static_cast<hipStream_t>(hip_stream));
 }
 
 int sspmm_sorted_row_swizzle(int m_vec, const int32_t *row_offsets, int32_t *row_indices, void *hip_stream) {

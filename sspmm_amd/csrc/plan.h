@@ -29,5 +29,10 @@ hipError_t plan_destroy(Plan *plan);
 // kernels launch_spmm picks.  Allocates nothing.
 hipError_t launch_spmm_planned(const Plan &plan, const SpmmArgs &args, bool out_f16, hipStream_t stream);
 
+// The single product with the load-balanced kernel and no plan: schedule and scratch in a static device array of
+// the library, rebuilt by every call.  Only for static_spmm_fits; batch must be 1.  Allocates nothing.
+bool static_spmm_fits(int m_vec, int N);
+hipError_t launch_spmm_static(const SpmmArgs &args, int V, bool out_f16, hipStream_t stream);
+
 }  // namespace sspmm
 #endif

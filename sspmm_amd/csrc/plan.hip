@@ -7,6 +7,7 @@
 // nothing.
 #include "plan.h"
 
+#include <mutex>
 #include <new>
 
 namespace sspmm {
@@ -75,7 +76,7 @@ hipError_t plan_create(int m_vec, int V, int K, const int32_t *row_offsets, int 
   pl->view.counters = reinterpret_cast<int32_t *>(base + off_counters);
   pl->view.partials = base + off_partials;
   e = hipMemcpyAsync(pl->view.header, pl->header, sizeof(pl->header), hipMemcpyHostToDevice, stream);
-  if (e == hipSuccess) e = launch_schedule_fill(m_vec, row_offsets, pl->view, (int64_t)n_items, (int64_t)pl->counters, stream);
+  if (e == hipSuccess) e = launch_schedule_fill(m_vec, row_offsets, pl->view, (int64_t)n_items, (int64_t)pl->counters, 0, stream);
   if (e == hipSuccess) e = hipStreamSynchronize(stream);  // products with the plan may come on any stream
   if (e != hipSuccess) {
     (void)hipFree(pl->memory);
@@ -103,6 +104,70 @@ hipError_t launch_spmm_planned(const Plan &pl, const SpmmArgs &a, bool out_f16, 
   if (can_balance && (forced == 7 || (forced == 0 && skewed)))
     return launch_spmm_balanced(a, pl.V, out_f16, pl.view, pl.header[kHdrItems], stream);
   return launch_spmm(a, pl.V, out_f16, stream);
+}
+
+// ------------------------------------------------------------------------------------------
+// The same product for callers that can neither allocate nor keep a plan (a pattern that changes from call to
+// call inside a captured graph, a serving loop, a harness that forbids allocation): the schedule, its counters and
+// the partial tiles live in one array of device memory that is part of the library's code object, so every GPU the
+// library runs on holds it from the first use of the library to the end of the process.  The schedule is built on
+// the device by every call (the host never sees the row offsets), and a grid of fixed size walks it.
+static constexpr int kStaticMaxRows = 32768;       // vector-rows
+static constexpr int kStaticMaxN = 4096;           // columns of B: 64 column tiles
+static constexpr int64_t kStaticMaxSlots = 4096;   // panels of cut rows
+static constexpr size_t kStaticItemsOff = 256;
+static constexpr size_t kStaticCountersOff = kStaticItemsOff + (size_t)(kStaticMaxRows + kStaticMaxSlots) * sizeof(ScheduleItem);
+static constexpr size_t kStaticCounters = (size_t)(kStaticMaxSlots / 2) * (kStaticMaxN / 64);  // a cut row has two panels or more
+static constexpr size_t kStaticPartialsOff = kStaticCountersOff + kStaticCounters * 4;
+static constexpr size_t kStaticPartialBytes = (size_t)8 << 20;
+static constexpr size_t kStaticScratchBytes = kStaticPartialsOff + kStaticPartialBytes;  // about 9.7 MB
+static_assert(kStaticPartialsOff % 256 == 0, "the partial tiles are read with 16-byte loads");
+
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// The array's address on each device (the name `scratch` is a host-side stand-in, not a device address), looked up
+// once per device with that device current.
+static constexpr int kStaticMaxDevices = 64;
+static unsigned char *g_scratch_ptr[kStaticMaxDevices] = {};
+static std::mutex g_scratch_mutex;
+
+static hipError_t static_scratch(unsigned char **ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= kStaticMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void *p = nullptr;
+    if ((e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch))) != hipSuccess) return e;
+    g_scratch_ptr[dev] = static_cast<unsigned char *>(p);
+  }
+  *ptr = g_scratch_ptr[dev];
+  return hipSuccess;
+}
+
+bool static_spmm_fits(int m_vec, int N) { return m_vec <= kStaticMaxRows && N <= kStaticMaxN; }
+
+hipError_t launch_spmm_static(const SpmmArgs &a, int V, bool out_f16, hipStream_t stream) {
+  if (!balanced_kernel_applies(a, V, out_f16)) return launch_spmm(a, V, out_f16, stream);  // (needs no scratch)
+  unsigned char *base = nullptr;
+  hipError_t e = static_scratch(&base);
+  if (e != hipSuccess) return e;
+  ScheduleView view;
+  view.header = reinterpret_cast<int32_t *>(base);
+  view.items = reinterpret_cast<ScheduleItem *>(base + kStaticItemsOff);
+  view.counters = reinterpret_cast<int32_t *>(base + kStaticCountersOff);
+  view.partials = base + kStaticPartialsOff;
+  const int64_t tiles = ((int64_t)a.N + 63) / 64;
+  int64_t slot_cap = schedule_slot_cap(kStaticPartialBytes, V, a.N, 1);
+  if (slot_cap > kStaticMaxSlots) slot_cap = kStaticMaxSlots;
+  // Everything the product reads is rewritten first: header, items, and the counters of the rows that are cut
+  // (kernels on the caller's stream, which order themselves; no memset node for a capturing caller).
+  if ((e = launch_schedule_measure(a.m_vec, a.row_offsets, 0, slot_cap, view.header, stream)) != hipSuccess) return e;
+  if ((e = launch_schedule_fill(a.m_vec, a.row_offsets, view, (int64_t)kStaticMaxRows + kStaticMaxSlots, -1, tiles, stream)) !=
+      hipSuccess)
+    return e;
+  return launch_spmm_balanced(a, V, out_f16, view, -1, stream);
 }
 
 }  // namespace sspmm

@@ -56,9 +56,10 @@ struct ScheduleView {
 hipError_t launch_schedule_measure(int m_vec, const int32_t *row_offsets, int budget, int64_t slot_cap, int32_t *header,
                                    hipStream_t stream);
 // Writes the items for the budget the header holds (at most item_cap of them: the caller sizes from the header,
-// or passes bounds that hold for every pattern), and clears `counters_to_clear` counters.  One workgroup.
+// or passes bounds that hold for every pattern), and clears `counters_to_clear` counters, or when that is
+// negative the counters_per_cut_row counters of every cut row the header reports.  One workgroup.
 hipError_t launch_schedule_fill(int m_vec, const int32_t *row_offsets, const ScheduleView &view, int64_t item_cap,
-                                int64_t counters_to_clear, hipStream_t stream);
+                                int64_t counters_to_clear, int64_t counters_per_cut_row, hipStream_t stream);
 
 }  // namespace sspmm
 #endif

@@ -111,8 +111,10 @@ __device__ __forceinline__ unsigned long long block_exclusive_scan64(unsigned lo
 __global__ __launch_bounds__(kBuildThreads) void schedule_fill_kernel(int m_vec, const int32_t *__restrict__ row_offsets,
                                                                       const int32_t *__restrict__ header,
                                                                       ScheduleItem *__restrict__ items, long long item_cap,
-                                                                      int32_t *__restrict__ counters, long long counters_to_clear) {
+                                                                      int32_t *__restrict__ counters, long long counters_to_clear,
+                                                                      long long counters_per_cut_row) {
   __shared__ unsigned long long scratch[kBuildThreads / 64];
+  if (counters_to_clear < 0) counters_to_clear = (long long)header[kHdrSplitRows] * counters_per_cut_row;
   for (long long i = threadIdx.x; i < counters_to_clear; i += kBuildThreads) counters[i] = 0;
   const int budget = header[kHdrBudget];
   const long long n_slots = header[kHdrSlots];
@@ -180,9 +182,10 @@ hipError_t launch_schedule_measure(int m_vec, const int32_t *row_offsets, int bu
 }
 
 hipError_t launch_schedule_fill(int m_vec, const int32_t *row_offsets, const ScheduleView &view, int64_t item_cap,
-                                int64_t counters_to_clear, hipStream_t stream) {
+                                int64_t counters_to_clear, int64_t counters_per_cut_row, hipStream_t stream) {
   hipLaunchKernelGGL(schedule_fill_kernel, dim3(1), dim3(kBuildThreads), 0, stream, m_vec, row_offsets, view.header,
-                     view.items, (long long)item_cap, view.counters, (long long)counters_to_clear);
+                     view.items, (long long)item_cap, view.counters, (long long)counters_to_clear,
+                     (long long)counters_per_cut_row);
   return hipGetLastError();
 }
 

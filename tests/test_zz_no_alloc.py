@@ -1,0 +1,76 @@
+"""The allocation-free entry point (schedule and scratch in a static device array of the library) against the
+entry point it is a variant of, the product with a plan."""
+import numpy as np
+import pytest
+import torch
+
+from sspmm_amd import _lib, synth
+from sspmm_amd.plan import Plan
+from gpu_util import TIGHT_F32, dev, max_rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def _pattern(m_vec, K, V, seed, long_rows):
+    rng = np.random.default_rng(seed)
+    lens = rng.integers(0, 60, m_vec)
+    lens[rng.choice(m_vec, long_rows, replace=False)] = rng.integers(500, min(K, 3000), long_rows)
+    lens[0] = 0
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cols = np.concatenate([rng.permutation(K)[:n] for n in lens]).astype(np.int32)
+    vals = (rng.standard_normal(cols.size * V) * 0.1).astype(np.float16)
+    return synth.VectorSparse(m_vec * V, K, V, m_vec, off, cols, vals, cols.size * V)
+
+
+def _both(L, vs, B, N):
+    """(allocation-free entry point, product with a plan) on the same operands, through the C ABI."""
+    ro, ci, vv, dB = dev(vs.row_offsets), dev(vs.col_idx), dev(vs.values), dev(B)
+    stream = torch.cuda.current_stream().cuda_stream
+    got = torch.full((vs.m_vec * vs.V, N), 7.0, device="cuda")
+    print("noalloc m_vec=%d V=%d K=%d N=%d nvec=%d" % (vs.m_vec, vs.V, vs.K, N, vs.col_idx.size), flush=True)
+    rc = L.sspmm_noalloc_f16_f32(vs.m_vec, vs.V, N, vs.K, ro.data_ptr(), ci.data_ptr(), vv.data_ptr(), dB.data_ptr(),
+                                 got.data_ptr(), stream)
+    assert rc == 0, rc
+    plan = Plan(ro, vs.V, vs.K, max_N=N)
+    want = torch.full((vs.m_vec * vs.V, N), -7.0, device="cuda")
+    rc = L.sspmm_plan_batched_f16_f32(plan.handle, 1, N, ro.data_ptr(), ci.data_ptr(), vv.data_ptr(), 0, dB.data_ptr(), 0,
+                                      want.data_ptr(), 0, stream)
+    assert rc == 0, rc
+    torch.cuda.synchronize()
+    cut = plan.info().cut_rows
+    plan.destroy()
+    return got, want, cut
+
+
+@pytest.mark.parametrize("V", [8, 16])
+def test_two_calls_in_a_row_the_second_smaller(oracle, built_library, V):
+    L = _lib.lib()
+    # first call: 300 vector-rows, 24 of them long, four column tiles the last one partial
+    big = _pattern(300, 6000, V, seed=V, long_rows=24)
+    B1 = synth.dense_rhs(6000, 200, seed=1)
+    got1, want1, cut1 = _both(L, big, B1, 200)
+    assert cut1 > 0
+    assert torch.equal(got1, want1)
+    ref1 = oracle.spmm(big.m_vec, V, 200, 6000, big.row_offsets, big.col_idx, big.values, B1, threads=8)
+    assert max_rel_err(got1.cpu().numpy(), ref1) <= TIGHT_F32
+    # second call: fewer rows, fewer cut rows, one column tile: whatever the first call left in the scratch array
+    # (a longer work list, counters, partial tiles) must not show
+    small = _pattern(40, 2000, V, seed=100 + V, long_rows=3)
+    B2 = synth.dense_rhs(2000, 64, seed=2)
+    got2, want2, cut2 = _both(L, small, B2, 64)
+    assert 0 < cut2 < cut1
+    assert torch.equal(got2, want2)
+    ref2 = oracle.spmm(small.m_vec, V, 64, 2000, small.row_offsets, small.col_idx, small.values, B2, threads=8)
+    assert max_rel_err(got2.cpu().numpy(), ref2) <= TIGHT_F32
+    assert not got2[:V].any()  # the empty first vector-row is written as zeros
+
+
+def test_sizes_beyond_the_static_scratch_are_rejected(built_library):
+    L = _lib.lib()
+    one = 1  # rejected calls never dereference their pointers
+    too_small = 9001
+    assert L.sspmm_noalloc_f16_f32(32769, 8, 64, 64, one, one, one, one, one, None) == too_small
+    assert L.sspmm_noalloc_f16_f32(64, 8, 4104, 64, one, one, one, one, one, None) == too_small
+    assert b"static scratch" in L.sspmm_error_string(too_small)
+    assert L.sspmm_noalloc_f16_f32(64, 4, 64, 64, one, one, one, one, one, None) == 1
+    assert L.sspmm_noalloc_f16_f32(0, 8, 64, 64, None, None, None, None, None, None) == 0

@@ -12,9 +12,13 @@ SSpMM/sspmm_test.cpp:197, with nnz the scalar non-zeros).
 
 `roofline` prices the SpMM kernel against the 8 TB/s HBM peak with the algorithmic bytes of one
 launch (every operand read once, C written once).  `cpu_baseline` times the CPU oracle (a port of
-the reference's host loop) on one batch element, single thread.  `extra` carries the other
-configurations (single launches, V=16 shapes, the SVC against the Python RowMerge, the dense GEMM
-comparator).
+the reference's host loop) on one batch element, single thread.  `extra` carries every other
+benchmark configuration as single launches (mean, median and minimum launch time, the dense GEMM
+of the same shape beside each), the SVC against the Python RowMerge, the encoder layer and the
+sparse attention block.
+
+    python bench.py --only NAME[,NAME...]   runs just those entries of `extra` (what the profiles/ summaries use)
+    python bench.py --list                  prints their names
 """
 import argparse
 import json
@@ -26,10 +30,14 @@ import numpy as np
 
 HBM_PEAK_GBPS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
-# HBM bytes per launch of the headline workload at the default batch of 128, from hardware counters
-# (FETCH_SIZE and WRITE_SIZE, each scaled by its reading for a 256 MiB device copy): see
-# profiles/spmm_slab_v8_f32_cfg2_batch128_hbm_traffic.txt.  Other batch sizes report null.
-MEASURED_TRAFFIC_BYTES = {128: 66.1e6 + 268.4e6}
+# HBM bytes per launch from hardware counters (FETCH_SIZE and WRITE_SIZE in separate runs, each scaled by its
+# reading for a plain 256 MiB device copy), keyed by kernel and workload; `source` names the summary it comes from.
+MEASURED_TRAFFIC = {
+    "headline_batch128": {"kernel": "spmm_slab_kernel<8,float,*,4>", "bytes": 66.1e6 + 268.4e6,
+                          "source": "profiles/spmm_slab_v8_f32_cfg2_batch128_hbm_traffic.txt"},
+}
+KERNEL_NAMES = {1: "spmm_generic_kernel", 2: "spmm_gather_kernel", 3: "spmm_slab_kernel<*,4>", 4: "spmm_gather_split_kernel",
+                5: "spmm_slab_kernel<*,2>", 6: "spmm_stage_kernel", 7: "spmm_balanced_kernel"}
 
 
 def parse_args():
@@ -43,8 +51,10 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--batch", type=int, default=128, help="independent value/B/C sets per step")
     ap.add_argument("--quick", action="store_true", help="skip the extra configurations and CPU legs")
+    ap.add_argument("--only", default="", help="comma-separated names of extra entries: run only those and print them")
+    ap.add_argument("--list", action="store_true", help="print the names --only accepts")
     ap.add_argument("--attention-only", action="store_true",
-                    help="run only the sparse attention block (bsddmm, bcsr_softmax, bspmm) and print its figures")
+                    help="run only the sparse attention block (same as --only sparse_attention_seq4096_d64_v8_s0.9_heads48)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy (its hardware-counter readings calibrate FETCH_SIZE / "
                          "WRITE_SIZE when the run is profiled)")
@@ -53,41 +63,79 @@ def parse_args():
     return ap.parse_args()
 
 
-def time_launches(fn, steps, warmup, series=None):
-    """Average milliseconds per call over `steps` calls, HIP events on the launch stream."""
+def time_launches(fn, steps, warmup, series=None, stats=None):
+    """Average milliseconds per call over `steps` calls, HIP events on the launch stream.  `stats`, a dict, receives
+    the median and the minimum of the averages over chunks of ten launches."""
     import torch
     chunk = 10
     marks = []
 
-    def run(n):
+    def run(n, keep):
         for i in range(n):
-            if series is not None and i % chunk == 0:
+            if keep and i % chunk == 0:
                 ev = torch.cuda.Event(enable_timing=True)
                 ev.record()
                 marks.append((ev, min(chunk, n - i)))
             fn()
 
-    run(warmup)
+    run(warmup, series is not None)
     torch.cuda.synchronize()
     n_warm = len(marks)
     start = torch.cuda.Event(enable_timing=True)
     end = torch.cuda.Event(enable_timing=True)
     start.record()
-    run(steps)
+    run(steps, True)
     end.record()
     torch.cuda.synchronize()
+    bounds = [m[0] for m in marks] + [end]
+    per_chunk = [ev.elapsed_time(bounds[i + 1]) / n for i, (ev, n) in enumerate(marks)]
     if series is not None:
-        # (events on the launch stream: microseconds per launch for every chunk of 10 launches; the chunk that ends
-        # the warm-up runs into the host synchronisation and is left out)
-        bounds = [m[0] for m in marks] + [end]
-        for i, (ev, n) in enumerate(marks):
-            series.append(ev.elapsed_time(bounds[i + 1]) / n * 1e3 if i != n_warm - 1 else None)
+        # (microseconds per launch for every chunk of 10 launches; the chunk that ends the warm-up runs into the host
+        # synchronisation and is left out)
+        for i, v in enumerate(per_chunk):
+            series.append(v * 1e3 if i != n_warm - 1 else None)
+    if stats is not None:
+        timed = sorted(per_chunk[n_warm:])
+        stats["ms_median"] = timed[len(timed) // 2]
+        stats["ms_min"] = timed[0]
     return start.elapsed_time(end) / steps
 
 
-def spmm_case(L, torch, synth, M, K, V, sparsity, N, batch, out_f32, std, seed, steps, warmup, dense=False, series=None):
-    """Times one SpMM configuration; returns a dict of figures."""
-    vs = synth.vector_sparse(M, K, V, sparsity, seed=seed, std=std)
+def graph_time(fn, launches=20, replays=20):
+    """Milliseconds per launch when `launches` of them are recorded into one HIP graph and the graph is replayed:
+    the host's cost of enqueueing a launch is out of the picture."""
+    import torch
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        fn(s.cuda_stream)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=s):
+        for _ in range(launches):
+            fn(torch.cuda.current_stream().cuda_stream)
+    for _ in range(3):
+        g.replay()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(replays):
+        g.replay()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / (launches * replays)
+
+
+def figures(ms, alg_bytes, flops):
+    return {"ms": ms, "useful_tflops": flops / ms / 1e9, "alg_bytes": alg_bytes, "hbm_gbps": alg_bytes / ms / 1e6,
+            "hbm_frac": alg_bytes / ms / 1e6 / HBM_PEAK_GBPS}
+
+
+def spmm_case(L, torch, synth, M, K, V, sparsity, N, batch, out_f32, std, seed, steps, warmup, dense=False, series=None,
+              plan=False, graph=False, vs=None, handles_out=None):
+    """Times one SpMM configuration (a seeded vector-sparse pattern unless `vs` is given); returns a dict of figures."""
+    from sspmm_amd.plan import Plan
+    if vs is None:
+        vs = synth.vector_sparse(M, K, V, sparsity, seed=seed, std=std)
     g = torch.Generator(device="cuda").manual_seed(seed)
     ro = torch.from_numpy(vs.row_offsets).cuda()
     ci = torch.from_numpy(vs.col_idx).cuda()
@@ -95,26 +143,39 @@ def spmm_case(L, torch, synth, M, K, V, sparsity, N, batch, out_f32, std, seed, 
     vals = (torch.randn(batch, nv * V, generator=g, device="cuda") * std).half()
     B = torch.randn(batch, K, N, generator=g, device="cuda").half()
     C = torch.empty(batch, vs.m_vec * V, N, dtype=torch.float32 if out_f32 else torch.float16, device="cuda")
-    fn = L.sspmm_batched_f16_f32 if out_f32 else L.sspmm_batched_f16_f16
-    stream = torch.cuda.current_stream().cuda_stream
+    the_plan = Plan(ro, V, K, max_N=N, max_batch=batch) if plan else None
+    if the_plan is not None:
+        fn = L.sspmm_plan_batched_f16_f32 if out_f32 else L.sspmm_plan_batched_f16_f16
+    else:
+        fn = L.sspmm_batched_f16_f32 if out_f32 else L.sspmm_batched_f16_f16
 
-    def launch():
-        rc = fn(batch, vs.m_vec, V, N, K, None, ro.data_ptr(), ci.data_ptr(), vals.data_ptr(), nv * V, B.data_ptr(),
-                K * N, C.data_ptr(), vs.m_vec * V * N, stream)
+    def launch_on(stream):
+        if the_plan is not None:
+            rc = fn(the_plan.handle, batch, N, ro.data_ptr(), ci.data_ptr(), vals.data_ptr(), nv * V, B.data_ptr(), K * N,
+                    C.data_ptr(), vs.m_vec * V * N, stream)
+        else:
+            rc = fn(batch, vs.m_vec, V, N, K, None, ro.data_ptr(), ci.data_ptr(), vals.data_ptr(), nv * V, B.data_ptr(),
+                    K * N, C.data_ptr(), vs.m_vec * V * N, stream)
         if rc:
             raise RuntimeError("sspmm failed: %d" % rc)
 
-    ms = time_launches(launch, steps, warmup, series)
+    stream = torch.cuda.current_stream().cuda_stream
+    stats = {}
+    ms = time_launches(lambda: launch_on(stream), steps, warmup, series, stats)
     bytes_alg = batch * synth.spmm_algorithmic_bytes(vs.m_vec, V, nv, K, N, 4 if out_f32 else 2) \
         - (batch - 1) * (4 * nv + 4 * (vs.m_vec + 1))  # the pattern is shared by the batch
     flops = 2.0 * vs.nnz * N * batch
-    out = {
-        "workload": "A %dx%d V=%d s=%.2f, B %dx%d, C %s, batch %d" % (M, K, V, sparsity, K, N,
-                                                                       "fp32" if out_f32 else "fp16", batch),
-        "ms": ms, "useful_tflops": flops / ms / 1e9, "alg_bytes": bytes_alg, "hbm_gbps": bytes_alg / ms / 1e6,
-        "hbm_frac": bytes_alg / ms / 1e6 / HBM_PEAK_GBPS,
-        "gather_bytes_no_reuse": batch * 2 * nv * N,
-    }
+    out = {"workload": "A %dx%d V=%d s=%.2f, B %dx%d, C %s, batch %d%s" % (
+        vs.m_vec * V, K, V, sparsity, K, N, "fp32" if out_f32 else "fp16", batch, ", with a plan" if plan else "")}
+    out.update(figures(ms, bytes_alg, flops))
+    out.update(stats)
+    out["hbm_frac_at_min"] = bytes_alg / stats["ms_min"] / 1e6 / HBM_PEAK_GBPS
+    out["kernel"] = KERNEL_NAMES.get(L.sspmm_last_kernel(), "unknown")
+    out["gather_bytes_no_reuse"] = batch * 2 * nv * N
+    if graph:
+        gms = graph_time(launch_on)
+        out["ms_in_a_graph"] = gms
+        out["hbm_frac_in_a_graph"] = bytes_alg / gms / 1e6 / HBM_PEAK_GBPS
     if dense:
         A = torch.zeros(vs.m_vec * V, K, dtype=torch.float16, device="cuda")
         Ad = A.unsqueeze(0).expand(batch, -1, -1).contiguous()
@@ -123,8 +184,12 @@ def spmm_case(L, torch, synth, M, K, V, sparsity, N, batch, out_f32, std, seed, 
         out["dense_gemm_effective_tflops"] = flops / dms / 1e9
         out["speedup_vs_dense"] = dms / ms
         del A, Ad
-    handles = (vs, vals, B, C)
-    return out, handles
+    if handles_out is not None:
+        handles_out.extend([vs, vals, B, C])
+    if the_plan is not None:
+        out["plan"] = the_plan.info()._asdict()
+        the_plan.destroy()
+    return out
 
 
 def attention_block(torch, synth, sspmm_amd, st, wu):
@@ -141,7 +206,7 @@ def attention_block(torch, synth, sspmm_amd, st, wu):
     t_sddmm = time_launches(lambda: sspmm_amd.bsddmm(None, offA, colA, qA, kA, VA), st, wu)
     t_soft = time_launches(lambda: sspmm_amd.bcsr_softmax(None, offA, wA, 0.125, VA, bA), st, wu)
     t_av = time_launches(lambda: sspmm_amd.bspmm(None, offA, colA, pA, vA, VA), st, wu)
-    t_dense = time_launches(lambda: torch.nn.functional.scaled_dot_product_attention(qA, kA, vA), st, wu)
+    t_dense = time_launches(lambda: torch.nn.functional.scaled_dot_product_attention(qA, kA, vA), max(5, st // 10), 2)
     by_sddmm = bA * (2 * seqA * dA * 2 + 2 * nvA * VA) + 4 * nvA + 4 * (mk_a.m_vec + 1)
     by_soft = bA * 2 * 2 * nvA * VA + 4 * (mk_a.m_vec + 1)
     by_av = bA * (2 * nvA * VA + 2 * seqA * dA + 2 * seqA * dA) + 4 * nvA + 4 * (mk_a.m_vec + 1)
@@ -156,8 +221,353 @@ def attention_block(torch, synth, sspmm_amd, st, wu):
     return res
 
 
+# ---- the entries of `extra` ------------------------------------------------------------------------------------------
+
+def single_launch_cases(batch):
+    """name -> arguments of spmm_case: every benchmark configuration as one launch (and the batched forms)."""
+    cases = {}
+    for (M, K) in ((2048, 512), (512, 2048)):
+        for s in (0.7, 0.9, 0.98):
+            cases["cfg2_%dx%d_v8_s%g_n256" % (M, K, s)] = dict(M=M, K=K, V=8, sparsity=s, N=256, batch=1, out_f32=True,
+                                                               std=0.02, seed=2)
+    cases["cfg2_batched_fp16_out"] = dict(M=2048, K=512, V=8, sparsity=0.9, N=256, batch=batch, out_f32=False, std=0.02, seed=2)
+    cases["cfg2_shape_v16_batched"] = dict(M=2048, K=512, V=16, sparsity=0.9, N=256, batch=batch, out_f32=True, std=0.02, seed=2)
+    cases["cfg2_shape_v16_batched_fp16_out"] = dict(M=2048, K=512, V=16, sparsity=0.9, N=256, batch=batch, out_f32=False,
+                                                    std=0.02, seed=2)
+    for (M, K) in ((1024, 2304), (2048, 1024)):
+        for s in (0.8, 0.95):
+            for N in (256, 3136):
+                cases["cfg3_%dx%d_v16_s%g_n%d" % (M, K, s, N)] = dict(M=M, K=K, V=16, sparsity=s, N=N, batch=1, out_f32=True,
+                                                                      std=0.05, seed=3)
+    for name, (M, K, seed) in (("q", (768, 768, 51)), ("ffn1", (3072, 768, 55)), ("ffn2", (768, 3072, 56))):
+        cases["cfg5_%s_%dx%d_v16_s0.9_n4096" % (name, M, K)] = dict(M=M, K=K, V=16, sparsity=0.9, N=4096, batch=1,
+                                                                    out_f32=False, std=0.02, seed=seed)
+    cases["cfg5_ffn1_batched8"] = dict(M=3072, K=768, V=16, sparsity=0.9, N=4096, batch=8, out_f32=False, std=0.02, seed=55)
+    return cases
+
+
+def run_cfg1(L, torch, synth, sspmm_amd, O, st, wu):
+    """The CPU-runnable configuration end to end on both sides: RowMerge then SpMM of a 512x512 matrix (V=8, 90 %),
+    B 512x256.  GPU: svc_count + svc_fill + sspmm_f16_f32 (kernels only, outputs sized beforehand).  CPU: the Python
+    RowMerge (list(set(...)) per member row, the reference's algorithm) and the host loop in C, single thread."""
+    V, K, N = 8, 512, 256
+    vs = synth.vector_sparse(512, K, V, 0.9, seed=1)
+    csr = synth.expand_to_csr(vs)
+    Bh = synth.dense_rhs(K, N, seed=11)
+    rp, ci, cv, B = (torch.from_numpy(x).cuda() for x in (csr.row_ptr, csr.col_ind, csr.values, Bh))
+    nnz = csr.col_ind.size
+    r = sspmm_amd.svc(rp, ci, cv, csr.M, csr.K, V)
+    ws = torch.empty(L.svc_workspace_bytes(csr.M, nnz, V), dtype=torch.uint8, device="cuda")
+    vrp = torch.zeros(csr.M // V + 1, dtype=torch.int32, device="cuda")
+    vcol = torch.empty(r.num_vec, dtype=torch.int32, device="cuda")
+    vval = torch.empty(r.num_vec * V, dtype=torch.float16, device="cuda")
+    C = torch.empty(csr.M, N, dtype=torch.float32, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def svc_only():
+        assert L.svc_count(csr.M, K, V, rp.data_ptr(), ci.data_ptr(), nnz, 0, vrp.data_ptr(), ws.data_ptr(), stream) == 0
+        assert L.svc_fill(csr.M, K, V, rp.data_ptr(), ci.data_ptr(), cv.data_ptr(), nnz, 0, vrp.data_ptr(), ws.data_ptr(),
+                          vcol.data_ptr(), vval.data_ptr(), stream) == 0
+
+    def spmm_only():
+        assert L.sspmm_f16_f32(csr.M // V, V, N, K, None, vrp.data_ptr(), vcol.data_ptr(), vval.data_ptr(), B.data_ptr(),
+                               C.data_ptr(), stream) == 0
+
+    def pipeline():
+        svc_only()
+        spmm_only()
+
+    pipeline()
+    torch.cuda.synchronize()
+    t_svc, t_spmm, t_pipe = (time_launches(f, st, wu) for f in (svc_only, spmm_only, pipeline))
+    lists = O.csr_col_lists(csr.M, csr.row_ptr, csr.col_ind)
+    py = []
+    for _ in range(5):
+        t0 = time.perf_counter()
+        ptr, flat = O.rowmerge_python(csr.M, V, lists)
+        py.append((time.perf_counter() - t0) * 1e3)
+    wrp, wcol, wval = O.svc(csr.M, K, V, csr.row_ptr, csr.col_ind, csr.values)
+    t0, reps = time.perf_counter(), 0
+    while reps < 50 and (time.perf_counter() - t0 < 2.0 or reps < 3):
+        want = O.spmm(csr.M // V, V, N, K, wrp, wcol, wval, Bh, threads=1)
+        reps += 1
+    cpu_spmm_ms = (time.perf_counter() - t0) * 1e3 / reps
+    same = vrp.cpu().numpy().tolist() == ptr and vcol.cpu().numpy().tolist() == flat
+    err = float(np.abs(C.cpu().numpy() - want).max() / np.abs(want).max())
+    nv = int(r.num_vec)
+    by = synth.spmm_algorithmic_bytes(csr.M // V, V, nv, K, N, 4)
+    res = {"workload": "CSR 512x512 (V=8 vectors, 90 %% sparse, nnz %d) -> SVC -> SpMM with B 512x256, C fp32" % nnz,
+           "gpu_svc_ms": t_svc, "gpu_spmm_ms": t_spmm, "gpu_pipeline_ms": t_pipe,
+           "cpu_python_rowmerge_ms_samples": py, "cpu_python_rowmerge_ms": sorted(py)[len(py) // 2],
+           "cpu_host_spmm_ms": cpu_spmm_ms, "cpu_cores": 1,
+           "cpu_pipeline_ms": sorted(py)[len(py) // 2] + cpu_spmm_ms,
+           "svc_bit_exact_vs_python": bool(same), "spmm_max_rel_err_vs_host_loop": err}
+    res["speedup_pipeline"] = res["cpu_pipeline_ms"] / t_pipe
+    res["spmm"] = figures(t_spmm, by, 2.0 * vs.nnz * N)
+    return res
+
+
+def run_cfg4(L, torch, synth, sspmm_amd, O, st, wu):
+    """The unstructured configuration: SVC of a 16384^2 Zipf CSR matrix (both column orders) against the Python
+    RowMerge and the C oracle, and the SpMM that consumes its output, without and with a plan."""
+    from sspmm_amd.plan import Plan
+    V = 8
+    csr = synth.zipf_csr(16384, 16384, seed=4)
+    rp, ci, cv = (torch.from_numpy(x).cuda() for x in (csr.row_ptr, csr.col_ind, csr.values))
+    nnz = csr.col_ind.size
+    r = sspmm_amd.svc(rp, ci, cv, csr.M, csr.K, V)
+    torch.cuda.synchronize()
+    svc_ms = time_launches(lambda: sspmm_amd.svc(rp, ci, cv, csr.M, csr.K, V), 20, 3)
+    # kernels only (no allocation, no host read-back): outputs sized beforehand
+    ws = torch.empty(L.svc_workspace_bytes(csr.M, nnz, V), dtype=torch.uint8, device="cuda")
+    vrp = torch.zeros(csr.M // V + 1, dtype=torch.int32, device="cuda")
+    vcol = torch.empty(r.num_vec, dtype=torch.int32, device="cuda")
+    vval = torch.empty(r.num_vec * V, dtype=torch.float16, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def svc_kernels(order):
+        def f():
+            assert L.svc_count(csr.M, csr.K, V, rp.data_ptr(), ci.data_ptr(), nnz, order, vrp.data_ptr(), ws.data_ptr(), stream) == 0
+            assert L.svc_fill(csr.M, csr.K, V, rp.data_ptr(), ci.data_ptr(), cv.data_ptr(), nnz, order, vrp.data_ptr(),
+                              ws.data_ptr(), vcol.data_ptr(), vval.data_ptr(), stream) == 0
+        return f
+
+    st_k = {}
+    svc_k_ms = time_launches(svc_kernels(0), 30, 5, stats=st_k)
+    svc_sorted_ms = time_launches(svc_kernels(1), 30, 5)
+    sorted_cols = vcol.cpu().numpy()
+    lists = O.csr_col_lists(csr.M, csr.row_ptr, csr.col_ind)
+    py = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        ptr, flat = O.rowmerge_python(csr.M, V, lists)
+        py.append((time.perf_counter() - t0) * 1e3)
+    py_ms = sorted(py)[1]
+    t0 = time.perf_counter()
+    O.svc(csr.M, csr.K, V, csr.row_ptr, csr.col_ind, csr.values)
+    c_ms = (time.perf_counter() - t0) * 1e3
+    same = (r.vec_row_ptr.cpu().numpy().tolist() == ptr) and (r.vec_col.cpu().numpy().tolist() == flat)
+    off_h = r.vec_row_ptr.cpu().numpy()
+    sorted_ok = all(np.array_equal(sorted_cols[off_h[i]:off_h[i + 1]], np.sort(np.asarray(flat[off_h[i]:off_h[i + 1]])))
+                    for i in range(0, csr.M // V, 64))
+    svc_bytes = synth.svc_algorithmic_bytes(csr.M, nnz, csr.M // V, r.num_vec, V)
+    out = {"svc_cfg4_zipf_16384_v8": {
+        "gpu_ms_with_alloc_and_readback": svc_ms, "gpu_ms_kernels": svc_k_ms, "gpu_ms_kernels_median": st_k["ms_median"],
+        "gpu_ms_kernels_min": st_k["ms_min"], "gpu_ms_kernels_sorted_order": svc_sorted_ms,
+        "python_rowmerge_ms_samples": py, "python_rowmerge_ms": py_ms, "c_oracle_ms": c_ms,
+        "speedup_vs_python": py_ms / svc_k_ms, "speedup_vs_python_with_alloc_and_readback": py_ms / svc_ms,
+        "speedup_vs_python_sorted_order": py_ms / svc_sorted_ms, "bit_exact_vs_python": bool(same),
+        "sorted_order_is_the_sorted_python_rows": bool(sorted_ok),
+        "nnz": int(nnz), "nvec": int(r.num_vec), "fill_ratio": nnz / (r.num_vec * 8.0),
+        "max_vector_row": int(np.diff(off_h).max()), "alg_bytes": svc_bytes, "hbm_gbps": svc_bytes / svc_k_ms / 1e6,
+        "hbm_frac": svc_bytes / svc_k_ms / 1e6 / HBM_PEAK_GBPS,
+        "hbm_frac_sorted_order": svc_bytes / svc_sorted_ms / 1e6 / HBM_PEAK_GBPS}}
+
+    # ... and the SpMM that consumes it: the skewed pattern straight from the SVC, B 16384 x 256
+    N4 = 256
+    B4 = torch.from_numpy(synth.dense_rhs(csr.K, N4, seed=14)).cuda()
+    C4 = torch.empty(csr.M, N4, dtype=torch.float32, device="cuda")
+    m_vec4 = csr.M // 8
+    plan = Plan(r.vec_row_ptr, V, csr.K, max_N=N4)
+
+    def spmm_cfg4(stream_):
+        assert L.sspmm_f16_f32(m_vec4, 8, N4, csr.K, None, r.vec_row_ptr.data_ptr(), r.vec_col.data_ptr(),
+                               r.vec_val.data_ptr(), B4.data_ptr(), C4.data_ptr(), stream_) == 0
+
+    def spmm_cfg4_plan(stream_):
+        assert L.sspmm_plan_batched_f16_f32(plan.handle, 1, N4, r.vec_row_ptr.data_ptr(), r.vec_col.data_ptr(),
+                                            r.vec_val.data_ptr(), 0, B4.data_ptr(), 0, C4.data_ptr(), 0, stream_) == 0
+
+    def spmm_cfg4_noalloc(stream_):
+        assert L.sspmm_noalloc_f16_f32(m_vec4, 8, N4, csr.K, r.vec_row_ptr.data_ptr(), r.vec_col.data_ptr(),
+                                       r.vec_val.data_ptr(), B4.data_ptr(), C4.data_ptr(), stream_) == 0
+
+    lens = np.diff(off_h)
+    touched = int(np.unique(r.vec_col.cpu().numpy()).size)
+    bytes4 = synth.spmm_algorithmic_bytes(m_vec4, 8, int(r.num_vec), csr.K, N4, 4, k_touched=touched)
+    want = None
+    for name, f in (("cfg4_spmm_on_svc_output", spmm_cfg4), ("cfg4_spmm_on_svc_output_with_plan", spmm_cfg4_plan),
+                    ("cfg4_spmm_on_svc_output_allocation_free_entry", spmm_cfg4_noalloc)):
+        stt = {}
+        ms4 = time_launches(lambda: f(stream), st, wu, stats=stt)
+        res = {"workload": "A 16384x16384 Zipf rows (nnz %d) after SVC V=8, B 16384x%d, C fp32" % (nnz, N4)}
+        res.update(figures(ms4, bytes4, 2.0 * nnz * N4))
+        res.update(stt)
+        res["kernel"] = KERNEL_NAMES.get(L.sspmm_last_kernel(), "unknown")
+        res["ms_in_a_graph"] = graph_time(f)
+        res["hbm_frac_in_a_graph"] = bytes4 / res["ms_in_a_graph"] / 1e6 / HBM_PEAK_GBPS
+        res.update({"vector_row_len_max": int(lens.max()), "vector_row_len_mean": float(lens.mean()),
+                    "steps_of_longest_row": int((lens.max() + 31) // 32), "steps_total": int(((lens + 31) // 32).sum()),
+                    "gather_bytes_no_reuse": int(2 * r.num_vec * N4)})
+        if want is None:  # parity of all three against the oracle
+            want = O.spmm(m_vec4, 8, N4, csr.K, off_h, r.vec_col.cpu().numpy(), r.vec_val.cpu().numpy(), B4.cpu().numpy(),
+                          threads=min(os.cpu_count(), 16))
+        torch.cuda.synchronize()
+        res["max_rel_err_vs_host_loop"] = float(np.abs(C4.cpu().numpy() - want).max() / np.abs(want).max())
+        if "plan" in name:
+            res["plan"] = plan.info()._asdict()
+        out[name] = res
+    plan.destroy()
+
+    # the same pass on the shape of the matrices the reference's RowMerge is run on (its dataset of pruned
+    # transformer weights): 2048 x 2048, 90 % of the entries zero at random, V = 8 and 16
+    rng_d = np.random.default_rng(7)
+    mask_d = rng_d.random((2048, 2048)) < 0.1
+    d_ptr = np.concatenate([[0], np.cumsum(mask_d.sum(axis=1))]).astype(np.int32)
+    d_col = np.nonzero(mask_d)[1].astype(np.int32)
+    d_rp, d_ci = torch.from_numpy(d_ptr).cuda(), torch.from_numpy(d_col).cuda()
+    d_lists = O.csr_col_lists(2048, d_ptr, d_col)
+    for Vd in (8, 16):
+        rd = sspmm_amd.svc(d_rp, d_ci, None, 2048, 2048, Vd)
+        d_ms = time_launches(lambda: sspmm_amd.svc(d_rp, d_ci, None, 2048, 2048, Vd), 20, 3)
+        t0 = time.perf_counter()
+        d_want_ptr, d_want_cols = O.rowmerge_python(2048, Vd, d_lists)
+        d_py = (time.perf_counter() - t0) * 1e3
+        out["svc_pruned_weight_2048x2048_s0.9_v%d" % Vd] = {
+            "gpu_ms_with_alloc_and_readback": d_ms, "python_rowmerge_ms": d_py, "speedup_vs_python": d_py / d_ms,
+            "bit_exact_vs_python": bool(rd.vec_row_ptr.cpu().numpy().tolist() == d_want_ptr and
+                                        rd.vec_col.cpu().numpy().tolist() == d_want_cols),
+            "nnz": int(d_col.size), "nvec": int(rd.num_vec),
+        }
+    return out
+
+
+def run_cfg5_layer(L, torch, synth, st, wu):
+    """One BERT-base shaped encoder layer (hidden 768, 12 heads, FFN 3072, 8 x 512 tokens) with six vector-sparse
+    weights (V=16, 90 %) and dense attention in torch; the same layer with dense fp16 matmuls on the densified
+    weights beside it."""
+    from sspmm_amd.layers import SparseEncoderLayer, SparseLinear
+    hid, heads, ffn, V5, bsz, seq = 768, 12, 3072, 16, 8, 512
+
+    def mk(o, i, seed):
+        w = synth.vector_sparse(o, i, V5, 0.9, seed=seed, std=0.02)
+        return SparseLinear.from_cvse(i, V5, torch.from_numpy(w.row_offsets).cuda(), torch.from_numpy(w.col_idx).cuda(),
+                                      torch.from_numpy(w.values).cuda())
+
+    layer = SparseEncoderLayer(hid, heads, ffn, mk(hid, hid, 51), mk(hid, hid, 52), mk(hid, hid, 53), mk(hid, hid, 54),
+                               mk(ffn, hid, 55), mk(hid, ffn, 56)).cuda().half()
+    x5 = (torch.randn(hid, bsz * seq, device="cuda") * 1.0).half()
+    dense_w = {n: getattr(layer, n).dense_weight() for n in ("q", "k", "v", "o", "ffn1", "ffn2")}
+    with torch.no_grad():
+        y_sp = layer(x5, bsz, seq)
+        y_de = layer(x5, bsz, seq, linear=lambda n, lin, t: dense_w[n] @ t)
+        sp_ms = time_launches(lambda: layer(x5, bsz, seq), st, wu)
+        de_ms = time_launches(lambda: layer(x5, bsz, seq, linear=lambda n, lin, t: dense_w[n] @ t), st, wu)
+        per = {}
+        for n in ("q", "o", "ffn1", "ffn2"):
+            lin = getattr(layer, n)
+            xin = torch.randn(lin.in_features, bsz * seq, device="cuda").half()
+            per[n] = {"sparse_ms": time_launches(lambda: lin(xin), st, wu),
+                      "dense_ms": time_launches(lambda: dense_w[n] @ xin, st, wu)}
+        per.update(layer.time_parts(x5, bsz, seq, lambda f: time_launches(f, st, wu)) if hasattr(layer, "time_parts") else {})
+    return {"sparse_layer_ms": sp_ms, "dense_layer_ms": de_ms, "speedup_vs_dense_layer": de_ms / sp_ms,
+            "max_rel_diff_vs_dense_layer": float((y_sp.float() - y_de.float()).abs().max() / y_de.float().abs().max()),
+            "projections": per}
+
+
+def run_reorder(L, torch, synth, sspmm_amd):
+    """Row reordering ahead of the SVC: 16384 rows that are noisy copies of 256 prototype rows, shuffled."""
+    rc_csr = synth.clustered_csr(16384, 16384, 256, 128, seed=6, keep=0.9, extras=1)
+    rrp, rci, rcv = (torch.from_numpy(x).cuda() for x in (rc_csr.row_ptr, rc_csr.col_ind, rc_csr.values))
+    plain = sspmm_amd.svc(rrp, rci, rcv, rc_csr.M, rc_csr.K, 8, order="sorted")
+    reo = sspmm_amd.svc_reordered(rrp, rci, rcv, rc_csr.M, rc_csr.K, 8, order="sorted")
+    rws = torch.empty(L.svc_reorder_workspace_bytes(rc_csr.M), dtype=torch.uint8, device="cuda")
+    rperm = torch.empty(rc_csr.M, dtype=torch.int32, device="cuda")
+    o_rp, o_ci, o_cv = torch.empty_like(rrp), torch.empty_like(rci), torch.empty_like(rcv)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def reorder_order():
+        rc = L.svc_reorder_minhash(rc_csr.M, rrp.data_ptr(), rci.data_ptr(), rperm.data_ptr(), rws.data_ptr(),
+                                   rws.numel(), stream)
+        assert rc == 0, rc
+
+    def reorder_apply():
+        rc = L.svc_permute_csr(rc_csr.M, rperm.data_ptr(), rrp.data_ptr(), rci.data_ptr(), rcv.data_ptr(),
+                               o_rp.data_ptr(), o_ci.data_ptr(), o_cv.data_ptr(), rws.data_ptr(), rws.numel(),
+                               stream)
+        assert rc == 0, rc
+
+    reorder_order()
+    t_order = time_launches(reorder_order, 20, 3)
+    t_apply = time_launches(reorder_apply, 20, 3)
+    rnnz = int(rc_csr.col_ind.size)
+    by_order = 4 * (rc_csr.M + 1) + 4 * rnnz + 4 * rc_csr.M   # row pointer + columns read, order written
+    by_apply = 4 * rc_csr.M + 2 * 4 * (rc_csr.M + 1) + 2 * (4 + 2) * rnnz  # CSR read once, written once
+    return {
+        "workload": "16384 x 16384 CSR, rows = noisy copies of 256 prototypes (nnz %d), shuffled; V=8" % rnnz,
+        "order_ms": t_order, "order_alg_bytes": by_order, "order_hbm_gbps": by_order / t_order / 1e6,
+        "apply_ms": t_apply, "apply_alg_bytes": by_apply, "apply_hbm_gbps": by_apply / t_apply / 1e6,
+        "nvec_without_reordering": int(plain.num_vec), "nvec_with_reordering": int(reo.svc.num_vec),
+        "fill_without_reordering": rnnz / (plain.num_vec * 8.0), "fill_with_reordering": rnnz / (reo.svc.num_vec * 8.0),
+    }
+
+
+ATTENTION = "sparse_attention_seq4096_d64_v8_s0.9_heads48"
+GROUPS = ["cfg1_rowmerge_then_spmm_512x512", "cfg4", "cfg5_encoder_layer_v16_s0.9_tokens4096", ATTENTION,
+          "reorder_clustered_16384_v8", "headline_batched_cold"]
+
+
+def headline_cold(L, torch, synth, batch, st, wu):
+    """The headline launch with nothing left in a cache from the launch before: two complete operand sets (values, B,
+    C: 2 x 329 MB, more than the 256 MB memory-side cache) used in turn."""
+    M, K, V, N = 2048, 512, 8, 256
+    vs = synth.vector_sparse(M, K, V, 0.9, seed=2, std=0.02)
+    ro, ci = torch.from_numpy(vs.row_offsets).cuda(), torch.from_numpy(vs.col_idx).cuda()
+    nv = vs.col_idx.size
+    g = torch.Generator(device="cuda").manual_seed(3)
+    sets = []
+    for _ in range(2):
+        sets.append(((torch.randn(batch, nv * V, generator=g, device="cuda") * 0.02).half(),
+                     torch.randn(batch, K, N, generator=g, device="cuda").half(),
+                     torch.empty(batch, M, N, dtype=torch.float32, device="cuda")))
+    stream = torch.cuda.current_stream().cuda_stream
+    turn = [0]
+
+    def launch():
+        vals, B, C = sets[turn[0] & 1]
+        turn[0] += 1
+        rc = L.sspmm_batched_f16_f32(batch, vs.m_vec, V, N, K, None, ro.data_ptr(), ci.data_ptr(), vals.data_ptr(), nv * V,
+                                     B.data_ptr(), K * N, C.data_ptr(), M * N, stream)
+        assert rc == 0, rc
+
+    stt = {}
+    ms = time_launches(launch, st, wu, stats=stt)
+    by = batch * synth.spmm_algorithmic_bytes(vs.m_vec, V, nv, K, N, 4) - (batch - 1) * (4 * nv + 4 * (vs.m_vec + 1))
+    res = {"workload": "the headline launch (batch %d), two operand sets of %d MB in rotation" % (batch, by // 1000000)}
+    res.update(figures(ms, by, 2.0 * vs.nnz * N * batch))
+    res.update(stt)
+    return res
+
+
+def run_extra(name, env):
+    """One entry (or group of entries) of `extra` by name; returns a dict name -> figures."""
+    L, torch, synth, sspmm_amd, O, st, wu, batch = (env[k] for k in ("L", "torch", "synth", "sspmm_amd", "O", "st", "wu", "batch"))
+    cases = single_launch_cases(batch)
+    if name in cases:
+        kw = cases[name]
+        res = spmm_case(L, torch, synth, steps=st, warmup=wu, dense=True, graph=kw["batch"] == 1, **kw)
+        torch.cuda.empty_cache()
+        return {name: res}
+    if name == "cfg1_rowmerge_then_spmm_512x512":
+        return {name: run_cfg1(L, torch, synth, sspmm_amd, O, st, wu)}
+    if name == "cfg4":
+        return run_cfg4(L, torch, synth, sspmm_amd, O, st, wu)
+    if name == "cfg5_encoder_layer_v16_s0.9_tokens4096":
+        return {name: run_cfg5_layer(L, torch, synth, st, wu)}
+    if name == ATTENTION:
+        return {name: attention_block(torch, synth, sspmm_amd, st, wu)}
+    if name == "reorder_clustered_16384_v8":
+        return {name: run_reorder(L, torch, synth, sspmm_amd)}
+    if name == "headline_batched_cold":
+        return {name: headline_cold(L, torch, synth, batch, st, wu)}
+    raise SystemExit("unknown entry %r (see --list)" % name)
+
+
 def main():
     args = parse_args()
+    if args.list:
+        print("\n".join(list(single_launch_cases(args.batch)) + GROUPS))
+        return
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU leg (vector-rows shard without "
               "communication); run with --gpus 1", file=sys.stderr)
@@ -172,9 +582,17 @@ def main():
     L = _lib.lib()
     torch.cuda.set_device(0)
     L.sspmm_select_kernel({"auto": 0, "generic": 1, "gather": 2, "slab": 3}[args.kernel])
-    if args.attention_only:
-        print(json.dumps({"sparse_attention_seq4096_d64_v8_s0.9_heads48":
-                          attention_block(torch, synth, sspmm_amd, args.steps, args.warmup)}))
+    env = {"L": L, "torch": torch, "synth": synth, "sspmm_amd": sspmm_amd, "O": None, "st": args.steps, "wu": args.warmup,
+           "batch": args.batch}
+    only = [ATTENTION] if args.attention_only else [n for n in args.only.split(",") if n]
+    if only:
+        from oracle import oracle as O
+        O.build()
+        env["O"] = O
+        out = {}
+        for n in only:
+            out.update(run_extra(n, env))
+        print(json.dumps(out))
         return
 
     if args.calibrate_copy:
@@ -186,13 +604,13 @@ def main():
         del src, dst
 
     M, K, V, sparsity, N = 2048, 512, 8, 0.9, 256
-    kernel_names = {1: "spmm_generic_kernel<8,float>", 2: "spmm_gather_kernel<8,float>", 3: "spmm_slab_kernel<8,float,*,4>",
-                    4: "spmm_gather_split_kernel<8,float>", 5: "spmm_slab_kernel<8,float,*,2>", 6: "spmm_stage_kernel<8,float>"}
-    series = []
-    main_res, (vs, vals, B, C) = spmm_case(L, torch, synth, M, K, V, sparsity, N, args.batch, True, 0.02, 2,
-                                           args.steps, args.warmup, dense=not args.quick, series=series)
+    series, handles = [], []
+    main_res = spmm_case(L, torch, synth, M, K, V, sparsity, N, args.batch, True, 0.02, 2, args.steps, args.warmup,
+                         dense=not args.quick, series=series, handles_out=handles)
+    vs, vals, B, C = handles
     torch.cuda.synchronize()
-    main_kernel = kernel_names.get(L.sspmm_last_kernel(), "unknown")
+    main_kernel = {3: "spmm_slab_kernel<8,float,*,4>", 2: "spmm_gather_kernel<8,float>", 1: "spmm_generic_kernel<8,float>",
+                   6: "spmm_stage_kernel<8,float>"}.get(L.sspmm_last_kernel(), "unknown")
 
     # the same workload as 128 separate launches, one batch element each, rotating through the 335 MB of distinct
     # operands (nothing a launch touches is still in a cache from the launch before): per-launch time when
@@ -212,9 +630,9 @@ def main():
 
         cold_ms = time_launches(one_cold, 4 * args.batch, args.batch)
         one_bytes = synth.spmm_algorithmic_bytes(vs.m_vec, V, vs.col_idx.size, K, N, 4)
-        cold = {"workload": "one batch element per launch, %d distinct operand sets in rotation" % args.batch,
-                "ms": cold_ms, "useful_tflops": 2.0 * vs.nnz * N / cold_ms / 1e9, "alg_bytes": one_bytes,
-                "hbm_gbps": one_bytes / cold_ms / 1e6, "hbm_frac": one_bytes / cold_ms / 1e6 / HBM_PEAK_GBPS}
+        cold = {"workload": "one batch element per launch, %d distinct operand sets in rotation" % args.batch}
+        cold.update(figures(cold_ms, one_bytes, 2.0 * vs.nnz * N))
+        # (leaves C as the batched launch wrote it: same operands, same results)
 
     # what this box's memory system sustains for plain streams of the same size class, measured the same way
     # (50 launches after warm-up): a device copy (half reads, half writes) and a fill (writes only)
@@ -229,25 +647,35 @@ def main():
         ceilings["frac_of_device_copy"] = main_res["hbm_gbps"] / ceilings["device_copy_1GiB_gbps"]
         del src, dst
 
-    # parity of batch element 0 against the CPU oracle, and the CPU baseline on the same element
+    # parity of batch elements spread over the launch (first, last, and one per way the batch is dealt to the XCDs)
+    # against the CPU oracle, and the CPU baseline on element 0
     cpu = None
     parity = None
     if not args.quick:
         from oracle import oracle as O
         O.build()
+        env["O"] = O
+        ncores = os.cpu_count()
+        errs = {}
+        for b in sorted(set(x for x in (0, 7, 8, 63, args.batch // 2 + 1, args.batch - 1) if 0 <= x < args.batch)):
+            want_b = O.spmm(vs.m_vec, V, N, K, vs.row_offsets, vs.col_idx, vals[b].cpu().numpy(), B[b].cpu().numpy(),
+                            threads=min(ncores, 16))
+            errs[b] = float(np.abs(C[b].cpu().numpy() - want_b).max() / max(np.abs(want_b).max(), 1e-30))
+        parity = max(errs.values())
+        if not parity <= 1e-2:
+            print("bench.py: the timed launch disagrees with the host loop: max relative error per batch element %r"
+                  % errs, file=sys.stderr)
+            sys.exit(3)
         v0 = vals[0].cpu().numpy()
         b0 = B[0].cpu().numpy()
         t0 = time.perf_counter()
         reps = 0
         while True:
-            want = O.spmm(vs.m_vec, V, N, K, vs.row_offsets, vs.col_idx, v0, b0, threads=1)
+            O.spmm(vs.m_vec, V, N, K, vs.row_offsets, vs.col_idx, v0, b0, threads=1)
             reps += 1
             if time.perf_counter() - t0 > 10.0 or reps >= 200:
                 break
         cpu_s = (time.perf_counter() - t0) / reps
-        got = C[0].cpu().numpy()
-        parity = float(np.abs(got - want).max() / max(np.abs(want).max(), 1e-30))
-        ncores = os.cpu_count()
         t0 = time.perf_counter()
         O.spmm(vs.m_vec, V, N, K, vs.row_offsets, vs.col_idx, v0, b0, threads=min(ncores, 16))
         cpu_mt_s = time.perf_counter() - t0
@@ -255,8 +683,8 @@ def main():
                "sample": "%d repeats of one batch element (A 2048x512 V=8 s=0.9, B 512x256), host loop of "
                          "sspmm_test.cpp:75-95 in C, -O2, single thread; %.1f ms each" % (reps, cpu_s * 1e3),
                "all_cores_value": 2.0 * vs.nnz * N / cpu_mt_s / 1e12, "all_cores": min(ncores, 16),
-               "host_cpus": ncores}
-    del vals, B, C
+               "host_cpus": ncores, "parity_checked_batch_elements": sorted(errs)}
+    del vals, B, C, handles
 
     extra = {}
     # launch time (us) averaged over chunks of 100 launches, from the first warm-up launch to the last timed one
@@ -265,6 +693,8 @@ def main():
         part = [v for v in series[i:i + 10] if v is not None]
         per100.append(round(sum(part) / len(part), 1) if part else None)
     extra["headline_us_per_chunk"] = {"chunk": 100, "warmup_chunks": (args.warmup + 99) // 100, "us": per100}
+    extra["headline_launch_ms_median_min"] = {"ms_median": main_res["ms_median"], "ms_min": main_res["ms_min"],
+                                              "hbm_frac_at_min": main_res["hbm_frac_at_min"]}
     # the window the reference's harness times (200 launches after 10 warm-ups, sspmm_test.cpp:22-23,181-195), read
     # from the same series: launches 10..209 of this process, while the clocks are still settling
     if args.warmup >= 220 and all(v is not None for v in series[1:21]):
@@ -273,183 +703,9 @@ def main():
     if cold:
         extra["cfg2_single_launches_cold"] = cold
     if not args.quick:
-        st, wu = args.steps, args.warmup  # (the other shapes meet the same clock transient)
-        cases = {
-            "cfg2_single_launch": dict(M=2048, K=512, V=8, sparsity=0.9, N=256, batch=1, out_f32=True, std=0.02, seed=2),
-            "cfg2_batched_fp16_out": dict(M=2048, K=512, V=8, sparsity=0.9, N=256, batch=args.batch, out_f32=False,
-                                          std=0.02, seed=2),
-            "cfg2_shape_v16_batched": dict(M=2048, K=512, V=16, sparsity=0.9, N=256, batch=args.batch, out_f32=True,
-                                           std=0.02, seed=2),
-            "cfg2_shape_v16_batched_fp16_out": dict(M=2048, K=512, V=16, sparsity=0.9, N=256, batch=args.batch,
-                                                    out_f32=False, std=0.02, seed=2),
-            "cfg3_1024x2304_v16_s0.8_n3136": dict(M=1024, K=2304, V=16, sparsity=0.8, N=3136, batch=1, out_f32=True,
-                                                  std=0.05, seed=3),
-            "cfg3_2048x1024_v16_s0.95_n3136": dict(M=2048, K=1024, V=16, sparsity=0.95, N=3136, batch=1,
-                                                   out_f32=True, std=0.05, seed=3),
-            "cfg5_ffn1_3072x768_v16_s0.9_n4096": dict(M=3072, K=768, V=16, sparsity=0.9, N=4096, batch=1,
-                                                      out_f32=False, std=0.02, seed=5),
-            "cfg5_ffn2_768x3072_v16_s0.9_n4096": dict(M=768, K=3072, V=16, sparsity=0.9, N=4096, batch=1,
-                                                      out_f32=False, std=0.02, seed=5),
-            "cfg5_ffn1_batched8": dict(M=3072, K=768, V=16, sparsity=0.9, N=4096, batch=8, out_f32=False, std=0.02,
-                                       seed=5),
-        }
-        for name, kw in cases.items():
-            res, handles = spmm_case(L, torch, synth, steps=st, warmup=wu, dense=True, **kw)
-            del handles
-            torch.cuda.empty_cache()
-            extra[name] = res
-
-        # SVC: cfg4 (Zipf CSR 16384^2) on the GPU against the Python RowMerge and the C oracle
-        from oracle import oracle as O
-        csr = synth.zipf_csr(16384, 16384, seed=4)
-        rp, ci, cv = (torch.from_numpy(x).cuda() for x in (csr.row_ptr, csr.col_ind, csr.values))
-        r = sspmm_amd.svc(rp, ci, cv, csr.M, csr.K, 8)
-        torch.cuda.synchronize()
-        svc_ms = time_launches(lambda: sspmm_amd.svc(rp, ci, cv, csr.M, csr.K, 8), 20, 3)
-        # kernels only (no allocation, no host read-back)
-        ws = torch.empty(L.svc_workspace_bytes(csr.M, csr.col_ind.size, 8), dtype=torch.uint8, device="cuda")
-        vrp = torch.zeros(csr.M // 8 + 1, dtype=torch.int32, device="cuda")
-        vcol = torch.empty(r.num_vec, dtype=torch.int32, device="cuda")
-        vval = torch.empty(r.num_vec * 8, dtype=torch.float16, device="cuda")
-        stream = torch.cuda.current_stream().cuda_stream
-
-        def svc_kernels():
-            L.svc_count(csr.M, csr.K, 8, rp.data_ptr(), ci.data_ptr(), csr.col_ind.size, 0, vrp.data_ptr(),
-                        ws.data_ptr(), stream)
-            L.svc_fill(csr.M, csr.K, 8, rp.data_ptr(), ci.data_ptr(), cv.data_ptr(), csr.col_ind.size, 0,
-                       vrp.data_ptr(), ws.data_ptr(), vcol.data_ptr(), vval.data_ptr(), stream)
-
-        svc_k_ms = time_launches(svc_kernels, 20, 3)
-        lists = O.csr_col_lists(csr.M, csr.row_ptr, csr.col_ind)
-        t0 = time.perf_counter()
-        ptr, flat = O.rowmerge_python(csr.M, 8, lists)
-        py_ms = (time.perf_counter() - t0) * 1e3
-        t0 = time.perf_counter()
-        O.svc(csr.M, csr.K, 8, csr.row_ptr, csr.col_ind, csr.values)
-        c_ms = (time.perf_counter() - t0) * 1e3
-        same = (r.vec_row_ptr.cpu().numpy().tolist() == ptr) and (r.vec_col.cpu().numpy().tolist() == flat)
-        nnz = csr.col_ind.size
-        svc_bytes = synth.svc_algorithmic_bytes(csr.M, nnz, csr.M // 8, r.num_vec, 8)
-        extra["svc_cfg4_zipf_16384_v8"] = {
-            "gpu_ms_with_alloc_and_readback": svc_ms, "gpu_ms_kernels": svc_k_ms, "python_rowmerge_ms": py_ms,
-            "c_oracle_ms": c_ms, "speedup_vs_python": py_ms / svc_k_ms, "bit_exact_vs_python": bool(same),
-            "nnz": int(nnz), "nvec": int(r.num_vec), "fill_ratio": nnz / (r.num_vec * 8.0),
-            "max_vector_row": int(np.diff(r.vec_row_ptr.cpu().numpy()).max()),
-            "alg_bytes": svc_bytes, "hbm_gbps": svc_bytes / svc_k_ms / 1e6,
-        }
-
-        # the same pass on the shape of the matrices the reference's RowMerge is run on (its dataset of pruned
-        # transformer weights): 2048 x 2048, 90 % of the entries zero at random, V = 8 and 16
-        rng_d = np.random.default_rng(7)
-        mask_d = rng_d.random((2048, 2048)) < 0.1
-        d_ptr = np.concatenate([[0], np.cumsum(mask_d.sum(axis=1))]).astype(np.int32)
-        d_col = np.nonzero(mask_d)[1].astype(np.int32)
-        d_rp, d_ci = torch.from_numpy(d_ptr).cuda(), torch.from_numpy(d_col).cuda()
-        d_lists = O.csr_col_lists(2048, d_ptr, d_col)
-        for Vd in (8, 16):
-            rd = sspmm_amd.svc(d_rp, d_ci, None, 2048, 2048, Vd)
-            d_ms = time_launches(lambda: sspmm_amd.svc(d_rp, d_ci, None, 2048, 2048, Vd), 20, 3)
-            t0 = time.perf_counter()
-            d_want_ptr, d_want_cols = O.rowmerge_python(2048, Vd, d_lists)
-            d_py = (time.perf_counter() - t0) * 1e3
-            extra["svc_pruned_weight_2048x2048_s0.9_v%d" % Vd] = {
-                "gpu_ms_with_alloc_and_readback": d_ms, "python_rowmerge_ms": d_py, "speedup_vs_python": d_py / d_ms,
-                "bit_exact_vs_python": bool(rd.vec_row_ptr.cpu().numpy().tolist() == d_want_ptr and
-                                            rd.vec_col.cpu().numpy().tolist() == d_want_cols),
-                "nnz": int(d_col.size), "nvec": int(rd.num_vec),
-            }
-
-        # ... and the SpMM that consumes it: the skewed pattern straight from the SVC, B 16384 x 256
-        N4 = 256
-        B4 = torch.from_numpy(synth.dense_rhs(csr.K, N4, seed=14)).cuda()
-        C4 = torch.empty(csr.M, N4, dtype=torch.float32, device="cuda")
-        m_vec4 = csr.M // 8
-
-        def spmm_cfg4():
-            rc = L.sspmm_f16_f32(m_vec4, 8, N4, csr.K, None, r.vec_row_ptr.data_ptr(), r.vec_col.data_ptr(),
-                                 r.vec_val.data_ptr(), B4.data_ptr(), C4.data_ptr(), stream)
-            assert rc == 0, rc
-
-        ms4 = time_launches(spmm_cfg4, st, wu)
-        lens = np.diff(r.vec_row_ptr.cpu().numpy())
-        touched = int(np.unique(r.vec_col.cpu().numpy()).size)
-        bytes4 = synth.spmm_algorithmic_bytes(m_vec4, 8, int(r.num_vec), csr.K, N4, 4, k_touched=touched)
-        extra["cfg4_spmm_on_svc_output"] = {
-            "workload": "A 16384x16384 Zipf rows (nnz %d) after SVC V=8, B 16384x%d, C fp32" % (nnz, N4),
-            "ms": ms4, "useful_tflops": 2.0 * nnz * N4 / ms4 / 1e9, "alg_bytes": bytes4,
-            "hbm_gbps": bytes4 / ms4 / 1e6, "hbm_frac": bytes4 / ms4 / 1e6 / HBM_PEAK_GBPS,
-            "kernel": kernel_names.get(L.sspmm_last_kernel(), "unknown"),
-            "vector_row_len_max": int(lens.max()), "vector_row_len_mean": float(lens.mean()),
-            "steps_of_longest_row": int((lens.max() + 31) // 32), "steps_total": int(((lens + 31) // 32).sum()),
-        }
-
-        # cfg5: one BERT-base shaped encoder layer (hidden 768, 12 heads, FFN 3072, 8 x 512 tokens) with
-        # six vector-sparse weights (V=16, 90 %) and dense attention in torch; the same layer with dense fp16
-        # matmuls on the densified weights beside it
-        from sspmm_amd.layers import SparseEncoderLayer, SparseLinear
-        hid, heads, ffn, V5, bsz, seq = 768, 12, 3072, 16, 8, 512
-
-        def mk(o, i, seed):
-            w = synth.vector_sparse(o, i, V5, 0.9, seed=seed, std=0.02)
-            return SparseLinear.from_cvse(i, V5, torch.from_numpy(w.row_offsets).cuda(), torch.from_numpy(w.col_idx).cuda(),
-                                          torch.from_numpy(w.values).cuda())
-
-        layer = SparseEncoderLayer(hid, heads, ffn, mk(hid, hid, 51), mk(hid, hid, 52), mk(hid, hid, 53), mk(hid, hid, 54),
-                                   mk(ffn, hid, 55), mk(hid, ffn, 56)).cuda().half()
-        x5 = (torch.randn(hid, bsz * seq, device="cuda") * 1.0).half()
-        dense_w = {n: getattr(layer, n).dense_weight() for n in ("q", "k", "v", "o", "ffn1", "ffn2")}
-        with torch.no_grad():
-            y_sp = layer(x5, bsz, seq)
-            y_de = layer(x5, bsz, seq, linear=lambda n, lin, t: dense_w[n] @ t)
-            sp_ms = time_launches(lambda: layer(x5, bsz, seq), st, wu)
-            de_ms = time_launches(lambda: layer(x5, bsz, seq, linear=lambda n, lin, t: dense_w[n] @ t), st, wu)
-            per = {}
-            for n in ("q", "o", "ffn1", "ffn2"):
-                lin = getattr(layer, n)
-                xin = torch.randn(lin.in_features, bsz * seq, device="cuda").half()
-                per[n] = {"sparse_ms": time_launches(lambda: lin(xin), st, wu),
-                          "dense_ms": time_launches(lambda: dense_w[n] @ xin, st, wu)}
-        extra["cfg5_encoder_layer_v16_s0.9_tokens4096"] = {
-            "sparse_layer_ms": sp_ms, "dense_layer_ms": de_ms, "speedup_vs_dense_layer": de_ms / sp_ms,
-            "max_rel_diff_vs_dense_layer": float((y_sp.float() - y_de.float()).abs().max() / y_de.float().abs().max()),
-            "projections": per,
-        }
-
-        extra["sparse_attention_seq4096_d64_v8_s0.9_heads48"] = attention_block(torch, synth, sspmm_amd, st, wu)
-
-        # row reordering ahead of the SVC: 16384 rows that are noisy copies of 256 prototype rows, shuffled
-        rc_csr = synth.clustered_csr(16384, 16384, 256, 128, seed=6, keep=0.9, extras=1)
-        rrp, rci, rcv = (torch.from_numpy(x).cuda() for x in (rc_csr.row_ptr, rc_csr.col_ind, rc_csr.values))
-        plain = sspmm_amd.svc(rrp, rci, rcv, rc_csr.M, rc_csr.K, 8, order="sorted")
-        reo = sspmm_amd.svc_reordered(rrp, rci, rcv, rc_csr.M, rc_csr.K, 8, order="sorted")
-        rws = torch.empty(L.svc_reorder_workspace_bytes(rc_csr.M), dtype=torch.uint8, device="cuda")
-        rperm = torch.empty(rc_csr.M, dtype=torch.int32, device="cuda")
-        o_rp, o_ci, o_cv = torch.empty_like(rrp), torch.empty_like(rci), torch.empty_like(rcv)
-
-        def reorder_order():
-            rc = L.svc_reorder_minhash(rc_csr.M, rrp.data_ptr(), rci.data_ptr(), rperm.data_ptr(), rws.data_ptr(),
-                                       rws.numel(), stream)
-            assert rc == 0, rc
-
-        def reorder_apply():
-            rc = L.svc_permute_csr(rc_csr.M, rperm.data_ptr(), rrp.data_ptr(), rci.data_ptr(), rcv.data_ptr(),
-                                   o_rp.data_ptr(), o_ci.data_ptr(), o_cv.data_ptr(), rws.data_ptr(), rws.numel(),
-                                   stream)
-            assert rc == 0, rc
-
-        reorder_order()
-        t_order = time_launches(reorder_order, 20, 3)
-        t_apply = time_launches(reorder_apply, 20, 3)
-        rnnz = int(rc_csr.col_ind.size)
-        by_order = 4 * (rc_csr.M + 1) + 4 * rnnz + 4 * rc_csr.M   # row pointer + columns read, order written
-        by_apply = 4 * rc_csr.M + 2 * 4 * (rc_csr.M + 1) + 2 * (4 + 2) * rnnz  # CSR read once, written once
-        extra["reorder_clustered_16384_v8"] = {
-            "workload": "16384 x 16384 CSR, rows = noisy copies of 256 prototypes (nnz %d), shuffled; V=8" % rnnz,
-            "order_ms": t_order, "order_alg_bytes": by_order, "order_hbm_gbps": by_order / t_order / 1e6,
-            "apply_ms": t_apply, "apply_alg_bytes": by_apply, "apply_hbm_gbps": by_apply / t_apply / 1e6,
-            "nvec_without_reordering": int(plain.num_vec), "nvec_with_reordering": int(reo.svc.num_vec),
-            "fill_without_reordering": rnnz / (plain.num_vec * 8.0), "fill_with_reordering": rnnz / (reo.svc.num_vec * 8.0),
-        }
+        for name in list(single_launch_cases(args.batch)) + GROUPS:
+            extra.update(run_extra(name, env))
+        extra["measured_hbm_traffic"] = MEASURED_TRAFFIC
 
     line = {
         "metric": "SpMM useful TFLOP/s (2*nnz*N/t), V=8 @90% sparsity, fp16 in / fp32 accumulate",
@@ -460,8 +716,11 @@ def main():
                    "hbm_gbps": main_res["hbm_gbps"]},
         "roofline": {"bound": "hbm", "achieved": main_res["hbm_gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": main_res["hbm_frac"],
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.batch) if args.kernel == "auto" else None,
+                     "traffic": MEASURED_TRAFFIC["headline_batch128"]["bytes"] if (args.kernel == "auto" and args.batch == 128) else None,
+                     "traffic_source": MEASURED_TRAFFIC["headline_batch128"]["source"],
                      "kernel": main_kernel, "alg_bytes_per_launch": main_res["alg_bytes"],
+                     "operands": "warm: the same 329 MB of operands every launch (the cold rotation of two sets is "
+                                 "extra.headline_batched_cold)",
                      "measured_stream_rates": ceilings},
         "cpu_baseline": cpu,
         "parity_max_rel_err": parity,

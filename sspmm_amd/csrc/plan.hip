@@ -102,7 +102,7 @@ hipError_t launch_spmm_planned(const Plan &pl, const SpmmArgs &a, bool out_f16, 
   // an even pattern keeps the kernels chosen by shape.
   const bool skewed = pl.header[kHdrSplitRows] > 0;
   if (can_balance && (forced == 7 || (forced == 0 && skewed)))
-    return launch_spmm_balanced(a, pl.V, out_f16, pl.view, pl.header[kHdrItems], stream);
+    return launch_spmm_balanced(a, pl.V, out_f16, pl.view, pl.header[kHdrItems], false, stream);
   return launch_spmm(a, pl.V, out_f16, stream);
 }
 
@@ -111,7 +111,8 @@ hipError_t launch_spmm_planned(const Plan &pl, const SpmmArgs &a, bool out_f16, 
 // call inside a captured graph, a serving loop, a harness that forbids allocation): the schedule, its counters and
 // the partial tiles live in one array of device memory that is part of the library's code object, so every GPU the
 // library runs on holds it from the first use of the library to the end of the process.  The schedule is built on
-// the device by every call (the host never sees the row offsets), and a grid of fixed size walks it.
+// the device by every call (the host never sees the row offsets); the product's grid covers the most items the
+// schedule can have, and the workgroups beyond its end return at once.
 static constexpr int kStaticMaxRows = 32768;       // vector-rows
 static constexpr int kStaticMaxN = 4096;           // columns of B: 64 column tiles
 static constexpr int64_t kStaticMaxSlots = 4096;   // panels of cut rows
@@ -163,11 +164,14 @@ hipError_t launch_spmm_static(const SpmmArgs &a, int V, bool out_f16, hipStream_
   if (slot_cap > kStaticMaxSlots) slot_cap = kStaticMaxSlots;
   // Everything the product reads is rewritten first: header, items, and the counters of the rows that are cut
   // (kernels on the caller's stream, which order themselves; no memset node for a capturing caller).
-  if ((e = launch_schedule_measure(a.m_vec, a.row_offsets, 0, slot_cap, view.header, stream)) != hipSuccess) return e;
-  if ((e = launch_schedule_fill(a.m_vec, a.row_offsets, view, (int64_t)kStaticMaxRows + kStaticMaxSlots, -1, tiles, stream)) !=
-      hipSuccess)
+  if ((e = launch_schedule_build(a.m_vec, a.row_offsets, slot_cap, view, (int64_t)kStaticMaxRows + kStaticMaxSlots, tiles,
+                                 stream)) != hipSuccess)
     return e;
-  return launch_spmm_balanced(a, V, out_f16, view, -1, stream);
+  // The schedule has at most one item per row that stays whole plus the panels of the cut rows; a row holds at most
+  // K vectors (ceil(K / 32) steps) and a panel at least kScheduleMinBudget steps.
+  int64_t panels_bound = (int64_t)a.m_vec * ((int64_t)a.K / (32 * kScheduleMinBudget) + 2);
+  if (panels_bound > slot_cap) panels_bound = slot_cap;
+  return launch_spmm_balanced(a, V, out_f16, view, a.m_vec + (int)panels_bound, true, stream);
 }
 
 }  // namespace sspmm

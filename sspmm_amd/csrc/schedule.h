@@ -61,5 +61,10 @@ hipError_t launch_schedule_measure(int m_vec, const int32_t *row_offsets, int bu
 hipError_t launch_schedule_fill(int m_vec, const int32_t *row_offsets, const ScheduleView &view, int64_t item_cap,
                                 int64_t counters_to_clear, int64_t counters_per_cut_row, hipStream_t stream);
 
+// launch_schedule_measure (budget chosen from the pattern) and launch_schedule_fill (clearing the counters of the
+// cut rows) as one launch.
+hipError_t launch_schedule_build(int m_vec, const int32_t *row_offsets, int64_t slot_cap, const ScheduleView &view,
+                                 int64_t item_cap, int64_t counters_per_cut_row, hipStream_t stream);
+
 }  // namespace sspmm
 #endif

@@ -38,10 +38,8 @@ __device__ __forceinline__ int block_max(int x, unsigned long long *scratch) {
   return s;
 }
 
-__global__ __launch_bounds__(kBuildThreads) void schedule_measure_kernel(int m_vec, const int32_t *__restrict__ row_offsets,
-                                                                         int budget_in, long long slot_cap,
-                                                                         int32_t *__restrict__ header) {
-  __shared__ unsigned long long scratch[kBuildThreads / 64];
+__device__ __forceinline__ void schedule_measure(int m_vec, const int32_t *__restrict__ row_offsets, int budget_in,
+                                                 long long slot_cap, int32_t *header, unsigned long long *scratch) {
   unsigned long long steps_sum = 0;
   int steps_max = 0;
   for (int r = threadIdx.x; r < m_vec; r += kBuildThreads) {
@@ -84,6 +82,13 @@ __global__ __launch_bounds__(kBuildThreads) void schedule_measure_kernel(int m_v
   }
 }
 
+__global__ __launch_bounds__(kBuildThreads) void schedule_measure_kernel(int m_vec, const int32_t *__restrict__ row_offsets,
+                                                                         int budget_in, long long slot_cap,
+                                                                         int32_t *__restrict__ header) {
+  __shared__ unsigned long long scratch[kBuildThreads / 64];
+  schedule_measure(m_vec, row_offsets, budget_in, slot_cap, header, scratch);
+}
+
 // Exclusive prefix sum of one 64-bit value per thread over the workgroup; *total = sum.  Contains barriers.
 __device__ __forceinline__ unsigned long long block_exclusive_scan64(unsigned long long x, unsigned long long *total,
                                                                       unsigned long long *scratch) {
@@ -108,12 +113,10 @@ __device__ __forceinline__ unsigned long long block_exclusive_scan64(unsigned lo
   return base + incl - x;
 }
 
-__global__ __launch_bounds__(kBuildThreads) void schedule_fill_kernel(int m_vec, const int32_t *__restrict__ row_offsets,
-                                                                      const int32_t *__restrict__ header,
-                                                                      ScheduleItem *__restrict__ items, long long item_cap,
-                                                                      int32_t *__restrict__ counters, long long counters_to_clear,
-                                                                      long long counters_per_cut_row) {
-  __shared__ unsigned long long scratch[kBuildThreads / 64];
+__device__ __forceinline__ void schedule_fill(int m_vec, const int32_t *__restrict__ row_offsets, const int32_t *header,
+                                              ScheduleItem *__restrict__ items, long long item_cap,
+                                              int32_t *__restrict__ counters, long long counters_to_clear,
+                                              long long counters_per_cut_row, unsigned long long *scratch) {
   if (counters_to_clear < 0) counters_to_clear = (long long)header[kHdrSplitRows] * counters_per_cut_row;
   for (long long i = threadIdx.x; i < counters_to_clear; i += kBuildThreads) counters[i] = 0;
   const int budget = header[kHdrBudget];
@@ -174,6 +177,28 @@ __global__ __launch_bounds__(kBuildThreads) void schedule_fill_kernel(int m_vec,
   }
 }
 
+__global__ __launch_bounds__(kBuildThreads) void schedule_fill_kernel(int m_vec, const int32_t *__restrict__ row_offsets,
+                                                                      const int32_t *__restrict__ header,
+                                                                      ScheduleItem *__restrict__ items, long long item_cap,
+                                                                      int32_t *__restrict__ counters, long long counters_to_clear,
+                                                                      long long counters_per_cut_row) {
+  __shared__ unsigned long long scratch[kBuildThreads / 64];
+  schedule_fill(m_vec, row_offsets, header, items, item_cap, counters, counters_to_clear, counters_per_cut_row, scratch);
+}
+
+// Both steps in one launch (the header passes through global memory inside the one workgroup).
+__global__ __launch_bounds__(kBuildThreads) void schedule_build_kernel(int m_vec, const int32_t *__restrict__ row_offsets,
+                                                                       long long slot_cap, int32_t *header,
+                                                                       ScheduleItem *__restrict__ items, long long item_cap,
+                                                                       int32_t *__restrict__ counters,
+                                                                       long long counters_per_cut_row) {
+  __shared__ unsigned long long scratch[kBuildThreads / 64];
+  schedule_measure(m_vec, row_offsets, 0, slot_cap, header, scratch);
+  __threadfence_block();
+  __syncthreads();
+  schedule_fill(m_vec, row_offsets, header, items, item_cap, counters, -1, counters_per_cut_row, scratch);
+}
+
 hipError_t launch_schedule_measure(int m_vec, const int32_t *row_offsets, int budget, int64_t slot_cap, int32_t *header,
                                    hipStream_t stream) {
   hipLaunchKernelGGL(schedule_measure_kernel, dim3(1), dim3(kBuildThreads), 0, stream, m_vec, row_offsets, budget,
@@ -186,6 +211,13 @@ hipError_t launch_schedule_fill(int m_vec, const int32_t *row_offsets, const Sch
   hipLaunchKernelGGL(schedule_fill_kernel, dim3(1), dim3(kBuildThreads), 0, stream, m_vec, row_offsets, view.header,
                      view.items, (long long)item_cap, view.counters, (long long)counters_to_clear,
                      (long long)counters_per_cut_row);
+  return hipGetLastError();
+}
+
+hipError_t launch_schedule_build(int m_vec, const int32_t *row_offsets, int64_t slot_cap, const ScheduleView &view,
+                                 int64_t item_cap, int64_t counters_per_cut_row, hipStream_t stream) {
+  hipLaunchKernelGGL(schedule_build_kernel, dim3(1), dim3(kBuildThreads), 0, stream, m_vec, row_offsets, (long long)slot_cap,
+                     view.header, view.items, (long long)item_cap, view.counters, (long long)counters_per_cut_row);
   return hipGetLastError();
 }
 

@@ -33,13 +33,14 @@ int set_kernel_override(int which);
 // Kernel the latest launch_spmm of the calling thread used (1 scalar, 2 gather, 3 LDS slab; 0 before any launch).
 int last_kernel();
 
-// Load-balanced kernel over a schedule (schedule.h).  n_items: the number of work items when the host knows it
-// (one workgroup per item and column tile), or -1 to let a fixed grid read it from the schedule's header.
+// Load-balanced kernel over a schedule (schedule.h), one workgroup per item and column tile.  n_items: the number of
+// work items; with device_count an upper bound of it (the kernel reads the count from the schedule's header and
+// the workgroups beyond it return at once).
 // Only where balanced_kernel_applies (the MFMA kernels' alignment and size conditions).
 struct ScheduleView;
 bool balanced_kernel_applies(const SpmmArgs &args, int V, bool out_f16);
 hipError_t launch_spmm_balanced(const SpmmArgs &args, int V, bool out_f16, const ScheduleView &schedule, int n_items,
-                                hipStream_t stream);
+                                bool device_count, hipStream_t stream);
 int kernel_override();
 
 hipError_t launch_sorted_row_swizzle(int m_vec, const int32_t *row_offsets, int32_t *row_indices,

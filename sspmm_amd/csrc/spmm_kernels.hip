@@ -1300,7 +1300,7 @@ struct BalancedArgs {
   const ScheduleItem *items;
   int32_t *counters;
   unsigned char *partials;
-  int n_items;            // what the host knows the schedule to hold, or -1: read the header (grid-stride loop)
+  int n_items;            // items the grid covers: the schedule's count, or an upper bound of it
   uint32_t tiles_padded;
 };
 
@@ -1340,28 +1340,26 @@ struct PartialTile {
 static_assert(PartialTile<8>::kLanes * 64u == partial_tile_bytes(8) && PartialTile<16>::kLanes * 64u == partial_tile_bytes(16),
               "a partial tile is four 16-byte pieces per lane that holds rows");
 
-// PERSISTENT: a fixed grid walks the work ids (the number of items is only known on the device).
-template <int V, typename OutT, bool PERSISTENT>
+// DEVICE_COUNT: the number of items is only known on the device; the grid covers an upper bound of it and the
+// workgroups beyond the schedule's end return at once.
+template <int V, typename OutT, bool DEVICE_COUNT>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void spmm_balanced_kernel(const SpmmArgs p, const BalancedArgs s) {
   __shared__ __align__(16) unsigned char stage[32 * kStagePitch];
   __shared__ __align__(16) unsigned char val_tile[val_tile_bytes(V)];
   const int lane = threadIdx.x;
   StageLane<V> x;
   x.init(lane, stage, val_tile);
-  const uint32_t n_items = PERSISTENT ? (uint32_t)s.header[kHdrItems] : (uint32_t)s.n_items;
-  const uint32_t per_batch = n_items * s.tiles_padded;
-  const uint32_t n_units = per_batch * (uint32_t)p.batch;  // (below 2^31: the launcher checks, or bounds, it)
+  // s.n_items: the schedule's item count, or with DEVICE_COUNT the bound the grid was sized for
+  const uint32_t per_batch = (uint32_t)s.n_items * s.tiles_padded;
   const uint32_t b_bytes = (uint32_t)p.K * (uint32_t)p.N * 2u;
   const uint32_t c_vrow_bytes = (uint32_t)V * (uint32_t)p.N * (uint32_t)sizeof(OutT);
-
-  for (uint32_t id = blockIdx.x; id < n_units; id += gridDim.x) {
+  {
+    const uint32_t id = blockIdx.x;
     const uint32_t batch = id / per_batch, rem = id % per_batch;
-    const uint32_t tile = rem % s.tiles_padded;
-    if (tile >= p.n_tiles) {
-      if (PERSISTENT) continue;
-      return;
-    }
-    const ScheduleItem *ip = s.items + rem / s.tiles_padded;
+    const uint32_t tile = rem % s.tiles_padded, item = rem / s.tiles_padded;
+    if (tile >= p.n_tiles) return;
+    if (DEVICE_COUNT && item >= (uint32_t)s.header[kHdrItems]) return;
+    const ScheduleItem *ip = s.items + item;
     // (the item is the same for the whole wave: scalar registers)
     const int row = __builtin_amdgcn_readfirstlane(ip->row), kbeg = __builtin_amdgcn_readfirstlane(ip->kbeg),
               kend = __builtin_amdgcn_readfirstlane(ip->kend), split_id = __builtin_amdgcn_readfirstlane(ip->split_id);
@@ -1396,10 +1394,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
       int seen = 0;
       if (lane == 0) seen = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       seen = __builtin_amdgcn_readfirstlane(seen);
-      if (seen != pieces - 1) {  // other panels of the row are still out: the last one adds up
-        if (PERSISTENT) continue;
-        return;
-      }
+      if (seen != pieces - 1) return;  // other panels of the row are still out: the last one adds up
       asm volatile("" ::: "memory");  // the loads below stay behind the count
       if (lane == 0) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
@@ -1414,7 +1409,6 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
     const __amdgpu_buffer_rsrc_t srd_c = make_srd(reinterpret_cast<OutT *>(p.C) + (int64_t)batch * p.stride_C,
                                                   (uint32_t)p.m_vec * c_vrow_bytes);
     out.store(acc, srd_c, (uint32_t)row * c_vrow_bytes);
-    if (!PERSISTENT) return;
   }
 }
 
@@ -1616,13 +1610,13 @@ bool balanced_kernel_applies(const SpmmArgs &a, int V, bool out_f16) {
 }
 
 template <int V, typename OutT>
-static void launch_balanced_v(const SpmmArgs &p, const BalancedArgs &s, uint32_t grid, hipStream_t stream) {
-  if (s.n_items >= 0) hipLaunchKernelGGL((spmm_balanced_kernel<V, OutT, false>), dim3(grid), dim3(64), 0, stream, p, s);
+static void launch_balanced_v(const SpmmArgs &p, const BalancedArgs &s, uint32_t grid, bool device_count, hipStream_t stream) {
+  if (!device_count) hipLaunchKernelGGL((spmm_balanced_kernel<V, OutT, false>), dim3(grid), dim3(64), 0, stream, p, s);
   else hipLaunchKernelGGL((spmm_balanced_kernel<V, OutT, true>), dim3(grid), dim3(64), 0, stream, p, s);
 }
 
 hipError_t launch_spmm_balanced(const SpmmArgs &a, int V, bool out_f16, const ScheduleView &sv, int n_items,
-                                hipStream_t stream) {
+                                bool device_count, hipStream_t stream) {
   SpmmArgs p = a;
   p.n_tiles = (uint32_t)((a.N + 63) / 64);
   BalancedArgs s;
@@ -1632,22 +1626,17 @@ hipError_t launch_spmm_balanced(const SpmmArgs &a, int V, bool out_f16, const Sc
   s.partials = sv.partials;
   s.n_items = n_items;
   s.tiles_padded = padded_tiles(p.n_tiles);
-  uint32_t grid;
-  if (n_items >= 0) {
-    const uint64_t units = (uint64_t)n_items * s.tiles_padded * (uint64_t)a.batch;
-    if (units >= (1ull << 31)) return hipErrorInvalidValue;
-    if (units == 0) return hipSuccess;
-    grid = (uint32_t)units;
-  } else {
-    grid = 32u * device_cus();  // a multiple of 8: a workgroup's ids stay on one XCD through the grid-stride loop
-  }
+  const uint64_t units = (uint64_t)n_items * s.tiles_padded * (uint64_t)a.batch;
+  if (units >= (1ull << 31)) return hipErrorInvalidValue;
+  if (units == 0) return hipSuccess;
+  const uint32_t grid = (uint32_t)units;
   g_last_kernel = 7;
   if (V == 8) {
-    if (out_f16) launch_balanced_v<8, _Float16>(p, s, grid, stream);
-    else launch_balanced_v<8, float>(p, s, grid, stream);
+    if (out_f16) launch_balanced_v<8, _Float16>(p, s, grid, device_count, stream);
+    else launch_balanced_v<8, float>(p, s, grid, device_count, stream);
   } else {
-    if (out_f16) launch_balanced_v<16, _Float16>(p, s, grid, stream);
-    else launch_balanced_v<16, float>(p, s, grid, stream);
+    if (out_f16) launch_balanced_v<16, _Float16>(p, s, grid, device_count, stream);
+    else launch_balanced_v<16, float>(p, s, grid, device_count, stream);
   }
   return hipGetLastError();
 }

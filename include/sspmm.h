@@ -260,6 +260,21 @@ int svc_permute_csr(int M, const int32_t *perm, const int32_t *row_ptr, const in
                     const sspmm_half_t *csr_val, int32_t *out_row_ptr, int32_t *out_col, sspmm_half_t *out_val,
                     void *workspace, size_t workspace_bytes, void *hip_stream);
 
+/* ------------------------------------------------------------------------------------------
+ * Coordinate list -> CSR, the step between a Matrix Market file and the RowMerge in the
+ * reference's SuiteSparse path: `csr = self.coo.tocsr()` in suite_matrix.coo2csr, reference
+ * RowMerge/suit_sparse_matrix.py:109-111 (scipy: rows ascending, inside a row the columns
+ * ascending, a (row, column) pair that occurs several times kept once).
+ *   coo_row[n], coo_col[n]  zero-based entries in any order; entries outside [0, M) x [0, K) are dropped
+ *   row_ptr[M + 1]          row_ptr[M] is the number of entries that remain (read it back)
+ *   col_ind[n]              sized for the case that nothing merges
+ * workspace of svc_coo_workspace_bytes(n) bytes (0 = no usable device).
+ * ---------------------------------------------------------------------------------------- */
+size_t svc_coo_workspace_bytes(int64_t n);
+
+int svc_coo_to_csr(int M, int K, int64_t n, const int32_t *coo_row, const int32_t *coo_col, int32_t *row_ptr,
+                   int32_t *col_ind, void *workspace, size_t workspace_bytes, void *hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

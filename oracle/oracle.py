@@ -192,6 +192,19 @@ def rowmerge_python(M, V, col_lists):
     return ptr, flat
 
 
+def coo_to_csr(M, K, rows, cols):
+    """The pattern of `coo.tocsr()` as the reference's SuiteSparse path uses it (RowMerge/suit_sparse_matrix.py:
+    109-111): scipy's conversion sorts each row's columns and merges repeated (row, column) pairs; entries
+    outside the matrix are dropped.  Pinned by scipy's own tocsr() and by the reference-written `_csr.mtx` files
+    (tests/test_suitesparse.py)."""
+    rows = np.asarray(rows, dtype=np.int64)
+    cols = np.asarray(cols, dtype=np.int64)
+    ok = (rows >= 0) & (rows < M) & (cols >= 0) & (cols < K)
+    keys = np.unique(rows[ok] * (1 << 32) + cols[ok])
+    row_ptr = np.searchsorted(keys >> 32, np.arange(M + 1), side="left").astype(np.int32)
+    return row_ptr, (keys & 0xffffffff).astype(np.int32)
+
+
 def csr_col_lists(M, row_ptr, col_ind):
     """colInd_list_array of the reference (sparse_matrix_format.py:41-53): per-row python lists."""
     ci = [int(c) for c in col_ind]

@@ -4,6 +4,7 @@
 
 #include "../../include/sspmm.h"
 #include "attention_kernels.h"
+#include "coo_kernels.h"
 #include "plan.h"
 #include "reorder_kernels.h"
 #include "spmm_kernels.h"
@@ -323,6 +324,16 @@ int svc_permute_csr(int M, const int32_t *perm, const int32_t *row_ptr, const in
   return (int)sspmm::launch_permute_csr(M, perm, row_ptr, col_ind, csr_val, out_row_ptr, out_col,
                                         csr_val ? out_val : nullptr, workspace, workspace_bytes,
                                         static_cast<hipStream_t>(hip_stream));
+}
+
+size_t svc_coo_workspace_bytes(int64_t n) { return sspmm::coo_workspace_bytes(n); }
+
+int svc_coo_to_csr(int M, int K, int64_t n, const int32_t *coo_row, const int32_t *coo_col, int32_t *row_ptr,
+                   int32_t *col_ind, void *workspace, size_t workspace_bytes, void *hip_stream) {
+  if (M < 0 || K < 0 || n < 0 || n >= (1ll << 31) - 1 || !row_ptr) return kInvalid;
+  if (n > 0 && (!coo_row || !coo_col || !col_ind || !workspace)) return kInvalid;
+  return (int)sspmm::launch_coo_to_csr(M, K, n, coo_row, coo_col, row_ptr, col_ind, workspace, workspace_bytes,
+                                       static_cast<hipStream_t>(hip_stream));
 }
 
 }  // extern "C"

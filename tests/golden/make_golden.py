@@ -10,6 +10,12 @@ reference's own CVSE class and CVSE_out writer produce:
 The fixtures pin the two things no closed form pins: the byte layout of the
 output file and the column order on realistic merged rows.  Tests read only the
 fixture files; the reference itself is never needed at test time.
+
+The SuiteSparse half (reference RowMerge/suit_sparse_matrix.py) gets the same treatment: seeded
+Matrix Market coordinate files <case>.mtx are written here, and the reference's suite_matrix
+(scipy.io.mmread, coo.tocsr()), its coo2csr(1) writer and CVSE / CVSE_out produce
+  <case>_csr.mtx       the CSR side file, exact bytes
+  <case>.mtx.v<V>.smtx the CVSE file, exact bytes
 """
 import os
 import random
@@ -68,5 +74,61 @@ def main():
             print(name, V, "num_vec_row", c.num_vec_row, "num_vec", c.num_vec)
 
 
+def mtx_cases():
+    """name -> text of a Matrix Market coordinate file."""
+    rng = random.Random(20241125)
+    out = {}
+    # general, real values, entries in shuffled order, some repeated (row, column) pairs, an explicit zero,
+    # empty rows, M not a multiple of 8
+    M, K = 37, 90
+    ent = [(rng.randrange(M), rng.randrange(K)) for _ in range(260)]
+    ent = [e for e in ent if e[0] not in (5, 6, 20)]
+    ent += ent[:9]  # duplicates
+    rng.shuffle(ent)
+    lines = ["%%MatrixMarket matrix coordinate real general", "% shuffled entries with duplicates", "%d %d %d" % (M, K, len(ent))]
+    lines += ["%d %d %s" % (r + 1, c + 1, "0.0" if i == 3 else repr(round(rng.uniform(-2, 2), 4))) for i, (r, c) in enumerate(ent)]
+    out["general_37x90"] = "\n".join(lines) + "\n"
+    # symmetric pattern (lower triangle stored): the reader mirrors the off-diagonal entries
+    n = 48
+    low = sorted(set((max(a, b), min(a, b)) for a, b in ((rng.randrange(n), rng.randrange(n)) for _ in range(150))))
+    rng.shuffle(low)
+    lines = ["%%MatrixMarket matrix coordinate pattern symmetric", "%d %d %d" % (n, n, len(low))]
+    lines += ["%d %d" % (r + 1, c + 1) for r, c in low]
+    out["symmetric_48x48"] = "\n".join(lines) + "\n"
+    # wide integer matrix with a heavy row group (set resizes) and large column numbers
+    M, K = 24, 70000
+    ent = []
+    for r in range(M):
+        cnt = 900 if r in (1, 2, 13) else rng.randrange(0, 12)
+        ent += [(r, c) for c in rng.sample(range(K), cnt)]
+    rng.shuffle(ent)
+    lines = ["%%MatrixMarket matrix coordinate integer general", "%d %d %d" % (M, K, len(ent))]
+    lines += ["%d %d %d" % (r + 1, c + 1, rng.randrange(1, 9)) for r, c in ent]
+    out["skew_24x70000"] = "\n".join(lines) + "\n"
+    return out
+
+
+def main_suitesparse():
+    sys.path.insert(0, "/root/reference/RowMerge")
+    os.environ.setdefault("MPLBACKEND", "Agg")
+    import sparse_matrix_format as ref
+    import suit_sparse_matrix as ref_suite  # the reference itself
+
+    for name, text in mtx_cases().items():
+        src = os.path.join(HERE, name + ".mtx")
+        with open(src, "w") as f:
+            f.write(text)
+        sm = ref_suite.suite_matrix(src)
+        sm.coo2csr(1)  # writes <case>_csr.mtx beside the source
+        lists = sm.colInd_list_array()
+        for V in (8, 16):
+            c = ref.CVSE(sm.M, sm.K, sm.nnz, lists, V)
+            c.CVSE_out(os.path.join(HERE, "%s.mtx.v%d.smtx" % (name, V)))
+            print(name, V, "M", sm.M, "K", sm.K, "nnz", sm.nnz, "num_vec", c.num_vec)
+
+
 if __name__ == "__main__":
-    main()
+    if "--suitesparse" in sys.argv:
+        main_suitesparse()
+    else:
+        main()

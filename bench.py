@@ -434,8 +434,8 @@ def run_cfg4(L, torch, synth, sspmm_amd, O, st, wu):
 
 def run_cfg5_layer(L, torch, synth, st, wu):
     """One BERT-base shaped encoder layer (hidden 768, 12 heads, FFN 3072, 8 x 512 tokens) with six vector-sparse
-    weights (V=16, 90 %) and dense attention in torch; the same layer with dense fp16 matmuls on the densified
-    weights beside it."""
+    weights (V=16, 90 %; query, key and value stacked into one product) and dense attention in torch; the same layer
+    with dense fp16 matmuls on the densified weights beside it, eager and replayed from a HIP graph."""
     from sspmm_amd.layers import SparseEncoderLayer, SparseLinear
     hid, heads, ffn, V5, bsz, seq = 768, 12, 3072, 16, 8, 512
 
@@ -448,19 +448,46 @@ def run_cfg5_layer(L, torch, synth, st, wu):
                                mk(ffn, hid, 55), mk(hid, ffn, 56)).cuda().half()
     x5 = (torch.randn(hid, bsz * seq, device="cuda") * 1.0).half()
     dense_w = {n: getattr(layer, n).dense_weight() for n in ("q", "k", "v", "o", "ffn1", "ffn2")}
+    dense_w["qkv"] = torch.cat([dense_w["q"], dense_w["k"], dense_w["v"]])  # the dense layer fuses the three as well
+    def graphed(fn):
+        """fn recorded into a HIP graph once; returns the replay (the host's per-launch cost is out of the picture)."""
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            fn()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            fn()
+        return g.replay
+
+    dense_lin = lambda n, lin, t: dense_w[n] @ t  # noqa: E731
     with torch.no_grad():
         y_sp = layer(x5, bsz, seq)
-        y_de = layer(x5, bsz, seq, linear=lambda n, lin, t: dense_w[n] @ t)
+        y_de = layer(x5, bsz, seq, linear=dense_lin)
         sp_ms = time_launches(lambda: layer(x5, bsz, seq), st, wu)
-        de_ms = time_launches(lambda: layer(x5, bsz, seq, linear=lambda n, lin, t: dense_w[n] @ t), st, wu)
+        de_ms = time_launches(lambda: layer(x5, bsz, seq, linear=dense_lin), st, wu)
+        sp_g = time_launches(graphed(lambda: layer(x5, bsz, seq)), st, wu)
+        de_g = time_launches(graphed(lambda: layer(x5, bsz, seq, linear=dense_lin)), st, wu)
         per = {}
-        for n in ("q", "o", "ffn1", "ffn2"):
-            lin = getattr(layer, n)
-            xin = torch.randn(lin.in_features, bsz * seq, device="cuda").half()
-            per[n] = {"sparse_ms": time_launches(lambda: lin(xin), st, wu),
-                      "dense_ms": time_launches(lambda: dense_w[n] @ xin, st, wu)}
-        per.update(layer.time_parts(x5, bsz, seq, lambda f: time_launches(f, st, wu)) if hasattr(layer, "time_parts") else {})
+        xin = {768: torch.randn(hid, bsz * seq, device="cuda").half(), 3072: torch.randn(ffn, bsz * seq, device="cuda").half()}
+        sparse_sum = dense_sum = 0.0
+        for n, lin in (("qkv", layer.qkv), ("o", layer.o), ("ffn1", layer.ffn1), ("ffn2", layer.ffn2)):
+            xi = xin[lin.in_features]
+            dw = dense_w[n]
+            dfn = lambda: dw @ xi  # noqa: E731
+            # (twenty calls per graph: a graph of one kernel is bound by the cost of launching a graph)
+            per[n] = {"sparse_ms_in_a_graph": graph_time(lambda s_: lin(xi)), "dense_ms_in_a_graph": graph_time(lambda s_: dfn())}
+            sparse_sum += per[n]["sparse_ms_in_a_graph"]
+            dense_sum += per[n]["dense_ms_in_a_graph"]
+        per["qkv"]["three_separate_dense_products_ms_in_a_graph"] = graph_time(
+            lambda s_: (dense_w["q"] @ xin[768], dense_w["k"] @ xin[768], dense_w["v"] @ xin[768]))
     return {"sparse_layer_ms": sp_ms, "dense_layer_ms": de_ms, "speedup_vs_dense_layer": de_ms / sp_ms,
+            "sparse_layer_ms_in_a_graph": sp_g, "dense_layer_ms_in_a_graph": de_g, "speedup_vs_dense_layer_in_a_graph": de_g / sp_g,
+            "products_sparse_ms_in_a_graph": sparse_sum, "products_dense_ms_in_a_graph": dense_sum,
+            "rest_of_the_layer_ms_in_a_graph": {"sparse_layer": sp_g - sparse_sum, "dense_layer": de_g - dense_sum},
+            "note": "both layers run the same glue around their four products: one relayout copy of q, k, v for torch's "
+                    "attention and one back, torch's GELU, and the residual add + LayerNorm in one kernel of this "
+                    "library on the feature-major activations; the products are one fused q/k/v, o, ffn1, ffn2",
             "max_rel_diff_vs_dense_layer": float((y_sp.float() - y_de.float()).abs().max() / y_de.float().abs().max()),
             "projections": per}
 

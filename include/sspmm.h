@@ -261,6 +261,18 @@ int svc_permute_csr(int M, const int32_t *perm, const int32_t *row_ptr, const in
                     void *workspace, size_t workspace_bytes, void *hip_stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Residual add + LayerNorm on feature-major activations [H features, T tokens] (the layout the
+ * SpMM takes and returns), fp16 in and out, statistics in fp32:
+ *   out[h, t] = (s[h, t] - mean_t) / sqrt(var_t + eps) * gamma[h] + beta[h],  s = fp16(x + a).
+ * No counterpart among the reference's kernels: its encoder block (reference
+ * end2end/sspmm_e2e/end_to_end.py:58-75) calls torch's LayerNorm on token-major tensors; on the
+ * SpMM's layout that costs two transposed copies per call.  a, gamma, beta may be NULL (no
+ * residual, scale one, shift zero).  T a multiple of 4, H up to 1024, 8-byte aligned pointers.
+ * ---------------------------------------------------------------------------------------- */
+int sspmm_add_layernorm_f16(int H, int T, const sspmm_half_t *x, const sspmm_half_t *a, const sspmm_half_t *gamma,
+                            const sspmm_half_t *beta, float eps, sspmm_half_t *out, void *hip_stream);
+
+/* ------------------------------------------------------------------------------------------
  * Coordinate list -> CSR, the step between a Matrix Market file and the RowMerge in the
  * reference's SuiteSparse path: `csr = self.coo.tocsr()` in suite_matrix.coo2csr, reference
  * RowMerge/suit_sparse_matrix.py:109-111 (scipy: rows ascending, inside a row the columns

@@ -5,6 +5,7 @@
 #include "../../include/sspmm.h"
 #include "attention_kernels.h"
 #include "coo_kernels.h"
+#include "layer_kernels.h"
 #include "plan.h"
 #include "reorder_kernels.h"
 #include "spmm_kernels.h"
@@ -324,6 +325,16 @@ int svc_permute_csr(int M, const int32_t *perm, const int32_t *row_ptr, const in
   return (int)sspmm::launch_permute_csr(M, perm, row_ptr, col_ind, csr_val, out_row_ptr, out_col,
                                         csr_val ? out_val : nullptr, workspace, workspace_bytes,
                                         static_cast<hipStream_t>(hip_stream));
+}
+
+int sspmm_add_layernorm_f16(int H, int T, const sspmm_half_t *x, const sspmm_half_t *a, const sspmm_half_t *gamma,
+                            const sspmm_half_t *beta, float eps, sspmm_half_t *out, void *hip_stream) {
+  if (H < 0 || T < 0 || T % 4 != 0 || H > 1024) return kInvalid;
+  if (H == 0 || T == 0) return 0;
+  if (!x || !out) return kInvalid;
+  if (reinterpret_cast<uintptr_t>(x) % 8 || reinterpret_cast<uintptr_t>(a) % 8 || reinterpret_cast<uintptr_t>(out) % 8)
+    return kInvalid;
+  return (int)sspmm::launch_add_layernorm(H, T, x, a, gamma, beta, eps, out, static_cast<hipStream_t>(hip_stream));
 }
 
 size_t svc_coo_workspace_bytes(int64_t n) { return sspmm::coo_workspace_bytes(n); }

@@ -1,0 +1,20 @@
+// Launch interface of the model-side glue kernels (feature-major residual add + LayerNorm).
+#ifndef SSPMM_AMD_LAYER_KERNELS_H
+#define SSPMM_AMD_LAYER_KERNELS_H
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace sspmm {
+
+// LDS bytes a workgroup needs for H features (the caller checks it against the 160 KB of a CU).
+size_t add_layernorm_lds_bytes(int H);
+
+// out[H, T] = LayerNorm over the H features of every token of fp16(x + a) (a may be null), fp16 in and out.
+// T must be a multiple of 4 and the pointers 8-byte aligned.
+hipError_t launch_add_layernorm(int H, int T, const uint16_t *x, const uint16_t *a, const uint16_t *gamma,
+                                const uint16_t *beta, float eps, uint16_t *out, hipStream_t stream);
+
+}  // namespace sspmm
+#endif

@@ -47,6 +47,28 @@ class SparseLinear(torch.nn.Module):
         return cls(in_features, m_vec * vec_length, vec_length, row_offsets, column_indices, values, bias, **kw)
 
     @classmethod
+    def concat(cls, layers):
+        """One layer whose output is the outputs of `layers` stacked along the feature axis: their patterns
+        concatenated along M.  Three projections of the same input (query, key, value) become one SpMM that reads
+        the input once."""
+        first = layers[0]
+        if any(l.in_features != first.in_features or l.vec_length != first.vec_length or l.out_dtype != first.out_dtype
+               for l in layers):
+            raise ValueError("the layers must share in_features, vec_length and output type")
+        offsets, base = [first.row_offsets[:1]], 0
+        for l in layers:
+            offsets.append(l.row_offsets[1:] + base)
+            base += int(l.column_indices.numel())
+        biases = [l.bias for l in layers]
+        bias = None
+        if any(b is not None for b in biases):
+            bias = torch.cat([b if b is not None else torch.zeros(l.out_features, dtype=torch.float16, device=first.values.device)
+                              for b, l in zip(biases, layers)])
+        return cls(first.in_features, sum(l.out_features for l in layers), first.vec_length,
+                   torch.cat(offsets).to(torch.int32).contiguous(), torch.cat([l.column_indices for l in layers]).contiguous(),
+                   torch.cat([l.values for l in layers]).contiguous(), bias, out_dtype=first.out_dtype)
+
+    @classmethod
     def from_dense(cls, weight, vec_length, bias=None, order="sorted", **kw):
         """weight: [out, in] fp16 GPU tensor; its non-zeros are merged V rows at a time (SVC on the GPU)."""
         if weight.dtype != torch.float16 or not weight.is_cuda:
@@ -59,11 +81,21 @@ class SparseLinear(torch.nn.Module):
         r = svc(row_ptr, col_ind, weight[mask].contiguous(), out_features, in_features, vec_length, order=order)
         return cls(in_features, out_features, vec_length, r.vec_row_ptr, r.vec_col, r.vec_val, bias, **kw)
 
+    def make_plan(self, max_tokens):
+        """Builds the pattern's plan (sspmm_amd.Plan) for inputs of up to max_tokens columns; later calls of the
+        layer use it.  Worth it for weights whose merged rows are uneven (unstructured pruning through RowMerge)."""
+        from .plan import Plan
+        self.plan = Plan(self.row_offsets, self.vec_length, self.in_features, max_N=max_tokens)
+        return self.plan
+
     def forward(self, x):
         if x.dim() != 2 or x.size(0) != self.in_features:
             raise ValueError("x must be [in_features, tokens] = [%d, *], got %s" % (self.in_features, tuple(x.shape)))
+        plan = getattr(self, "plan", None)
+        if plan is not None and x.size(1) > plan.max_N:
+            plan = None
         y = spmm(None, self.row_offsets, self.column_indices, self.values, x.contiguous(), self.vec_length,
-                 out_dtype=self.out_dtype)
+                 out_dtype=self.out_dtype, plan=plan)
         if self.bias is not None:
             y = y + self.bias[:, None].to(y.dtype)
         return y
@@ -80,6 +112,27 @@ class SparseLinear(torch.nn.Module):
         return torch.from_numpy(W).to(self.values.device)
 
 
+def add_layernorm(x, a, ln):
+    """LayerNorm over the features of the feature-major sum x + a ([features, tokens] fp16; a may be None) with the
+    weights of `ln` (a torch.nn.LayerNorm over `features`).  One HIP kernel (sspmm_add_layernorm_f16 of the C ABI)
+    where its shape limits hold, torch on transposed copies otherwise."""
+    from . import _lib
+    H, T = x.shape
+    ok = (x.dtype == torch.float16 and x.is_cuda and x.is_contiguous() and T % 4 == 0 and H <= 1024 and
+          (a is None or (a.dtype == torch.float16 and a.is_contiguous() and a.shape == x.shape)) and
+          ln.weight is not None and ln.weight.dtype == torch.float16 and tuple(ln.normalized_shape) == (H,))
+    if not ok:
+        s = x if a is None else x + a
+        return ln(s.t()).t().contiguous()
+    out = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        rc = _lib.lib().sspmm_add_layernorm_f16(H, T, x.data_ptr(), 0 if a is None else a.data_ptr(), ln.weight.data_ptr(),
+                                                0 if ln.bias is None else ln.bias.data_ptr(), float(ln.eps), out.data_ptr(),
+                                                torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc, "sspmm_add_layernorm_f16")
+    return out
+
+
 class SparseEncoderLayer(torch.nn.Module):
     """Post-LayerNorm transformer encoder layer with vector-sparse Q, K, V, output and FFN weights
     and dense attention, on feature-major activations x[hidden, batch * seq]."""
@@ -88,23 +141,25 @@ class SparseEncoderLayer(torch.nn.Module):
         super().__init__()
         self.hidden, self.heads, self.ffn = hidden, heads, ffn
         self.q, self.k, self.v, self.o, self.ffn1, self.ffn2 = q, k, v, o, ffn1, ffn2
+        # query, key and value projections as one SpMM over the three patterns stacked along M
+        self.qkv = SparseLinear.concat([q, k, v])
         self.ln1 = torch.nn.LayerNorm(hidden)
         self.ln2 = torch.nn.LayerNorm(hidden)
 
-    def _attention(self, q, k, v, batch, seq):
+    def _attention(self, qkv, batch, seq):
+        """qkv: [3 * hidden, batch*seq] feature-major.  One copy brings the three projections into the
+        [batch, heads, seq, head size] layout torch's attention wants contiguous (on strided views of the
+        feature-major activations it runs ten times slower), one copy brings the context back."""
         h, d = self.heads, self.hidden // self.heads
-        # [hidden, batch*seq] -> [batch, heads, seq, d]
-        def split(t):
-            return t.view(h, d, batch, seq).permute(2, 0, 3, 1)
-        ctx = torch.nn.functional.scaled_dot_product_attention(split(q), split(k), split(v), scale=1.0 / math.sqrt(d))
+        c = qkv.view(3, h, d, batch, seq).permute(0, 3, 1, 4, 2).contiguous()
+        ctx = torch.nn.functional.scaled_dot_product_attention(c[0], c[1], c[2], scale=1.0 / math.sqrt(d))
         return ctx.permute(1, 3, 0, 2).reshape(self.hidden, batch * seq)
 
     def forward(self, x, batch, seq, linear=None):
-        """x: [hidden, batch*seq] fp16.  `linear(name, layer, x)` may replace how a projection is
-        evaluated (the benchmark passes a dense matmul there to time the same layer without sparsity)."""
+        """x: [hidden, batch*seq] fp16.  `linear(name, layer, x)` may replace how a projection ("qkv", "o", "ffn1",
+        "ffn2") is evaluated (the benchmark passes a dense matmul there to time the same layer without sparsity)."""
         f = linear or (lambda name, layer, t: layer(t))
-        q, k, v = f("q", self.q, x), f("k", self.k, x), f("v", self.v, x)
-        a = f("o", self.o, self._attention(q, k, v, batch, seq))
-        x = self.ln1((x + a).t()).t().contiguous()
+        a = f("o", self.o, self._attention(f("qkv", self.qkv, x), batch, seq))
+        x = add_layernorm(x, a, self.ln1)
         y = f("ffn2", self.ffn2, torch.nn.functional.gelu(f("ffn1", self.ffn1, x)))
-        return self.ln2((x + y).t()).t().contiguous()
+        return add_layernorm(x, y, self.ln2)

@@ -48,9 +48,33 @@ def test_encoder_layer_matches_the_same_layer_with_dense_products(built_library)
     layer = SparseEncoderLayer(hidden, heads, ffn, mk(hidden, hidden, 1), mk(hidden, hidden, 2), mk(hidden, hidden, 3),
                                mk(hidden, hidden, 4), mk(ffn, hidden, 5), mk(hidden, ffn, 6)).cuda().half()
     x = torch.randn(hidden, batch * seq, device="cuda", generator=torch.Generator("cuda").manual_seed(3)).half()
-    dense = {n: getattr(layer, n).dense_weight() for n in ("q", "k", "v", "o", "ffn1", "ffn2")}
+    dense = {n: getattr(layer, n).dense_weight() for n in ("qkv", "o", "ffn1", "ffn2")}
+    assert torch.equal(dense["qkv"], torch.cat([layer.q.dense_weight(), layer.k.dense_weight(), layer.v.dense_weight()]))
     with torch.no_grad():
         got = layer(x, batch, seq)
         want = layer(x, batch, seq, linear=lambda name, lin, t: (dense[name].float() @ t.float()).half())
     assert got.shape == (hidden, batch * seq)
     assert max_rel_err(got.float().cpu().numpy(), want.float().cpu().numpy()) <= 1e-2
+
+
+@pytest.mark.parametrize("H,T", [(768, 4096), (256, 128), (100, 36), (1024, 68), (1, 4)])
+@pytest.mark.parametrize("residual", [True, False])
+def test_feature_major_add_layernorm_matches_torch(built_library, H, T, residual):
+    """The fused kernel against torch's LayerNorm on the transposed sum: same fp16 sum, statistics in fp32."""
+    from sspmm_amd.layers import add_layernorm
+    g = torch.Generator("cuda").manual_seed(H + T)
+    x = (torch.randn(H, T, device="cuda", generator=g) * 2 + 0.5).half()
+    a = torch.randn(H, T, device="cuda", generator=g).half() if residual else None
+    ln = torch.nn.LayerNorm(H).cuda().half()
+    with torch.no_grad():
+        ln.weight.copy_(torch.randn(H, device="cuda", generator=g))
+        ln.bias.copy_(torch.randn(H, device="cuda", generator=g))
+        got = add_layernorm(x, a, ln)
+        s = x if a is None else x + a
+        want = torch.nn.functional.layer_norm(s.t().float(), (H,), ln.weight.float(), ln.bias.float(), ln.eps).t()
+    assert got.shape == (H, T) and got.dtype == torch.float16
+    assert (got.float() - want).abs().max().item() <= 4e-3 * max(1.0, want.abs().max().item())
+    # shapes outside the kernel's limits take torch and agree too
+    if T % 4 == 0 and H > 1:
+        odd = add_layernorm(x[:, :T - 1].contiguous(), None if a is None else a[:, :T - 1].contiguous(), ln)
+        assert (odd.float() - want[:, :T - 1]).abs().max().item() <= 4e-3 * max(1.0, want.abs().max().item())

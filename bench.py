@@ -33,8 +33,22 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch from hardware counters (FETCH_SIZE and WRITE_SIZE in separate runs, each scaled by its
 # reading for a plain 256 MiB device copy), keyed by kernel and workload; `source` names the summary it comes from.
 MEASURED_TRAFFIC = {
-    "headline_batch128": {"kernel": "spmm_slab_kernel<8,float,*,4>", "bytes": 66.1e6 + 268.4e6,
+    # HBM bytes per launch from rocprofv3 counters (FETCH_SIZE and WRITE_SIZE, each scaled by its reading of a plain
+    # 256 MiB copy), keyed by benchmark entry; measured in runs of their own, not in this one.
+    "headline_batch128": {"kernel": "spmm_slab_kernel<8,float,*,4>", "bytes": 66.2e6 + 268.4e6, "alg_bytes": 328781828,
                           "source": "profiles/spmm_slab_v8_f32_cfg2_batch128_hbm_traffic.txt"},
+    "cfg3_1024x2304_v16_s0.8_n3136": {"kernel": "spmm_gather_kernel<16,float,8>", "bytes": 26.9e6 + 12.8e6,
+                                      "alg_bytes": 28358148, "l2_request_bytes": 222.1e6,
+                                      "source": "profiles/spmm_gather_v16_f32_cfg3_1024x2304_s0.8_n3136_counters.txt"},
+    "cfg4_spmm_on_svc_output_with_plan": {"kernel": "spmm_balanced_kernel<8,float,false>", "bytes": 48.2e6 + 23.2e6,
+                                          "alg_bytes": 30393520, "l2_request_bytes": 215.0e6,
+                                          "source": "profiles/spmm_balanced_v8_f32_cfg4_zipf_n256_counters.txt"},
+    "cfg4_spmm_on_svc_output": {"kernel": "spmm_gather_split_kernel<8,float>", "bytes": 51.1e6 + 16.8e6,
+                                "alg_bytes": 30393520, "l2_request_bytes": 186.5e6,
+                                "source": "profiles/spmm_balanced_v8_f32_cfg4_zipf_n256_counters.txt"},
+    "svc_cfg4_zipf_16384_v8": {"kernel": "svc_count_distinct + svc_scan_classify + the four svc_merge kernels",
+                               "bytes": (1.717 + 0.012 + 1.947 + 0.733 + 0.023 + 0.042) * 1e6 + (0.039 + 0.010 + 2.879 + 0.506) * 1e6,
+                               "alg_bytes": 6866100, "source": "profiles/svc_kernels_cfg4_zipf_v8_counters.txt"},
 }
 KERNEL_NAMES = {1: "spmm_generic_kernel", 2: "spmm_gather_kernel", 3: "spmm_slab_kernel<*,4>", 4: "spmm_gather_split_kernel",
                 5: "spmm_slab_kernel<*,2>", 6: "spmm_stage_kernel", 7: "spmm_balanced_kernel"}
@@ -611,6 +625,13 @@ def main():
     L.sspmm_select_kernel({"auto": 0, "generic": 1, "gather": 2, "slab": 3}[args.kernel])
     env = {"L": L, "torch": torch, "synth": synth, "sspmm_amd": sspmm_amd, "O": None, "st": args.steps, "wu": args.warmup,
            "batch": args.batch}
+    if args.calibrate_copy:
+        src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     only = [ATTENTION] if args.attention_only else [n for n in args.only.split(",") if n]
     if only:
         from oracle import oracle as O
@@ -621,14 +642,6 @@ def main():
             out.update(run_extra(n, env))
         print(json.dumps(out))
         return
-
-    if args.calibrate_copy:
-        src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device="cuda")
-        dst = torch.empty_like(src)
-        for _ in range(5):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
 
     M, K, V, sparsity, N = 2048, 512, 8, 0.9, 256
     series, handles = [], []

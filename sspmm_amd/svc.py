@@ -15,13 +15,19 @@ SvcResult = collections.namedtuple("SvcResult", ["vec_row_ptr", "vec_col", "vec_
 _ORDERS = {"cpython": 0, "sorted": 1}
 
 
-def svc(row_ptr, col_ind, csr_val, M, K, V, order="cpython"):
+def svc(row_ptr, col_ind, csr_val, M, K, V, order="cpython", exact_size=True):
     """Merge every V consecutive rows of a CSR matrix into column vectors.
 
     row_ptr[M+1], col_ind[nnz]: int32 GPU tensors; csr_val: fp16 GPU tensor or None.
     order="cpython" gives exactly the column order the reference's RowMerge writes;
     order="sorted" gives ascending columns.
     Returns SvcResult(vec_row_ptr[int32 m_vec+1], vec_col[int32 nvec], vec_val[fp16 nvec*V] or None, nvec).
+
+    exact_size=True reads nvec back from the device between the two phases (the call's one synchronisation) and
+    returns arrays of exactly nvec vectors.  exact_size=False sizes them for the bound nvec <= nnz instead: the call
+    then never waits for the device (both phases are queued on the current stream), num_vec is None, the vectors
+    are the first vec_row_ptr[-1] entries of vec_col / vec_val and what lies behind them is unspecified.  The SpMM
+    operators take such arrays as they are: they read the extent from vec_row_ptr on the device.
     """
     if order not in _ORDERS:
         raise ValueError("order must be 'cpython' or 'sorted'")
@@ -46,9 +52,10 @@ def svc(row_ptr, col_ind, csr_val, M, K, V, order="cpython"):
                              None if csr_val is None else torch.empty(0, dtype=torch.float16, device=dev), 0)
         _lib.check(L.svc_count(M, K, V, row_ptr.data_ptr(), col_ind.data_ptr(), nnz, _ORDERS[order],
                                vec_row_ptr.data_ptr(), ws.data_ptr(), stream), "svc_count")
-        nvec = int(vec_row_ptr[-1].item())  # the one host read-back: sizes the outputs
-        vec_col = torch.empty(nvec, dtype=torch.int32, device=dev)
-        vec_val = None if csr_val is None else torch.empty(nvec * V, dtype=torch.float16, device=dev)
+        nvec = int(vec_row_ptr[-1].item()) if exact_size else None  # the one host read-back: sizes the outputs
+        cap = nvec if exact_size else nnz
+        vec_col = torch.empty(cap, dtype=torch.int32, device=dev)
+        vec_val = None if csr_val is None else torch.empty(cap * V, dtype=torch.float16, device=dev)
         _lib.check(L.svc_fill(M, K, V, row_ptr.data_ptr(), col_ind.data_ptr(),
                               0 if csr_val is None else csr_val.data_ptr(), nnz, _ORDERS[order],
                               vec_row_ptr.data_ptr(), ws.data_ptr(), vec_col.data_ptr(),

@@ -8,7 +8,7 @@ import pytest
 import torch
 
 import sspmm_amd
-from sspmm_amd import formats, synth
+from sspmm_amd import _lib, formats, synth
 from gpu_util import dev
 
 pytestmark = pytest.mark.gpu
@@ -262,6 +262,31 @@ def test_svc_then_spmm_equals_csr_matmul(oracle, built_library):
         A[i, csr.col_ind[csr.row_ptr[i]:csr.row_ptr[i + 1]]] = csr.values[csr.row_ptr[i]:csr.row_ptr[i + 1]]
     want = A @ B.astype(np.float64)
     assert np.abs(out.cpu().numpy() - want).max() <= 2e-5 * np.abs(want).max()
+
+
+@pytest.mark.parametrize("order", ["cpython", "sorted"])
+def test_outputs_sized_by_the_bound_need_no_read_back(oracle, built_library, order):
+    """exact_size=False: arrays of nnz vectors, the result in their first nvec entries, and the
+    SpMM takes them as they are (every kernel reads the extent from the row offsets)."""
+    rng = np.random.default_rng(21)
+    csr = _random_csr(rng, 256, 300, 40)
+    B = synth.dense_rhs(300, 64, seed=21)
+    args = (dev(csr.row_ptr), dev(csr.col_ind), dev(csr.values), csr.M, csr.K, 8)
+    exact = sspmm_amd.svc(*args, order=order)
+    loose = sspmm_amd.svc(*args, order=order, exact_size=False)
+    assert loose.num_vec is None and loose.vec_col.numel() == csr.col_ind.size
+    assert loose.vec_val.numel() == csr.col_ind.size * 8
+    n = exact.num_vec
+    assert torch.equal(loose.vec_row_ptr, exact.vec_row_ptr)
+    assert torch.equal(loose.vec_col[:n], exact.vec_col) and torch.equal(loose.vec_val[:n * 8], exact.vec_val)
+    want = sspmm_amd.spmm(None, exact.vec_row_ptr, exact.vec_col, exact.vec_val, dev(B), 8, out_dtype=torch.float32)
+    for force in (0, 1, 2, 6):
+        _lib.lib().sspmm_select_kernel(force)
+        try:
+            got = sspmm_amd.spmm(None, loose.vec_row_ptr, loose.vec_col, loose.vec_val, dev(B), 8, out_dtype=torch.float32)
+        finally:
+            _lib.lib().sspmm_select_kernel(0)
+        assert torch.allclose(got, want, rtol=0, atol=2e-5 * float(want.abs().max())), force
 
 
 def test_wide_matrices_and_giant_groups_take_the_64_bit_tables(oracle, built_library):

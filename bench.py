@@ -499,14 +499,50 @@ def run_cfg5_layer(L, torch, synth, st, wu):
             dense_sum += per[n]["dense_ms_in_a_graph"]
         per["qkv"]["three_separate_dense_products_ms_in_a_graph"] = graph_time(
             lambda s_: (dense_w["q"] @ xin[768], dense_w["k"] @ xin[768], dense_w["v"] @ xin[768]))
+        # the attention step alone: this library's kernel on the feature-major projections against torch's attention
+        # between the two relayout copies it needs on them
+        import sspmm_amd.layers as layers_mod
+        qkv5 = torch.randn(3 * hid, bsz * seq, device="cuda").half()
+        att_kernel = graph_time(lambda s_: layer._attention(qkv5, bsz, seq))
+        kernel_fn = layers_mod.attention_fm
+        layers_mod.attention_fm = lambda *a, **kw: None
+        try:
+            att_torch = graph_time(lambda s_: layer._attention(qkv5, bsz, seq))
+            sp_torch_att = time_launches(graphed(lambda: layer(x5, bsz, seq)), st, wu)
+            de_torch_att = time_launches(graphed(lambda: layer(x5, bsz, seq, linear=dense_lin)), st, wu)
+        finally:
+            layers_mod.attention_fm = kernel_fn
+        att_bytes = 4 * 2 * hid * bsz * seq  # q, k, v read, context written
+        # the layer as a torch user writes it: token-major activations, dense weights, torch's linear / attention /
+        # LayerNorm / GELU (no layout of this library anywhere)
+        xt = x5.t().contiguous()
+        wt = {n: dense_w[n] for n in ("qkv", "o", "ffn1", "ffn2")}
+        F = torch.nn.functional
+
+        def torch_layer():
+            q_, k_, v_ = (t.view(bsz, seq, heads, hid // heads).transpose(1, 2) for t in F.linear(xt, wt["qkv"]).chunk(3, dim=-1))
+            c = F.scaled_dot_product_attention(q_, k_, v_).transpose(1, 2).reshape(bsz * seq, hid)
+            h1 = layer.ln1(xt + F.linear(c, wt["o"]))
+            return layer.ln2(h1 + F.linear(F.gelu(F.linear(h1, wt["ffn1"])), wt["ffn2"]))
+
+        y_t = torch_layer()
+        torch_ms = time_launches(graphed(torch_layer), st, wu)
     return {"sparse_layer_ms": sp_ms, "dense_layer_ms": de_ms, "speedup_vs_dense_layer": de_ms / sp_ms,
             "sparse_layer_ms_in_a_graph": sp_g, "dense_layer_ms_in_a_graph": de_g, "speedup_vs_dense_layer_in_a_graph": de_g / sp_g,
             "products_sparse_ms_in_a_graph": sparse_sum, "products_dense_ms_in_a_graph": dense_sum,
             "rest_of_the_layer_ms_in_a_graph": {"sparse_layer": sp_g - sparse_sum, "dense_layer": de_g - dense_sum},
-            "note": "both layers run the same glue around their four products: one relayout copy of q, k, v for torch's "
-                    "attention and one back, torch's GELU, and the residual add + LayerNorm in one kernel of this "
-                    "library on the feature-major activations; the products are one fused q/k/v, o, ffn1, ffn2",
+            "attention_ms_in_a_graph": {"feature_major_kernel": att_kernel, "torch_between_two_relayout_copies": att_torch,
+                                        "kernel_alg_bytes": att_bytes, "kernel_hbm_frac": att_bytes / att_kernel / 1e6 / HBM_PEAK_GBPS},
+            "with_torch_attention_ms_in_a_graph": {"sparse_layer": sp_torch_att, "dense_layer": de_torch_att,
+                                                   "speedup": de_torch_att / sp_torch_att},
+            "torch_token_major_dense_layer_ms_in_a_graph": torch_ms,
+            "speedup_vs_torch_token_major_dense_layer_in_a_graph": torch_ms / sp_g,
+            "note": "both layers run the same glue around their four products: this library's attention kernel on the "
+                    "feature-major projections, torch's GELU, and the residual add + LayerNorm in one kernel of this "
+                    "library; the products are one fused q/k/v, o, ffn1, ffn2.  torch_token_major_dense_layer is the "
+                    "same arithmetic written with torch alone on token-major activations",
             "max_rel_diff_vs_dense_layer": float((y_sp.float() - y_de.float()).abs().max() / y_de.float().abs().max()),
+            "max_rel_diff_vs_torch_token_major_layer": float((y_sp.float() - y_t.t().float()).abs().max() / y_t.float().abs().max()),
             "projections": per}
 
 

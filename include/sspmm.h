@@ -273,6 +273,21 @@ int sspmm_add_layernorm_f16(int H, int T, const sspmm_half_t *x, const sspmm_hal
                             const sspmm_half_t *beta, float eps, sspmm_half_t *out, void *hip_stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Dense attention on feature-major activations: out = softmax(Q^T K * scale) V per (batch element,
+ * head), the dense attention of the reference's comparison block (reference
+ * end2end/sspmm_e2e/end_to_end.py:84-97, attention.py), which runs in torch on token-major tensors.
+ * The SpMM leaves q, k, v as [features, tokens]; this entry point reads them in that layout and
+ * writes the context in it, which saves the transposed copies either side of a token-major attention.
+ *   q, k, v   fp16 [heads * head_dim, batch * seq]: feature f of token t at f * ld + t, token
+ *             t = b * seq + s (they may be three row ranges of one fused projection)
+ *   out       fp16, same layout with ld_out
+ * Supported: head_dim = 64, seq a multiple of 64 up to 16384, ld and ld_out multiples of 8 and at
+ * least batch * seq, 16-byte aligned pointers; anything else returns hipErrorInvalidValue.
+ * ---------------------------------------------------------------------------------------- */
+int sspmm_attention_fm_f16(int batch, int heads, int seq, int head_dim, const sspmm_half_t *q, const sspmm_half_t *k,
+                           const sspmm_half_t *v, int64_t ld, sspmm_half_t *out, int64_t ld_out, float scale, void *hip_stream);
+
+/* ------------------------------------------------------------------------------------------
  * Coordinate list -> CSR, the step between a Matrix Market file and the RowMerge in the
  * reference's SuiteSparse path: `csr = self.coo.tocsr()` in suite_matrix.coo2csr, reference
  * RowMerge/suit_sparse_matrix.py:109-111 (scipy: rows ascending, inside a row the columns

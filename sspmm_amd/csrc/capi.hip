@@ -337,6 +337,15 @@ int sspmm_add_layernorm_f16(int H, int T, const sspmm_half_t *x, const sspmm_hal
   return (int)sspmm::launch_add_layernorm(H, T, x, a, gamma, beta, eps, out, static_cast<hipStream_t>(hip_stream));
 }
 
+int sspmm_attention_fm_f16(int batch, int heads, int seq, int head_dim, const sspmm_half_t *q, const sspmm_half_t *k,
+                           const sspmm_half_t *v, int64_t ld, sspmm_half_t *out, int64_t ld_out, float scale, void *hip_stream) {
+  if (batch < 0 || heads < 0 || seq < 0 || head_dim <= 0) return kInvalid;
+  if (batch == 0 || heads == 0 || seq == 0) return 0;
+  if (!q || !k || !v || !out || ld < (int64_t)batch * seq || ld_out < (int64_t)batch * seq) return kInvalid;
+  if (!sspmm::attention_fm_applies(batch, heads, seq, head_dim, q, k, v, ld, out, ld_out)) return kInvalid;
+  return (int)sspmm::launch_attention_fm(batch, heads, seq, q, k, v, ld, out, ld_out, scale, static_cast<hipStream_t>(hip_stream));
+}
+
 size_t svc_coo_workspace_bytes(int64_t n) { return sspmm::coo_workspace_bytes(n); }
 
 int svc_coo_to_csr(int M, int K, int64_t n, const int32_t *coo_row, const int32_t *coo_col, int32_t *row_ptr,

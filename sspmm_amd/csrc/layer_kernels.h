@@ -16,5 +16,13 @@ size_t add_layernorm_lds_bytes(int H);
 hipError_t launch_add_layernorm(int H, int T, const uint16_t *x, const uint16_t *a, const uint16_t *gamma,
                                 const uint16_t *beta, float eps, uint16_t *out, hipStream_t stream);
 
+// Dense attention softmax(Q^T K * scale) V on feature-major activations: q, k, v are [heads * 64, batch * seq] with
+// `ld` elements between consecutive features, out likewise with ld_out; fp16, fp32 accumulation.  Applies to a head
+// size of 64, seq a multiple of 64 up to 16384, ld and ld_out multiples of 8 and 16-byte aligned pointers.
+bool attention_fm_applies(int batch, int heads, int seq, int head_dim, const void *q, const void *k, const void *v,
+                          long long ld, const void *out, long long ld_out);
+hipError_t launch_attention_fm(int batch, int heads, int seq, const uint16_t *q, const uint16_t *k, const uint16_t *v,
+                               long long ld, uint16_t *out, long long ld_out, float scale, hipStream_t stream);
+
 }  // namespace sspmm
 #endif

@@ -120,4 +120,225 @@ hipError_t launch_add_layernorm(int H, int T, const uint16_t *x, const uint16_t 
   return hipGetLastError();
 }
 
+// ------------------------------------------------------------------------------------------
+// Dense softmax(Q^T K / sqrt(d)) attention on feature-major activations (the dense attention of the
+// reference's comparison block, reference end2end/sspmm_e2e/end_to_end.py:84-97, which runs it in torch on
+// token-major tensors).  The SpMM that produces q, k, v leaves them as [features, tokens]; torch's attention
+// wants [batch, heads, tokens, head size] with the head size contiguous, which costs one transposed copy of all
+// three before it and one of the context behind it.  Here a workgroup of four waves owns 64 queries of one
+// (batch element, head): its 64 columns of Q go to LDS once, and the head's K and V pass through LDS in blocks of
+// 64 keys (64 features x 64 tokens each, as they lie in memory; two buffers, the next block's loads in flight in
+// registers while the current one is computed, one barrier per block), 45 KB of LDS in all, so three workgroups
+// share a CU.  Each wave computes for its 16 queries
+//     scores^T[key, query] = sum_d K[d, key] Q[d, query]          (MFMA; both operands by transpose reads)
+//     out[d, query]        = sum_key V[d, key] P[query, key]       (MFMA; V read directly, P from registers)
+// per block with the running maximum and sum of the usual one-pass softmax.  The scores come out of the first
+// product with a query per lane and four consecutive keys per accumulator, which is the second product's operand
+// layout once its contraction slots are numbered accordingly (slots 0-3 and 4-7 of lane group g = keys 4g .. 4g+3
+// of two neighbouring 16-key tiles; V is read with the same numbering), so the probabilities never leave the
+// registers.  The context goes back through LDS and is written feature-major in whole 128-byte lines.  Bound by
+// HBM in bytes (q, k, v read once, out written once: 8 * hidden * tokens bytes; a head's K and V are re-read by its
+// seq / 64 workgroups from L2), by the exponentials and the LDS reads in time.
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef uint32_t uintx2 __attribute__((ext_vector_type(2)));
+typedef uint32_t uintx4 __attribute__((ext_vector_type(4)));
+typedef short shortx4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) shortx4 lds_shortx4;
+
+static constexpr int kAttThreads = 256;
+static constexpr int kAttD = 64;          // head size
+static constexpr int kAttQueries = 64;    // per workgroup, 16 per wave
+static constexpr int kAttKeys = 64;       // per block of the softmax
+static constexpr uint32_t kAttPitch = 64 * 2 + 16;  // bytes; rows padded so that the rows a read touches spread over the banks
+static constexpr uint32_t kAttTile = kAttD * kAttPitch;
+static constexpr size_t kAttLds = 5 * (size_t)kAttTile;  // Q, two K blocks, two V blocks
+static constexpr int kAttMaxSeq = 16384;
+
+union AttOperand {
+  half8 h;
+  uint32_t u[4];
+};
+
+// Within 16 lanes, lane n receives element n of the four 32-byte runs addressed by lanes 0-3, 4-7, 8-11, 12-15.
+__device__ __forceinline__ uintx2 att_read_tr(const unsigned char *p) {
+  const shortx4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4 *)p);
+  return __builtin_bit_cast(uintx2, v);
+}
+
+__device__ __forceinline__ uint32_t att_pack(float lo, float hi) {
+  typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+  const half2v h = {(_Float16)lo, (_Float16)hi};
+  return __builtin_bit_cast(uint32_t, h);
+}
+
+struct AttentionArgs {
+  const _Float16 *q, *k, *v;
+  _Float16 *out;
+  long long ld, ld_out;  // elements between consecutive features
+  int S, heads;
+  float scale_log2e;
+};
+
+__global__ __launch_bounds__(kAttThreads, 3) void attention_fm_kernel(const AttentionArgs p) {
+  __shared__ __align__(16) unsigned char lds[kAttLds];
+  const int S = p.S, qblocks = S / kAttQueries, blocks = S / kAttKeys;
+  const int qb = blockIdx.x % qblocks, head = (blockIdx.x / qblocks) % p.heads, b = blockIdx.x / (qblocks * p.heads);
+  const int tid = threadIdx.x, lane = tid & 63, m = lane & 15, g = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  unsigned char *const q_tile = lds;
+  unsigned char *const k_tiles = lds + kAttTile;      // buffer i at k_tiles + i * kAttTile
+  unsigned char *const v_tiles = lds + 3 * kAttTile;
+  const long long tok0 = (long long)b * S;
+  const _Float16 *qg = p.q + (long long)(head * kAttD) * p.ld + tok0 + qb * kAttQueries;
+  const _Float16 *kg = p.k + (long long)(head * kAttD) * p.ld + tok0;
+  const _Float16 *vg = p.v + (long long)(head * kAttD) * p.ld + tok0;
+
+  // A 64 x 64 fp16 tile is 512 pieces of 16 bytes, two per thread: rows r0 and r0 + 32, piece pc.
+  const int r0 = tid >> 3, pc = tid & 7;
+  const long long g0 = (long long)r0 * p.ld + pc * 8, g1 = g0 + 32 * p.ld;
+  const uint32_t l0 = r0 * kAttPitch + pc * 16, l1 = l0 + 32 * kAttPitch;
+  uintx4 kk[2], vv[2];
+  kk[0] = *reinterpret_cast<const uintx4 *>(kg + g0);
+  kk[1] = *reinterpret_cast<const uintx4 *>(kg + g1);
+  vv[0] = *reinterpret_cast<const uintx4 *>(vg + g0);
+  vv[1] = *reinterpret_cast<const uintx4 *>(vg + g1);
+  *reinterpret_cast<uintx4 *>(q_tile + l0) = *reinterpret_cast<const uintx4 *>(qg + g0);
+  *reinterpret_cast<uintx4 *>(q_tile + l1) = *reinterpret_cast<const uintx4 *>(qg + g1);
+  *reinterpret_cast<uintx4 *>(k_tiles + l0) = kk[0];
+  *reinterpret_cast<uintx4 *>(k_tiles + l1) = kk[1];
+  *reinterpret_cast<uintx4 *>(v_tiles + l0) = vv[0];
+  *reinterpret_cast<uintx4 *>(v_tiles + l1) = vv[1];
+  __syncthreads();
+
+  // ---- the wave's 16 queries as the first product's second operand: lane (m, g) holds features 32u + 8g .. + 7 of query m
+  AttOperand qop[2];
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const unsigned char *a = q_tile + (32 * u + 8 * g + (m >> 2)) * kAttPitch + (16 * wave) * 2 + (m & 3) * 8;
+    const uintx2 lo = att_read_tr(a), hi = att_read_tr(a + 4 * kAttPitch);
+    qop[u].u[0] = lo[0]; qop[u].u[1] = lo[1]; qop[u].u[2] = hi[0]; qop[u].u[3] = hi[1];
+  }
+
+  const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+  floatx4 o[4] = {zero, zero, zero, zero};  // lane (m, g): features 16dt + 4g .. + 3 of query m
+  // of query m: the largest raw score so far, and this lane's share of the sum of 2^((score - max) * scale_log2e)
+  float run_max = -3.0e38f, run_sum = 0.f;
+  const float c = p.scale_log2e;  // > 0: the largest scaled score is the scaled largest score
+  const uint32_t k_rd = (8 * g + (m >> 2)) * kAttPitch + (m & 3) * 8;
+  const uint32_t v_rd = m * kAttPitch + (4 * g) * 2;
+  for (int kb = 0; kb < blocks; ++kb) {
+    const unsigned char *const k_tile = k_tiles + (kb & 1) * kAttTile;
+    const unsigned char *const v_tile = v_tiles + (kb & 1) * kAttTile;
+    const bool more = kb + 1 < blocks;  // uniform
+    if (more) {
+      const int off = (kb + 1) * kAttKeys;
+      kk[0] = *reinterpret_cast<const uintx4 *>(kg + g0 + off);
+      kk[1] = *reinterpret_cast<const uintx4 *>(kg + g1 + off);
+      vv[0] = *reinterpret_cast<const uintx4 *>(vg + g0 + off);
+      vv[1] = *reinterpret_cast<const uintx4 *>(vg + g1 + off);
+    }
+    floatx4 s[4] = {zero, zero, zero, zero};  // lane (m, g): keys 16kt + 4g .. + 3 of the block against query m
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const unsigned char *a = k_tile + k_rd + (32 * u) * kAttPitch + (16 * kt) * 2;
+        const uintx2 lo = att_read_tr(a), hi = att_read_tr(a + 4 * kAttPitch);
+        AttOperand kop;
+        kop.u[0] = lo[0]; kop.u[1] = lo[1]; kop.u[2] = hi[0]; kop.u[3] = hi[1];
+        s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kop.h, qop[u].h, s[kt], 0, 0, 0);
+      }
+    }
+    float mx = s[0][0];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[kt][r]);
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float new_max = fmaxf(run_max, mx);
+    const float alpha = __builtin_amdgcn_exp2f(fmaxf((run_max - new_max) * c, -126.0f));
+    run_max = new_max;
+    const float shift = -new_max * c;
+    float part = 0.f;
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        s[kt][r] = __builtin_amdgcn_exp2f(fmaf(s[kt][r], c, shift));
+        part += s[kt][r];
+      }
+    run_sum = run_sum * alpha + part;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) o[dt] *= alpha;
+    AttOperand pop[2];  // contraction slots 0-3 = keys 4g .. + 3 of tile 2t, slots 4-7 = the same keys of tile 2t + 1
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      pop[t].u[0] = att_pack(s[2 * t][0], s[2 * t][1]);
+      pop[t].u[1] = att_pack(s[2 * t][2], s[2 * t][3]);
+      pop[t].u[2] = att_pack(s[2 * t + 1][0], s[2 * t + 1][1]);
+      pop[t].u[3] = att_pack(s[2 * t + 1][2], s[2 * t + 1][3]);
+    }
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const unsigned char *a = v_tile + v_rd + (16 * dt) * kAttPitch + (32 * t) * 2;
+        const uintx2 lo = *reinterpret_cast<const uintx2 *>(a), hi = *reinterpret_cast<const uintx2 *>(a + 32);
+        AttOperand vop;
+        vop.u[0] = lo[0]; vop.u[1] = lo[1]; vop.u[2] = hi[0]; vop.u[3] = hi[1];
+        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vop.h, pop[t].h, o[dt], 0, 0, 0);
+      }
+    }
+    if (more) {  // the other buffer: every wave finished reading it before the barrier that ended the previous block
+      unsigned char *const kn = k_tiles + ((kb + 1) & 1) * kAttTile, *const vn = v_tiles + ((kb + 1) & 1) * kAttTile;
+      *reinterpret_cast<uintx4 *>(kn + l0) = kk[0];
+      *reinterpret_cast<uintx4 *>(kn + l1) = kk[1];
+      *reinterpret_cast<uintx4 *>(vn + l0) = vv[0];
+      *reinterpret_cast<uintx4 *>(vn + l1) = vv[1];
+    }
+    __syncthreads();
+  }
+  run_sum += __shfl_xor(run_sum, 16, 64);
+  run_sum += __shfl_xor(run_sum, 32, 64);
+  const float inv = 1.0f / run_sum;
+
+  // ---- the context through LDS (over the query tile: every wave read its queries before the first barrier of the
+  // loop) and out in whole lines
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      *reinterpret_cast<_Float16 *>(q_tile + (16 * dt + 4 * g + r) * kAttPitch + (16 * wave + m) * 2) = (_Float16)(o[dt][r] * inv);
+  __syncthreads();
+  _Float16 *og = p.out + (long long)(head * kAttD) * p.ld_out + tok0 + qb * kAttQueries;
+  *reinterpret_cast<uintx4 *>(og + (long long)r0 * p.ld_out + pc * 8) = *reinterpret_cast<const uintx4 *>(q_tile + l0);
+  *reinterpret_cast<uintx4 *>(og + (long long)(r0 + 32) * p.ld_out + pc * 8) = *reinterpret_cast<const uintx4 *>(q_tile + l1);
+}
+
+bool attention_fm_applies(int batch, int heads, int seq, int head_dim, const void *q, const void *k, const void *v,
+                          long long ld, const void *out, long long ld_out) {
+  const auto aligned = [](const void *x) { return (reinterpret_cast<uintptr_t>(x) & 15u) == 0; };
+  return batch > 0 && heads > 0 && head_dim == kAttD && seq >= kAttQueries && seq % kAttQueries == 0 && seq <= kAttMaxSeq &&
+         ld % 8 == 0 && ld_out % 8 == 0 && aligned(q) && aligned(k) && aligned(v) && aligned(out) &&
+         (long long)batch * heads * (seq / kAttQueries) <= 0x7fffffffLL;
+}
+
+hipError_t launch_attention_fm(int batch, int heads, int seq, const uint16_t *q, const uint16_t *k, const uint16_t *v,
+                               long long ld, uint16_t *out, long long ld_out, float scale, hipStream_t stream) {
+  AttentionArgs a;
+  a.q = reinterpret_cast<const _Float16 *>(q);
+  a.k = reinterpret_cast<const _Float16 *>(k);
+  a.v = reinterpret_cast<const _Float16 *>(v);
+  a.out = reinterpret_cast<_Float16 *>(out);
+  a.ld = ld;
+  a.ld_out = ld_out;
+  a.S = seq;
+  a.heads = heads;
+  a.scale_log2e = scale * 1.4426950408889634f;
+  const unsigned blocks = (unsigned)((long long)batch * heads * (seq / kAttQueries));
+  hipLaunchKernelGGL(attention_fm_kernel, dim3(blocks), dim3(kAttThreads), 0, stream, a);
+  return hipGetLastError();
+}
+
 }  // namespace sspmm

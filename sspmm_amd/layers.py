@@ -133,6 +133,28 @@ def add_layernorm(x, a, ln):
     return out
 
 
+def attention_fm(qkv, hidden, heads, batch, seq, scale=None):
+    """softmax(Q^T K * scale) V per (batch element, head) on the fused feature-major projections qkv
+    [3 * hidden, batch * seq] fp16 (rows 0 .. hidden-1 the queries, then keys, then values; token b * seq + s in
+    column b * seq + s); returns the context [hidden, batch * seq], or None where the kernel's shape limits do not
+    hold (the caller then takes another route)."""
+    from . import _lib
+    d = hidden // heads
+    T = batch * seq
+    if not (qkv.dtype == torch.float16 and qkv.is_cuda and qkv.is_contiguous() and tuple(qkv.shape) == (3 * hidden, T) and
+            d == 64 and hidden == heads * d and seq % 64 == 0 and 64 <= seq <= 16384 and T % 8 == 0):
+        return None
+    out = torch.empty(hidden, T, dtype=torch.float16, device=qkv.device)
+    esz = qkv.element_size()
+    with torch.cuda.device(qkv.device):
+        rc = _lib.lib().sspmm_attention_fm_f16(batch, heads, seq, d, qkv.data_ptr(), qkv.data_ptr() + hidden * T * esz,
+                                               qkv.data_ptr() + 2 * hidden * T * esz, T, out.data_ptr(), T,
+                                               float(1.0 / math.sqrt(d) if scale is None else scale),
+                                               torch.cuda.current_stream().cuda_stream)
+    _lib.check(rc, "sspmm_attention_fm_f16")
+    return out
+
+
 class SparseEncoderLayer(torch.nn.Module):
     """Post-LayerNorm transformer encoder layer with vector-sparse Q, K, V, output and FFN weights
     and dense attention, on feature-major activations x[hidden, batch * seq]."""
@@ -147,10 +169,15 @@ class SparseEncoderLayer(torch.nn.Module):
         self.ln2 = torch.nn.LayerNorm(hidden)
 
     def _attention(self, qkv, batch, seq):
-        """qkv: [3 * hidden, batch*seq] feature-major.  One copy brings the three projections into the
-        [batch, heads, seq, head size] layout torch's attention wants contiguous (on strided views of the
-        feature-major activations it runs ten times slower), one copy brings the context back."""
+        """qkv: [3 * hidden, batch*seq] feature-major; returns the context [hidden, batch*seq].  One HIP kernel that
+        reads and writes the feature-major layout (sspmm_attention_fm_f16 of the C ABI) where its shape limits hold
+        (head size 64, seq a multiple of 64).  Otherwise torch's attention between two relayout copies:
+        one brings the three projections into the [batch, heads, seq, head size] layout it wants contiguous (on
+        strided views of the feature-major activations it runs ten times slower), one brings the context back."""
         h, d = self.heads, self.hidden // self.heads
+        ctx = attention_fm(qkv, self.hidden, h, batch, seq)
+        if ctx is not None:
+            return ctx
         c = qkv.view(3, h, d, batch, seq).permute(0, 3, 1, 4, 2).contiguous()
         ctx = torch.nn.functional.scaled_dot_product_attention(c[0], c[1], c[2], scale=1.0 / math.sqrt(d))
         return ctx.permute(1, 3, 0, 2).reshape(self.hidden, batch * seq)

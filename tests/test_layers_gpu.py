@@ -78,3 +78,71 @@ def test_feature_major_add_layernorm_matches_torch(built_library, H, T, residual
     if T % 4 == 0 and H > 1:
         odd = add_layernorm(x[:, :T - 1].contiguous(), None if a is None else a[:, :T - 1].contiguous(), ln)
         assert (odd.float() - want[:, :T - 1]).abs().max().item() <= 4e-3 * max(1.0, want.abs().max().item())
+
+
+def _attention_reference(q, k, v, batch, heads, seq, scale):
+    """fp32 attention of feature-major [heads * d, batch * seq] operands, written out with plain matmuls."""
+    d = q.shape[0] // heads
+    f = lambda t: t.float().view(heads, d, batch, seq).permute(2, 0, 3, 1)  # noqa: E731  [batch, heads, seq, d]
+    p = torch.softmax(f(q) @ f(k).transpose(-1, -2) * scale, dim=-1)
+    return (p @ f(v)).permute(1, 3, 0, 2).reshape(heads * d, batch * seq)
+
+
+@pytest.mark.parametrize("batch,heads,seq", [(1, 1, 64), (2, 3, 128), (3, 2, 192), (8, 12, 512), (1, 2, 320), (1, 1, 1024)])
+def test_feature_major_attention_matches_fp32_attention(built_library, batch, heads, seq):
+    """sspmm_attention_fm_f16 through the C ABI, operands as three row ranges of one fused projection."""
+    from sspmm_amd import _lib
+    from sspmm_amd.layers import attention_fm
+    hidden, T = heads * 64, batch * seq
+    g = torch.Generator("cuda").manual_seed(seq + heads)
+    qkv = torch.randn(3 * hidden, T, device="cuda", generator=g).half()
+    qkv[:hidden] *= 2.0  # scores spread over several units, so the softmax is far from uniform
+    scale = 0.125
+    got = attention_fm(qkv, hidden, heads, batch, seq)
+    assert got is not None and got.shape == (hidden, T) and got.dtype == torch.float16
+    want = _attention_reference(qkv[:hidden], qkv[hidden:2 * hidden], qkv[2 * hidden:], batch, heads, seq, scale)
+    assert (got.float() - want).abs().max().item() <= 2e-3 * max(1.0, want.abs().max().item())
+    # separate operands with their own leading dimension, output into a wider array: the columns beyond stay untouched
+    ld, ld_out = T + 24, T + 8
+    q, k, v = (torch.randn(hidden, ld, device="cuda", generator=g).half() for _ in range(3))
+    out = torch.full((hidden, ld_out), 7.0, dtype=torch.float16, device="cuda")
+    rc = _lib.lib().sspmm_attention_fm_f16(batch, heads, seq, 64, q.data_ptr(), k.data_ptr(), v.data_ptr(), ld, out.data_ptr(),
+                                           ld_out, scale, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    want = _attention_reference(q[:, :T], k[:, :T], v[:, :T], batch, heads, seq, scale)
+    assert (out[:, :T].float() - want).abs().max().item() <= 2e-3 * max(1.0, want.abs().max().item())
+    assert torch.all(out[:, T:] == 7.0)
+
+
+def test_feature_major_attention_rejects_what_it_does_not_cover(built_library):
+    from sspmm_amd import _lib
+    L = _lib.lib()
+    t = torch.zeros(64, 1024, dtype=torch.float16, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+    args = lambda **kw: [kw.get("batch", 1), kw.get("heads", 1), kw.get("seq", 64), kw.get("d", 64), t.data_ptr() + kw.get("off", 0),  # noqa: E731
+                         t.data_ptr(), t.data_ptr(), kw.get("ld", 1024), t.data_ptr(), 1024, 0.125, s]
+    assert L.sspmm_attention_fm_f16(*args()) == 0
+    for bad in (dict(d=32), dict(seq=96), dict(seq=16448, ld=16448), dict(ld=1020), dict(off=2), dict(seq=512, batch=4, ld=1024), dict(batch=-1)):
+        assert L.sspmm_attention_fm_f16(*args(**bad)) == 1, bad
+    assert L.sspmm_attention_fm_f16(*args(batch=0)) == 0
+    torch.cuda.synchronize()
+
+
+def test_encoder_layer_at_the_benchmark_shape_takes_the_attention_kernel(built_library):
+    """hidden 768, 12 heads, 8 x 512 tokens: the layer with the feature-major attention kernel against the same layer
+    with torch's attention between relayout copies."""
+    hidden, heads, ffn, V, batch, seq = 768, 12, 3072, 16, 8, 512
+    mk = lambda o, i, s: _vector_sparse_linear(o, i, V, 0.9, seed=s)
+    layer = SparseEncoderLayer(hidden, heads, ffn, mk(hidden, hidden, 1), mk(hidden, hidden, 2), mk(hidden, hidden, 3),
+                               mk(hidden, hidden, 4), mk(ffn, hidden, 5), mk(hidden, ffn, 6)).cuda().half()
+    x = torch.randn(hidden, batch * seq, device="cuda", generator=torch.Generator("cuda").manual_seed(5)).half()
+    import sspmm_amd.layers as layers_mod
+    with torch.no_grad():
+        got = layer(x, batch, seq)
+        kernel = layers_mod.attention_fm
+        layers_mod.attention_fm = lambda *a, **kw: None
+        try:
+            want = layer(x, batch, seq)
+        finally:
+            layers_mod.attention_fm = kernel
+    assert max_rel_err(got.float().cpu().numpy(), want.float().cpu().numpy()) <= 1e-2

@@ -93,6 +93,22 @@ int sspmm_batched_f16_f32(int batch, int m_vec, int V, int N, int K, const int32
                           int64_t stride_C, void *hip_stream);
 
 /* ------------------------------------------------------------------------------------------
+ * A linear layer with a vector-sparse weight in one launch: C = act(A_cvse * B + bias), fp16 out.
+ * What the reference's model code does with nn.Linear (weight, bias) followed by the activation in
+ * torch (reference end2end/sspmm_e2e/end_to_end.py:55-56, 70-73); here bias and activation are
+ * applied to the fp32 sums before they are rounded, so C is written once and never re-read.
+ *   bias        fp16 device pointer, one value per output row (m_vec * V), or NULL
+ *   activation  SSPMM_ACT_NONE, or SSPMM_ACT_GELU = 0.5 x (1 + erf(x / sqrt 2)) (torch's default)
+ * With bias == NULL and SSPMM_ACT_NONE the result equals sspmm_f16_f16's.  Other arguments as
+ * sspmm_f16_f16 (no row_indices).
+ * ---------------------------------------------------------------------------------------- */
+#define SSPMM_ACT_NONE 0
+#define SSPMM_ACT_GELU 1
+int sspmm_linear_f16(int m_vec, int V, int N, int K, const int32_t *row_offsets, const int32_t *col_idx,
+                     const sspmm_half_t *values, const sspmm_half_t *B, const sspmm_half_t *bias, int activation,
+                     sspmm_half_t *C, void *hip_stream);
+
+/* ------------------------------------------------------------------------------------------
  * Plans: what the library can know about a sparsity pattern before its first product.
  *
  * The reference starts one thread block per vector-row whatever its length (reference
@@ -267,7 +283,7 @@ int svc_permute_csr(int M, const int32_t *perm, const int32_t *row_ptr, const in
  * No counterpart among the reference's kernels: its encoder block (reference
  * end2end/sspmm_e2e/end_to_end.py:58-75) calls torch's LayerNorm on token-major tensors; on the
  * SpMM's layout that costs two transposed copies per call.  a, gamma, beta may be NULL (no
- * residual, scale one, shift zero).  T a multiple of 4, H up to 1024, 8-byte aligned pointers.
+ * residual, scale one, shift zero).  T a multiple of 4, H up to 4096, 8-byte aligned pointers.
  * ---------------------------------------------------------------------------------------- */
 int sspmm_add_layernorm_f16(int H, int T, const sspmm_half_t *x, const sspmm_half_t *a, const sspmm_half_t *gamma,
                             const sspmm_half_t *beta, float eps, sspmm_half_t *out, void *hip_stream);

@@ -18,7 +18,7 @@ constexpr int kInvalid = (int)hipErrorInvalidValue;
 int spmm_entry(int batch, int m_vec, int V, int N, int K, const int32_t *row_indices, const int32_t *row_offsets,
                const int32_t *col_idx, const sspmm_half_t *values, int64_t stride_values, const sspmm_half_t *B,
                int64_t stride_B, void *C, int64_t stride_C, bool out_f16, void *stream,
-               const sspmm::Plan *plan = nullptr) {
+               const sspmm::Plan *plan = nullptr, const sspmm_half_t *bias = nullptr, int activation = 0) {
   if (V != 8 && V != 16) return kInvalid;
   if (batch < 0 || m_vec < 0 || N < 0 || K < 0) return kInvalid;
   if (batch == 0 || m_vec == 0 || N == 0) return 0;  // nothing to write
@@ -44,6 +44,8 @@ int spmm_entry(int batch, int m_vec, int V, int N, int K, const int32_t *row_ind
   a.stride_values = stride_values;
   a.stride_B = stride_B;
   a.stride_C = stride_C;
+  a.bias = bias;
+  a.act = activation;
   if (plan) return (int)sspmm::launch_spmm_planned(*plan, a, out_f16, static_cast<hipStream_t>(stream));
   return (int)sspmm::launch_spmm(a, V, out_f16, static_cast<hipStream_t>(stream));
 }
@@ -90,6 +92,14 @@ int sspmm_f16_f16(int m_vec, int V, int N, int K, const int32_t *row_indices, co
                   const int32_t *col_idx, const sspmm_half_t *values, const sspmm_half_t *B, sspmm_half_t *C,
                   void *hip_stream) {
   return spmm_entry(1, m_vec, V, N, K, row_indices, row_offsets, col_idx, values, 0, B, 0, C, 0, true, hip_stream);
+}
+
+int sspmm_linear_f16(int m_vec, int V, int N, int K, const int32_t *row_offsets, const int32_t *col_idx,
+                     const sspmm_half_t *values, const sspmm_half_t *B, const sspmm_half_t *bias, int activation,
+                     sspmm_half_t *C, void *hip_stream) {
+  if (activation != SSPMM_ACT_NONE && activation != SSPMM_ACT_GELU) return kInvalid;
+  return spmm_entry(1, m_vec, V, N, K, nullptr, row_offsets, col_idx, values, 0, B, 0, C, 0, true, hip_stream, nullptr, bias,
+                    activation);
 }
 
 int sspmm_batched_f16_f16(int batch, int m_vec, int V, int N, int K, const int32_t *row_indices,
@@ -329,7 +339,7 @@ int svc_permute_csr(int M, const int32_t *perm, const int32_t *row_ptr, const in
 
 int sspmm_add_layernorm_f16(int H, int T, const sspmm_half_t *x, const sspmm_half_t *a, const sspmm_half_t *gamma,
                             const sspmm_half_t *beta, float eps, sspmm_half_t *out, void *hip_stream) {
-  if (H < 0 || T < 0 || T % 4 != 0 || H > 1024) return kInvalid;
+  if (H < 0 || T < 0 || T % 4 != 0 || H > 4096) return kInvalid;
   if (H == 0 || T == 0) return 0;
   if (!x || !out) return kInvalid;
   if (reinterpret_cast<uintptr_t>(x) % 8 || reinterpret_cast<uintptr_t>(a) % 8 || reinterpret_cast<uintptr_t>(out) % 8)

@@ -9,7 +9,6 @@
 namespace sspmm {
 
 // LDS bytes a workgroup needs for H features (the caller checks it against the 160 KB of a CU).
-size_t add_layernorm_lds_bytes(int H);
 
 // out[H, T] = LayerNorm over the H features of every token of fp16(x + a) (a may be null), fp16 in and out.
 // T must be a multiple of 4 and the pointers 8-byte aligned.

@@ -101,7 +101,8 @@ hipError_t launch_spmm_planned(const Plan &pl, const SpmmArgs &a, bool out_f16, 
   // Rows are cut only when some row is much longer than the rest (the budget is at least twice the mean row):
   // an even pattern keeps the kernels chosen by shape.
   const bool skewed = pl.header[kHdrSplitRows] > 0;
-  if (can_balance && (forced == 7 || (forced == 0 && skewed)))
+  const bool epilogue = a.bias != nullptr || a.act != 0;  // (the load-balanced kernel does not apply one)
+  if (can_balance && !epilogue && (forced == 7 || (forced == 0 && skewed)))
     return launch_spmm_balanced(a, pl.V, out_f16, pl.view, pl.header[kHdrItems], false, stream);
   return launch_spmm(a, pl.V, out_f16, stream);
 }

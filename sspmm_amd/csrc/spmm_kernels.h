@@ -16,6 +16,11 @@ struct SpmmArgs {
   const uint16_t *B;
   void *C;
   int64_t stride_values, stride_B, stride_C;  // per-batch strides in elements
+  // Epilogue of the linear-layer entry point, applied to the fp32 sums before they are rounded and stored:
+  // C[r, n] = act(sum + bias[r]).  bias: fp16 per output row (m_vec * V), nullable; act: 0 none, 1 GELU (erf form).
+  // Honoured by the scalar, gather and staged gather kernels; launch_spmm keeps to those when either is set.
+  const uint16_t *bias;
+  int act;
   // filled by the launcher
   uint32_t n_tiles, total_work, per_xcd;
   uint32_t n_slabs, row_blocks, rows_per_block, group_by_batch;  // slab kernel

@@ -58,6 +58,29 @@ union Half8Bits {
   uint32_t u[4];
 };
 
+// erf with an absolute error below 2e-7 (Abramowitz and Stegun 7.1.26): a reciprocal, an exponential and five
+// multiply-adds, where the library's erff spends three times as many instructions on bits an fp16 result drops.
+__device__ __forceinline__ float erf_fast(float x) {
+  const float ax = __builtin_fabsf(x);
+  const float t = __builtin_amdgcn_rcpf(__builtin_fmaf(0.3275911f, ax, 1.0f));
+  float poly = __builtin_fmaf(1.061405429f, t, -1.453152027f);
+  poly = __builtin_fmaf(poly, t, 1.421413741f);
+  poly = __builtin_fmaf(poly, t, -0.284496736f);
+  poly = __builtin_fmaf(poly, t, 0.254829592f);
+  const float e = __builtin_amdgcn_exp2f(-1.4426950408889634f * ax * ax);
+  return __builtin_copysignf(__builtin_fmaf(-poly * t, e, 1.0f), x);
+}
+// The linear-layer epilogue on one fp32 sum: bias, then the activation (1 = GELU, 0.5 x (1 + erf(x / sqrt 2))).
+__device__ __forceinline__ float epilogue_value(float x, float bias, int act) {
+  x += bias;
+  if (act == 1) x = 0.5f * x * (1.0f + erf_fast(x * 0.70710678118654752f));
+  return x;
+}
+__device__ __forceinline__ bool has_epilogue(const SpmmArgs &p) { return p.bias != nullptr || p.act != 0; }
+__device__ __forceinline__ float bias_of_row(const SpmmArgs &p, int64_t out_row) {
+  return p.bias ? (float)reinterpret_cast<const _Float16 *>(p.bias)[out_row] : 0.0f;
+}
+
 template <typename OutT>
 struct Store8;
 
@@ -299,6 +322,12 @@ __global__ __launch_bounds__(64) void spmm_gather_kernel(const SpmmArgs p) {
   floatx4 acc[CPL];
 #pragma unroll
   for (int q = 0; q < CPL; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
+  // the bias of the lane's four output rows, fetched before the loop so that the row's end does not wait for it
+  _Float16 bias4[4] = {0, 0, 0, 0};
+  if (p.bias) {
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) bias4[rr] = reinterpret_cast<const _Float16 *>(p.bias)[(int64_t)row * V + ((4 * g + rr) & (V - 1))];
+  }
 
   if (beg < end) {
     // Heads run two chunks ahead of the arithmetic, bodies one (two buffers of each, used alternately).
@@ -329,6 +358,13 @@ __global__ __launch_bounds__(64) void spmm_gather_kernel(const SpmmArgs p) {
     }
   }
 
+  if (has_epilogue(p)) {  // (uniform) acc[q][rr] belongs to output row 4g + rr of the vector-row
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) {
+#pragma unroll
+      for (int q = 0; q < CPL; ++q) acc[q][rr] = epilogue_value(acc[q][rr], (float)bias4[rr], p.act);
+    }
+  }
   if constexpr (std::is_same<OutT, float>::value && CPL == 8) {
     __shared__ __align__(16) float ctile[V][128 + 4];
     store_tile_f32_lines<V>(ctile, acc, lane, reinterpret_cast<float *>(p.C) + (int64_t)batch * p.stride_C + (int64_t)row * V * p.N,
@@ -1262,7 +1298,15 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(V == 8 ? 5 :
   floatx4 acc[4];
 #pragma unroll
   for (int q = 0; q < 4; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
+  // (the bias of the lane's output row is fetched before the loop so that the row's end does not wait for it)
+  const float b = bias_of_row(p, (int64_t)row * V + (lane & (V - 1)));
   stage_accumulate<V>(acc, x, srd_cols, srd_vals, srd_b, beg, end, lane_n2, lane_col_off, b_bytes);
+  if (has_epilogue(p)) {  // (uniform) every accumulator of lane (m, g) belongs to output row m of the vector-row
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[q][r] = epilogue_value(acc[q][r], b, p.act);
+  }
 
   SlabStore<V, OutT, 4> out;
   out.init(lane, (int)tile * 64, p.N);
@@ -1436,6 +1480,10 @@ __global__ __launch_bounds__(64) void spmm_generic_kernel(const SpmmArgs p) {
 #pragma unroll
     for (int v = 0; v < V; ++v) acc[v] += (float)vals[(int64_t)j * V + v] * b;
   }
+  if (has_epilogue(p)) {
+#pragma unroll
+    for (int v = 0; v < V; ++v) acc[v] = epilogue_value(acc[v], bias_of_row(p, (int64_t)row * V + v), p.act);
+  }
   OutT *cbase = reinterpret_cast<OutT *>(p.C) + (int64_t)batch * p.stride_C;
 #pragma unroll
   for (int v = 0; v < V; ++v) cbase[((int64_t)row * V + v) * p.N + n] = (OutT)acc[v];
@@ -1554,13 +1602,14 @@ static hipError_t launch_v(const SpmmArgs &a, int which, hipStream_t stream) {
     // as many (about 10 % on launches of 4-5 us; from two to four waves per CU the register path is 10-20 % faster).
     // (Not for K above 3072: where such a matrix is denser than 90 % its long rows cost the staged form 1.5x.)
     const bool few_waves = a.K <= 3072 && p.total_work <= 2u * device_cus();
+    const bool epilogue = a.bias != nullptr || a.act != 0;  // (the split-row kernel does not apply one)
     if ((g_kernel_override == 6 || a.N <= 64 || (few_waves && g_kernel_override == 0)) && c_ok) {
       p.n_tiles = (uint32_t)((a.N + 63) / 64);
       p.total_work = (uint32_t)a.m_vec * p.n_tiles * (uint32_t)a.batch;
       p.per_xcd = (p.total_work + 7u) / 8u;
       g_last_kernel = 6;
       hipLaunchKernelGGL((spmm_stage_kernel<V, OutT>), dim3(p.per_xcd * 8u), dim3(64), 0, stream, p);
-    } else if (a.K > kSplitMinK) {
+    } else if (a.K > kSplitMinK && !epilogue) {
       g_last_kernel = 4;
       static_assert(kSplitWaves >= 4, "wave rr < 4 stores output row 4g + rr");
       p.total_work = (((uint32_t)a.m_vec + kSplitWaves - 1u) / kSplitWaves) * p.n_tiles * (uint32_t)a.batch;
@@ -1670,6 +1719,7 @@ hipError_t launch_spmm(const SpmmArgs &a, int V, bool out_f16, hipStream_t strea
     if (g_kernel_override == 2 || g_kernel_override == 6) which = 2;
     if (g_kernel_override == 3 && slab_ok) which = 3;
     if (g_kernel_override == 3 && narrow_ok) which = 5;
+    if (a.bias != nullptr || a.act != 0) which = 2;  // the kernels that apply the linear-layer epilogue
   }
   if (g_kernel_override == 1) which = 1;
   g_last_kernel = which;

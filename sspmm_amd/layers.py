@@ -18,7 +18,7 @@ import math
 import numpy as np
 import torch
 
-from .spmm import spmm
+from .spmm import linear as linear_op, spmm
 from .svc import svc
 
 
@@ -30,8 +30,9 @@ class SparseLinear(torch.nn.Module):
     takes them)."""
 
     def __init__(self, in_features, out_features, vec_length, row_offsets, column_indices, values, bias=None,
-                 out_dtype=torch.float16):
+                 out_dtype=torch.float16, activation=None):
         super().__init__()
+        self.activation = activation  # None or "gelu": applied to W @ x + bias
         if out_features % vec_length:
             raise ValueError("out_features must be a multiple of vec_length")
         self.in_features, self.out_features, self.vec_length = in_features, out_features, vec_length
@@ -94,10 +95,17 @@ class SparseLinear(torch.nn.Module):
         plan = getattr(self, "plan", None)
         if plan is not None and x.size(1) > plan.max_N:
             plan = None
+        fuse = plan is None and self.out_dtype == torch.float16 and (self.bias is None or self.bias.dtype == torch.float16)
+        if fuse and (self.bias is not None or self.activation is not None):
+            # bias and activation in the product's epilogue: one launch, the output written once
+            return linear_op(self.row_offsets, self.column_indices, self.values, x.contiguous(), self.vec_length,
+                             bias=self.bias, activation=self.activation)
         y = spmm(None, self.row_offsets, self.column_indices, self.values, x.contiguous(), self.vec_length,
                  out_dtype=self.out_dtype, plan=plan)
         if self.bias is not None:
             y = y + self.bias[:, None].to(y.dtype)
+        if self.activation == "gelu":
+            y = torch.nn.functional.gelu(y)
         return y
 
     def dense_weight(self):
@@ -118,7 +126,7 @@ def add_layernorm(x, a, ln):
     where its shape limits hold, torch on transposed copies otherwise."""
     from . import _lib
     H, T = x.shape
-    ok = (x.dtype == torch.float16 and x.is_cuda and x.is_contiguous() and T % 4 == 0 and H <= 1024 and
+    ok = (x.dtype == torch.float16 and x.is_cuda and x.is_contiguous() and T % 4 == 0 and H <= 4096 and
           (a is None or (a.dtype == torch.float16 and a.is_contiguous() and a.shape == x.shape)) and
           ln.weight is not None and ln.weight.dtype == torch.float16 and tuple(ln.normalized_shape) == (H,))
     if not ok:
@@ -165,6 +173,9 @@ class SparseEncoderLayer(torch.nn.Module):
         self.q, self.k, self.v, self.o, self.ffn1, self.ffn2 = q, k, v, o, ffn1, ffn2
         # query, key and value projections as one SpMM over the three patterns stacked along M
         self.qkv = SparseLinear.concat([q, k, v])
+        # the first feed-forward product with its GELU in the product's epilogue (shares ffn1's arrays)
+        self.ffn1_gelu = SparseLinear(ffn1.in_features, ffn1.out_features, ffn1.vec_length, ffn1.row_offsets, ffn1.column_indices,
+                                      ffn1.values, ffn1.bias, out_dtype=ffn1.out_dtype, activation="gelu")
         self.ln1 = torch.nn.LayerNorm(hidden)
         self.ln2 = torch.nn.LayerNorm(hidden)
 
@@ -183,10 +194,11 @@ class SparseEncoderLayer(torch.nn.Module):
         return ctx.permute(1, 3, 0, 2).reshape(self.hidden, batch * seq)
 
     def forward(self, x, batch, seq, linear=None):
-        """x: [hidden, batch*seq] fp16.  `linear(name, layer, x)` may replace how a projection ("qkv", "o", "ffn1",
-        "ffn2") is evaluated (the benchmark passes a dense matmul there to time the same layer without sparsity)."""
+        """x: [hidden, batch*seq] fp16.  `linear(name, layer, x)` may replace how a projection ("qkv", "o",
+        "ffn1_gelu", "ffn2"; "ffn1_gelu" is the first feed-forward product with the GELU behind it) is evaluated
+        (the benchmark passes a dense matmul there to time the same layer without sparsity)."""
         f = linear or (lambda name, layer, t: layer(t))
         a = f("o", self.o, self._attention(f("qkv", self.qkv, x), batch, seq))
         x = add_layernorm(x, a, self.ln1)
-        y = f("ffn2", self.ffn2, torch.nn.functional.gelu(f("ffn1", self.ffn1, x)))
+        y = f("ffn2", self.ffn2, f("ffn1_gelu", self.ffn1_gelu, x))
         return add_layernorm(x, y, self.ln2)

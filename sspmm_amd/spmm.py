@@ -70,6 +70,32 @@ def spmm(row_indices, row_offsets, column_indices, values, rhs_matrix, vec_lengt
     return out
 
 
+ACTIVATIONS = {None: 0, "none": 0, "gelu": 1}
+
+
+def linear(row_offsets, column_indices, values, rhs_matrix, vec_length, bias=None, activation=None):
+    """act(A_cvse @ rhs_matrix + bias[:, None]) as one launch, fp16 out (sspmm_linear_f16 of the C ABI): what the
+    reference's model code computes with nn.Linear and the activation behind it (reference
+    end2end/sspmm_e2e/end_to_end.py:55-56, 70-73), bias and activation applied to the fp32 sums.
+    bias: fp16 [m_vec * V] or None; activation: None / "none" / "gelu" (the erf form, torch's default)."""
+    _check_inputs(None, row_offsets, column_indices, values, rhs_matrix, vec_length)
+    if activation not in ACTIVATIONS:
+        raise ValueError("activation must be one of %r" % (sorted(k for k in ACTIVATIONS if k),))
+    if rhs_matrix.dim() != 2:
+        raise ValueError("rhs_matrix must be [K, N]")
+    m_vec = row_offsets.size(-1) - 1
+    K, N = rhs_matrix.size(0), rhs_matrix.size(1)
+    if bias is not None and (bias.dtype != torch.float16 or not bias.is_cuda or not bias.is_contiguous() or
+                             bias.numel() != m_vec * vec_length):
+        raise ValueError("bias must be a contiguous fp16 GPU tensor of m_vec * vec_length = %d elements" % (m_vec * vec_length))
+    out = torch.empty((m_vec * vec_length, N), dtype=torch.float16, device=rhs_matrix.device)
+    with torch.cuda.device(rhs_matrix.device):
+        rc = _lib.lib().sspmm_linear_f16(m_vec, vec_length, N, K, _ptr(row_offsets), _ptr(column_indices), _ptr(values),
+                                         _ptr(rhs_matrix), _ptr(bias), ACTIVATIONS[activation], _ptr(out), _stream())
+    _lib.check(rc, "sspmm_linear_f16")
+    return out
+
+
 def bspmm(row_indices, row_offsets, column_indices, values, rhs_matrix, vec_length, out_dtype=torch.float16, plan=None):
     """Batched SpMM with one pattern for the whole batch: values [batch, nvec*V],
     rhs_matrix [batch, K, N] -> [batch, m_vec*V, N] (reference batched_spmm_cuda,

@@ -52,12 +52,14 @@ def test_encoder_layer_matches_the_same_layer_with_dense_products(built_library)
     assert torch.equal(dense["qkv"], torch.cat([layer.q.dense_weight(), layer.k.dense_weight(), layer.v.dense_weight()]))
     with torch.no_grad():
         got = layer(x, batch, seq)
-        want = layer(x, batch, seq, linear=lambda name, lin, t: (dense[name].float() @ t.float()).half())
+        gelu = torch.nn.functional.gelu
+        want = layer(x, batch, seq, linear=lambda name, lin, t: (
+            gelu(dense["ffn1"].float() @ t.float()) if name == "ffn1_gelu" else dense[name].float() @ t.float()).half())
     assert got.shape == (hidden, batch * seq)
     assert max_rel_err(got.float().cpu().numpy(), want.float().cpu().numpy()) <= 1e-2
 
 
-@pytest.mark.parametrize("H,T", [(768, 4096), (256, 128), (100, 36), (1024, 68), (1, 4)])
+@pytest.mark.parametrize("H,T", [(768, 4096), (256, 128), (100, 36), (1024, 68), (1, 4), (3072, 520), (4096, 16)])
 @pytest.mark.parametrize("residual", [True, False])
 def test_feature_major_add_layernorm_matches_torch(built_library, H, T, residual):
     """The fused kernel against torch's LayerNorm on the transposed sum: same fp16 sum, statistics in fp32."""
@@ -146,3 +148,39 @@ def test_encoder_layer_at_the_benchmark_shape_takes_the_attention_kernel(built_l
         finally:
             layers_mod.attention_fm = kernel
     assert max_rel_err(got.float().cpu().numpy(), want.float().cpu().numpy()) <= 1e-2
+
+
+@pytest.mark.parametrize("V,out_f,in_f,N", [(16, 3072, 768, 4096), (8, 64, 100, 72), (16, 128, 5000, 64), (8, 256, 96, 33)])
+@pytest.mark.parametrize("activation", [None, "gelu"])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_linear_epilogue_matches_separate_bias_and_gelu(built_library, V, out_f, in_f, N, activation, with_bias):
+    """sspmm_linear_f16 against the fp32 product with bias and erf-GELU applied in fp32: the gather kernel (wide N),
+    the staged gather kernel (few waves, N <= 64, K above the split-row kernel's threshold) and the scalar kernel
+    (N not a multiple of 8)."""
+    from sspmm_amd.spmm import linear
+    vs = synth.vector_sparse(out_f, in_f, V, 0.9, seed=out_f + N, std=0.05)
+    g = torch.Generator("cuda").manual_seed(N)
+    x = torch.randn(in_f, N, device="cuda", generator=g).half()
+    bias = torch.randn(out_f, device="cuda", generator=g).half() if with_bias else None
+    ro, ci, va = dev(vs.row_offsets), dev(vs.col_idx), dev(vs.values)
+    got = linear(ro, ci, va, x, V, bias=bias, activation=activation)
+    want = sspmm_amd.spmm(None, ro, ci, va, x, V, out_dtype=torch.float32)
+    if bias is not None:
+        want = want + bias.float()[:, None]
+    if activation == "gelu":
+        want = torch.nn.functional.gelu(want)
+    assert got.dtype == torch.float16 and got.shape == (out_f, N)
+    assert max_rel_err(got.float().cpu().numpy(), want.cpu().numpy()) <= 2e-3
+    if bias is None and activation is None:
+        assert torch.equal(got, sspmm_amd.spmm(None, ro, ci, va, x, V))
+
+
+def test_sparse_linear_fuses_bias_and_activation(built_library):
+    lin = _vector_sparse_linear(256, 192, 16, 0.8, seed=71, activation="gelu")
+    lin.bias = torch.randn(256, device="cuda", generator=torch.Generator("cuda").manual_seed(4)).half()
+    x = torch.randn(192, 200, device="cuda", generator=torch.Generator("cuda").manual_seed(5)).half()
+    want = torch.nn.functional.gelu(lin.dense_weight().float() @ x.float() + lin.bias.float()[:, None])
+    assert max_rel_err(lin(x).float().cpu().numpy(), want.cpu().numpy()) <= 2e-3
+    from sspmm_amd import _lib
+    L = _lib.lib()
+    assert L.sspmm_linear_f16(1, 16, 8, 8, 0, 0, 0, 0, 0, 2, 0, 0) == 1  # unknown activation

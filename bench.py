@@ -139,6 +139,33 @@ def graph_time(fn, launches=20, replays=20):
     return start.elapsed_time(end) / (launches * replays)
 
 
+_PROBE = {}
+
+
+def gather_probe(L, torch, waves_per_cu, rows=2304, row_bytes=6144, steps=32):
+    """TB/s at which the device serves the gather kernels' access pattern (16 lanes read 256 contiguous bytes of a random
+    row of a matrix that fits the caches, eight 16-byte loads per lane in flight) with waves_per_cu waves on each of
+    the 256 CUs: sspmm_probe_gather of the C ABI, a loop of loads and nothing else."""
+    mat = torch.ones(rows * row_bytes // 2, dtype=torch.float16, device="cuda")
+    waves = 256 * waves_per_cu
+    sink = torch.empty(waves * 4, dtype=torch.int32, device="cuda")
+
+    def run():
+        rc = L.sspmm_probe_gather(mat.data_ptr(), rows, row_bytes, waves, steps, sink.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        if rc:
+            raise RuntimeError("sspmm_probe_gather failed: %d" % rc)
+
+    ms = time_launches(run, 50, 10)
+    return waves * steps * 8192 / ms / 1e9
+
+
+def gather_probe_rate(L, torch):
+    """The probe's rate at full occupancy (32 waves per CU), measured once per process."""
+    if "tbps" not in _PROBE:
+        _PROBE["tbps"] = gather_probe(L, torch, 32)
+    return _PROBE["tbps"]
+
+
 def figures(ms, alg_bytes, flops):
     return {"ms": ms, "useful_tflops": flops / ms / 1e9, "alg_bytes": alg_bytes, "hbm_gbps": alg_bytes / ms / 1e6,
             "hbm_frac": alg_bytes / ms / 1e6 / HBM_PEAK_GBPS}
@@ -190,6 +217,16 @@ def spmm_case(L, torch, synth, M, K, V, sparsity, N, batch, out_f32, std, seed, 
         gms = graph_time(launch_on)
         out["ms_in_a_graph"] = gms
         out["hbm_frac_in_a_graph"] = bytes_alg / gms / 1e6 / HBM_PEAK_GBPS
+        # a plain device copy that moves the same number of bytes (half read, half written), timed the same way:
+        # what one launch of this size can reach at all, launch and ramp included
+        src = torch.empty(bytes_alg // 2, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        cms = time_launches(lambda: dst.copy_(src), steps, warmup)
+        out["plain_copy_of_the_same_bytes_ms"] = cms
+        out["time_vs_plain_copy_of_the_same_bytes"] = ms / cms
+        # and what the gathers alone cost at the rate the device serves this access pattern from its caches
+        out["gather_bytes_at_the_probe_rate_ms"] = out["gather_bytes_no_reuse"] / gather_probe_rate(L, torch) / 1e9
+        del src, dst
     if dense:
         A = torch.zeros(vs.m_vec * V, K, dtype=torch.float16, device="cuda")
         Ad = A.unsqueeze(0).expand(batch, -1, -1).contiguous()
@@ -729,6 +766,8 @@ def main():
         ceilings = {"device_copy_1GiB_gbps": 2 * src.numel() * 4 / copy_ms / 1e6,
                     "device_fill_1GiB_gbps": src.numel() * 4 / fill_ms / 1e6}
         ceilings["frac_of_device_copy"] = main_res["hbm_gbps"] / ceilings["device_copy_1GiB_gbps"]
+        # the caches' side: the gather kernels' access pattern with nothing else in the loop, at 4, 8, 16 and 32 waves per CU
+        ceilings["cache_to_cu_gather_tbps_by_waves_per_cu"] = {str(w): gather_probe(L, torch, w) for w in (4, 8, 16, 32)}
         del src, dst
 
     # parity of batch elements spread over the launch (first, last, and one per way the batch is dealt to the XCDs)

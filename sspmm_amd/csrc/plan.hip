@@ -104,7 +104,10 @@ hipError_t launch_spmm_planned(const Plan &pl, const SpmmArgs &a, bool out_f16, 
   const bool epilogue = a.bias != nullptr || a.act != 0;  // (the load-balanced kernel does not apply one)
   if (can_balance && !epilogue && (forced == 7 || (forced == 0 && skewed)))
     return launch_spmm_balanced(a, pl.V, out_f16, pl.view, pl.header[kHdrItems], false, stream);
-  return launch_spmm(a, pl.V, out_f16, stream);
+  SpmmArgs b = a;
+  // (at least 1: an empty pattern is as sparse as it gets, and 0 would say the density is unknown)
+  b.mean_row_vectors = pl.m_vec > 0 ? (int)((int64_t)pl.header[kHdrNvec] / pl.m_vec) + 1 : 0;
+  return launch_spmm(b, pl.V, out_f16, stream);
 }
 
 // ------------------------------------------------------------------------------------------

@@ -21,6 +21,9 @@ struct SpmmArgs {
   // Honoured by the scalar, gather and staged gather kernels; launch_spmm keeps to those when either is set.
   const uint16_t *bias;
   int act;
+  // Mean number of stored vectors per vector-row when the caller knows it (products with a plan), else 0: the
+  // kernel choice then also looks at the density, not only at the shape.
+  int mean_row_vectors;
   // filled by the launcher
   uint32_t n_tiles, total_work, per_xcd;
   uint32_t n_slabs, row_blocks, rows_per_block, group_by_batch;  // slab kernel

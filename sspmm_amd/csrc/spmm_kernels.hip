@@ -1714,8 +1714,20 @@ hipError_t launch_spmm(const SpmmArgs &a, int V, bool out_f16, hipStream_t strea
     // wins)
     // (N <= 64: the alternative is the staged gather kernel, which the slab kernel beats by 1.2-1.3x from 512 on)
     const uint32_t enough = (V == 8 || a.N <= 64) ? 512u : out_f16 ? 1024u : 2048u;
-    which = (slab_ok && a.m_vec >= 64 && blocks >= enough) ? 3 : 2;
+    // With the density known (a plan carries the pattern's vector count), a block of 32 vector-rows is counted by
+    // the work in it: the thresholds above were measured at 90 % sparsity, and at 70 % the slab kernel pays from a
+    // third of the blocks on (measured 1.1-1.28x over the gather kernels on shapes just below the thresholds).
+    uint64_t weighted = blocks;
+    if (a.mean_row_vectors > 0 && a.K > 0) {
+      const uint64_t percent = ((uint64_t)a.mean_row_vectors * 100u) / (uint64_t)a.K;  // density in percent (vectors per row / K)
+      if (percent > 10u) weighted = blocks * (percent < 40u ? percent : 40u) / 10u;
+    }
+    which = (slab_ok && a.m_vec >= 64 && weighted >= enough) ? 3 : 2;
     if (narrow_ok && V == 8 && a.m_vec >= 256 && 2u * blocks >= 1024) which = 5;
+    // Very sparse patterns with V = 16 and fp32 C: a vector-row is one step, the slab kernel's per-row work (claim,
+    // table entry, store set-up) outweighs it, and the gather kernels win (measured at 95 and 98 % sparsity up to 32
+    // vectors per row: 1.13-1.18x; with V = 8 the two tie, and between the gather kernels the density changes nothing).
+    if (which == 3 && !out_f16 && V == 16 && a.mean_row_vectors > 0 && a.mean_row_vectors <= 32) which = 2;
     if (g_kernel_override == 2 || g_kernel_override == 6) which = 2;
     if (g_kernel_override == 3 && slab_ok) which = 3;
     if (g_kernel_override == 3 && narrow_ok) which = 5;

@@ -248,3 +248,33 @@ def test_plan_argument_checks(built_library):
         plan.info()
     empty = Plan(torch.zeros(1, dtype=torch.int32, device="cuda"), 16, 32, max_N=8)
     assert empty.info().items == 0
+
+
+@pytest.mark.parametrize("M,K,V,sparsity,N,batch,want_plain,want_planned", [
+    (1024, 2304, 16, 0.95, 256, 16, 2, 2),   # between the gather kernels the density changes nothing
+    (2048, 1024, 16, 0.98, 256, 128, 3, 2),  # one step per row: a gather kernel in place of the slab kernel
+    (3072, 768, 8, 0.7, 64, 16, 6, 3),       # dense for this format: the slab kernel from fewer blocks on
+    (2048, 512, 8, 0.9, 256, 128, 3, 3),     # the density the thresholds were measured at: no change
+])
+def test_plan_of_an_even_pattern_picks_the_kernel_by_density(oracle, built_library, M, K, V, sparsity, N, batch, want_plain,
+                                                             want_planned):
+    """A plan knows the pattern's vector count; products with it choose between the slab, gather and staged kernels
+    by density as well as by shape.  The results agree with the oracle either way."""
+    L = _lib.lib()
+    vs = synth.vector_sparse(M, K, V, sparsity, seed=M + N, std=0.05)
+    g = torch.Generator("cuda").manual_seed(N)
+    vals = (torch.randn(batch, vs.col_idx.size * V, device="cuda", generator=g) * 0.05).half()
+    B = torch.randn(batch, K, N, device="cuda", generator=g).half()
+    ro, ci = dev(vs.row_offsets), dev(vs.col_idx)
+    plain = sspmm_amd.bspmm(None, ro, ci, vals, B, V, out_dtype=torch.float32)
+    assert L.sspmm_last_kernel() == want_plain
+    plan = Plan(ro, V, K, max_N=N, max_batch=batch)
+    assert plan.info().cut_rows == 0
+    planned = sspmm_amd.bspmm(None, ro, ci, vals, B, V, out_dtype=torch.float32, plan=plan)
+    assert L.sspmm_last_kernel() == want_planned
+    torch.cuda.synchronize()
+    for b in sorted({0, batch - 1}):
+        want = oracle.spmm(vs.m_vec, V, N, K, vs.row_offsets, vs.col_idx, vals[b].cpu().numpy(), B[b].cpu().numpy())
+        assert max_rel_err(planned[b].cpu().numpy(), want) <= TIGHT_F32
+        assert max_rel_err(plain[b].cpu().numpy(), want) <= TIGHT_F32
+    plan.destroy()

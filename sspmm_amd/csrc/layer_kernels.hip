@@ -153,7 +153,7 @@ hipError_t launch_add_layernorm(int H, int T, const uint16_t *x, const uint16_t 
 // (batch element, head): its 64 columns of Q go to LDS once, and the head's K and V pass through LDS in blocks of
 // 64 keys (64 features x 64 tokens each, as they lie in memory; two buffers, the next block's loads in flight in
 // registers while the current one is computed, one barrier per block), 45 KB of LDS in all, so three workgroups
-// share a CU.  Each wave computes for its 16 queries
+// share a CU.  Each wave computes for 32 queries (two sets of 16) and half of every block's keys
 //     scores^T[key, query] = sum_d K[d, key] Q[d, query]          (MFMA; both operands by transpose reads)
 //     out[d, query]        = sum_key V[d, key] P[query, key]       (MFMA; V read directly, P from registers)
 // per block with the running maximum and sum of the usual one-pass softmax.  The scores come out of the first
@@ -173,9 +173,14 @@ static constexpr int kAttThreads = 256;
 static constexpr int kAttD = 64;          // head size
 static constexpr int kAttQueries = 64;    // per workgroup, 16 per wave
 static constexpr int kAttKeys = 64;       // per block of the softmax
-static constexpr uint32_t kAttPitch = 64 * 2 + 16;  // bytes; rows padded so that the rows a read touches spread over the banks
-static constexpr uint32_t kAttTile = kAttD * kAttPitch;
-static constexpr size_t kAttLds = 5 * (size_t)kAttTile;  // Q, two K blocks, two V blocks
+// Row pitches in bytes, chosen so that the rows one LDS pass touches fall into different banks.  Q and K are read by
+// transpose reads, 32 lanes = eight consecutive rows of 32 bytes per pass: 160-byte rows put them at bank offsets
+// 0, 40, 16, 56, 32, 8, 48, 24 (of 64 four-byte banks), each eight banks wide.  V is read eight bytes per lane from
+// sixteen consecutive rows: 144-byte rows put those at sixteen different multiples of four banks.
+static constexpr uint32_t kAttPitchK = 64 * 2 + 32;
+static constexpr uint32_t kAttPitchV = 64 * 2 + 16;
+static constexpr uint32_t kAttTileK = kAttD * kAttPitchK, kAttTileV = kAttD * kAttPitchV;
+static constexpr size_t kAttLds = 3 * (size_t)kAttTileK + 2 * (size_t)kAttTileV;  // Q, two K blocks, two V blocks
 static constexpr int kAttMaxSeq = 16384;
 
 union AttOperand {
@@ -199,19 +204,24 @@ struct AttentionArgs {
   const _Float16 *q, *k, *v;
   _Float16 *out;
   long long ld, ld_out;  // elements between consecutive features
-  int S, heads;
+  int S, heads, units;  // units = batch elements x heads
   float scale_log2e;
 };
 
 __global__ __launch_bounds__(kAttThreads, 3) void attention_fm_kernel(const AttentionArgs p) {
   __shared__ __align__(16) unsigned char lds[kAttLds];
   const int S = p.S, qblocks = S / kAttQueries, blocks = S / kAttKeys;
-  const int qb = blockIdx.x % qblocks, head = (blockIdx.x / qblocks) % p.heads, b = blockIdx.x / (qblocks * p.heads);
+  // Workgroup ids go round-robin to the 8 XCDs, each with its own L2: the query blocks of one (batch element, head)
+  // take ids 8 apart, so that the head's K and V are fetched from memory once and found in that L2 by the others.
+  const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+  const int qb = idx % qblocks, unit = (idx / qblocks) * 8 + xcd;
+  if (unit >= p.units) return;  // (the grid is padded to a multiple of eight units)
+  const int head = unit % p.heads, b = unit / p.heads;
   const int tid = threadIdx.x, lane = tid & 63, m = lane & 15, g = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   unsigned char *const q_tile = lds;
-  unsigned char *const k_tiles = lds + kAttTile;      // buffer i at k_tiles + i * kAttTile
-  unsigned char *const v_tiles = lds + 3 * kAttTile;
+  unsigned char *const k_tiles = lds + kAttTileK;      // buffer i at k_tiles + i * kAttTileK
+  unsigned char *const v_tiles = lds + 3 * kAttTileK;  // buffer i at v_tiles + i * kAttTileV
   const long long tok0 = (long long)b * S;
   const _Float16 *qg = p.q + (long long)(head * kAttD) * p.ld + tok0 + qb * kAttQueries;
   const _Float16 *kg = p.k + (long long)(head * kAttD) * p.ld + tok0;
@@ -220,7 +230,8 @@ __global__ __launch_bounds__(kAttThreads, 3) void attention_fm_kernel(const Atte
   // A 64 x 64 fp16 tile is 512 pieces of 16 bytes, two per thread: rows r0 and r0 + 32, piece pc.
   const int r0 = tid >> 3, pc = tid & 7;
   const long long g0 = (long long)r0 * p.ld + pc * 8, g1 = g0 + 32 * p.ld;
-  const uint32_t l0 = r0 * kAttPitch + pc * 16, l1 = l0 + 32 * kAttPitch;
+  const uint32_t l0 = r0 * kAttPitchK + pc * 16, l1 = l0 + 32 * kAttPitchK;    // in a Q or K tile
+  const uint32_t lv0 = r0 * kAttPitchV + pc * 16, lv1 = lv0 + 32 * kAttPitchV;  // in a V tile
   uintx4 kk[2], vv[2];
   kk[0] = *reinterpret_cast<const uintx4 *>(kg + g0);
   kk[1] = *reinterpret_cast<const uintx4 *>(kg + g1);
@@ -230,29 +241,38 @@ __global__ __launch_bounds__(kAttThreads, 3) void attention_fm_kernel(const Atte
   *reinterpret_cast<uintx4 *>(q_tile + l1) = *reinterpret_cast<const uintx4 *>(qg + g1);
   *reinterpret_cast<uintx4 *>(k_tiles + l0) = kk[0];
   *reinterpret_cast<uintx4 *>(k_tiles + l1) = kk[1];
-  *reinterpret_cast<uintx4 *>(v_tiles + l0) = vv[0];
-  *reinterpret_cast<uintx4 *>(v_tiles + l1) = vv[1];
+  *reinterpret_cast<uintx4 *>(v_tiles + lv0) = vv[0];
+  *reinterpret_cast<uintx4 *>(v_tiles + lv1) = vv[1];
   __syncthreads();
 
-  // ---- the wave's 16 queries as the first product's second operand: lane (m, g) holds features 32u + 8g .. + 7 of query m
-  AttOperand qop[2];
+  // ---- Wave w works on queries 32 * (w / 2) .. + 31 of the workgroup's 64 (two sets of 16) against keys
+  // 32 * (w % 2) .. + 31 of every block: an operand read of K or V then serves two products (the two query sets),
+  // which halves the LDS reads per product, and the two waves that share queries merge their softmax states at the end.
+  // The contraction slots of the first product are numbered so that a transpose read of 32 lanes touches eight
+  // consecutive rows: slots 0-3 of lane group g are features 32u + 4g .. + 3, slots 4-7 features 32u + 16 + 4g .. + 3
+  // (the same numbering for Q and K).
+  const int qhalf = wave >> 1, khalf = wave & 1;
+  AttOperand qop[2][2];  // [query set][u]: lane (m, g) holds its slots of query 32 * qhalf + 16 * set + m
 #pragma unroll
-  for (int u = 0; u < 2; ++u) {
-    const unsigned char *a = q_tile + (32 * u + 8 * g + (m >> 2)) * kAttPitch + (16 * wave) * 2 + (m & 3) * 8;
-    const uintx2 lo = att_read_tr(a), hi = att_read_tr(a + 4 * kAttPitch);
-    qop[u].u[0] = lo[0]; qop[u].u[1] = lo[1]; qop[u].u[2] = hi[0]; qop[u].u[3] = hi[1];
-  }
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const unsigned char *a = q_tile + (32 * u + 4 * g + (m >> 2)) * kAttPitchK + (32 * qhalf + 16 * j) * 2 + (m & 3) * 8;
+      const uintx2 lo = att_read_tr(a), hi = att_read_tr(a + 16 * kAttPitchK);
+      qop[j][u].u[0] = lo[0]; qop[j][u].u[1] = lo[1]; qop[j][u].u[2] = hi[0]; qop[j][u].u[3] = hi[1];
+    }
 
   const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
-  floatx4 o[4] = {zero, zero, zero, zero};  // lane (m, g): features 16dt + 4g .. + 3 of query m
-  // of query m: the largest raw score so far, and this lane's share of the sum of 2^((score - max) * scale_log2e)
-  float run_max = -3.0e38f, run_sum = 0.f;
+  floatx4 o[2][4] = {{zero, zero, zero, zero}, {zero, zero, zero, zero}};  // [set][dt], lane (m, g): features 16dt + 4g .. + 3 of query m
+  // per query set, of query m: the largest raw score so far, and this lane's share of the sum of
+  // 2^((score - max) * scale_log2e), over the keys of this wave
+  float run_max[2] = {-3.0e38f, -3.0e38f}, run_sum[2] = {0.f, 0.f};
   const float c = p.scale_log2e;  // > 0: the largest scaled score is the scaled largest score
-  const uint32_t k_rd = (8 * g + (m >> 2)) * kAttPitch + (m & 3) * 8;
-  const uint32_t v_rd = m * kAttPitch + (4 * g) * 2;
+  const uint32_t k_rd = (4 * g + (m >> 2)) * kAttPitchK + (m & 3) * 8 + (32 * khalf) * 2;
+  const uint32_t v_rd = m * kAttPitchV + (4 * g) * 2 + (32 * khalf) * 2;
   for (int kb = 0; kb < blocks; ++kb) {
-    const unsigned char *const k_tile = k_tiles + (kb & 1) * kAttTile;
-    const unsigned char *const v_tile = v_tiles + (kb & 1) * kAttTile;
+    const unsigned char *const k_tile = k_tiles + (kb & 1) * kAttTileK;
+    const unsigned char *const v_tile = v_tiles + (kb & 1) * kAttTileV;
     const bool more = kb + 1 < blocks;  // uniform
     if (more) {
       const int off = (kb + 1) * kAttKeys;
@@ -261,79 +281,108 @@ __global__ __launch_bounds__(kAttThreads, 3) void attention_fm_kernel(const Atte
       vv[0] = *reinterpret_cast<const uintx4 *>(vg + g0 + off);
       vv[1] = *reinterpret_cast<const uintx4 *>(vg + g1 + off);
     }
-    floatx4 s[4] = {zero, zero, zero, zero};  // lane (m, g): keys 16kt + 4g .. + 3 of the block against query m
+    // scores^T: s[set][kt], lane (m, g): keys 32 * khalf + 16kt + 4g .. + 3 of the block against query m of the set
+    floatx4 s[2][2] = {{zero, zero}, {zero, zero}};
 #pragma unroll
-    for (int kt = 0; kt < 4; ++kt) {
+    for (int kt = 0; kt < 2; ++kt) {
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
-        const unsigned char *a = k_tile + k_rd + (32 * u) * kAttPitch + (16 * kt) * 2;
-        const uintx2 lo = att_read_tr(a), hi = att_read_tr(a + 4 * kAttPitch);
+        const unsigned char *a = k_tile + k_rd + (32 * u) * kAttPitchK + (16 * kt) * 2;
+        const uintx2 lo = att_read_tr(a), hi = att_read_tr(a + 16 * kAttPitchK);
         AttOperand kop;
         kop.u[0] = lo[0]; kop.u[1] = lo[1]; kop.u[2] = hi[0]; kop.u[3] = hi[1];
-        s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kop.h, qop[u].h, s[kt], 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) s[j][kt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kop.h, qop[j][u].h, s[j][kt], 0, 0, 0);
       }
     }
-    float mx = s[0][0];
+    AttOperand pop[2];  // per set: contraction slots 0-3 = keys 4g .. + 3 of tile 0, slots 4-7 = the same keys of tile 1
 #pragma unroll
-    for (int kt = 0; kt < 4; ++kt)
+    for (int j = 0; j < 2; ++j) {
+      float mx = s[j][0][0];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[kt][r]);
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float new_max = fmaxf(run_max, mx);
-    const float alpha = __builtin_amdgcn_exp2f(fmaxf((run_max - new_max) * c, -126.0f));
-    run_max = new_max;
-    const float shift = -new_max * c;
-    float part = 0.f;
+      for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-    for (int kt = 0; kt < 4; ++kt)
+        for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[j][kt][r]);
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float new_max = fmaxf(run_max[j], mx);
+      const float alpha = __builtin_amdgcn_exp2f(fmaxf((run_max[j] - new_max) * c, -126.0f));
+      run_max[j] = new_max;
+      const float shift = -new_max * c;
+      float part = 0.f;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        s[kt][r] = __builtin_amdgcn_exp2f(fmaf(s[kt][r], c, shift));
-        part += s[kt][r];
-      }
-    run_sum = run_sum * alpha + part;
+      for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt) o[dt] *= alpha;
-    AttOperand pop[2];  // contraction slots 0-3 = keys 4g .. + 3 of tile 2t, slots 4-7 = the same keys of tile 2t + 1
+        for (int r = 0; r < 4; ++r) {
+          s[j][kt][r] = __builtin_amdgcn_exp2f(fmaf(s[j][kt][r], c, shift));
+          part += s[j][kt][r];
+        }
+      run_sum[j] = run_sum[j] * alpha + part;
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      pop[t].u[0] = att_pack(s[2 * t][0], s[2 * t][1]);
-      pop[t].u[1] = att_pack(s[2 * t][2], s[2 * t][3]);
-      pop[t].u[2] = att_pack(s[2 * t + 1][0], s[2 * t + 1][1]);
-      pop[t].u[3] = att_pack(s[2 * t + 1][2], s[2 * t + 1][3]);
+      for (int dt = 0; dt < 4; ++dt) o[j][dt] *= alpha;
+      pop[j].u[0] = att_pack(s[j][0][0], s[j][0][1]);
+      pop[j].u[1] = att_pack(s[j][0][2], s[j][0][3]);
+      pop[j].u[2] = att_pack(s[j][1][0], s[j][1][1]);
+      pop[j].u[3] = att_pack(s[j][1][2], s[j][1][3]);
     }
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt) {
+      const unsigned char *a = v_tile + v_rd + (16 * dt) * kAttPitchV;
+      const uintx2 lo = *reinterpret_cast<const uintx2 *>(a), hi = *reinterpret_cast<const uintx2 *>(a + 32);
+      AttOperand vop;
+      vop.u[0] = lo[0]; vop.u[1] = lo[1]; vop.u[2] = hi[0]; vop.u[3] = hi[1];
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        const unsigned char *a = v_tile + v_rd + (16 * dt) * kAttPitch + (32 * t) * 2;
-        const uintx2 lo = *reinterpret_cast<const uintx2 *>(a), hi = *reinterpret_cast<const uintx2 *>(a + 32);
-        AttOperand vop;
-        vop.u[0] = lo[0]; vop.u[1] = lo[1]; vop.u[2] = hi[0]; vop.u[3] = hi[1];
-        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vop.h, pop[t].h, o[dt], 0, 0, 0);
-      }
+      for (int j = 0; j < 2; ++j) o[j][dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vop.h, pop[j].h, o[j][dt], 0, 0, 0);
     }
     if (more) {  // the other buffer: every wave finished reading it before the barrier that ended the previous block
-      unsigned char *const kn = k_tiles + ((kb + 1) & 1) * kAttTile, *const vn = v_tiles + ((kb + 1) & 1) * kAttTile;
+      unsigned char *const kn = k_tiles + ((kb + 1) & 1) * kAttTileK, *const vn = v_tiles + ((kb + 1) & 1) * kAttTileV;
       *reinterpret_cast<uintx4 *>(kn + l0) = kk[0];
       *reinterpret_cast<uintx4 *>(kn + l1) = kk[1];
-      *reinterpret_cast<uintx4 *>(vn + l0) = vv[0];
-      *reinterpret_cast<uintx4 *>(vn + l1) = vv[1];
+      *reinterpret_cast<uintx4 *>(vn + lv0) = vv[0];
+      *reinterpret_cast<uintx4 *>(vn + lv1) = vv[1];
     }
     __syncthreads();
   }
-  run_sum += __shfl_xor(run_sum, 16, 64);
-  run_sum += __shfl_xor(run_sum, 32, 64);
-  const float inv = 1.0f / run_sum;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    run_sum[j] += __shfl_xor(run_sum[j], 16, 64);
+    run_sum[j] += __shfl_xor(run_sum[j], 32, 64);
+  }
 
-  // ---- the context through LDS (over the query tile: every wave read its queries before the first barrier of the
-  // loop) and out in whole lines
+  // ---- The two waves of a query half merge: the one with the upper keys leaves its state in LDS (over the K tiles:
+  // the loop's last barrier is behind every read of them), the other adds it to its own.
+  floatx4 *const xo = reinterpret_cast<floatx4 *>(k_tiles) + qhalf * (2 * 4 * 64);  // [set][dt][lane]
+  float *const xs = reinterpret_cast<float *>(k_tiles + 2 * (2 * 4 * 64) * 16) + qhalf * (2 * 2 * 64);  // [set][max, sum][lane]
+  if (khalf == 1) {
 #pragma unroll
-  for (int dt = 0; dt < 4; ++dt)
+    for (int j = 0; j < 2; ++j) {
 #pragma unroll
-    for (int r = 0; r < 4; ++r)
-      *reinterpret_cast<_Float16 *>(q_tile + (16 * dt + 4 * g + r) * kAttPitch + (16 * wave + m) * 2) = (_Float16)(o[dt][r] * inv);
+      for (int dt = 0; dt < 4; ++dt) xo[(j * 4 + dt) * 64 + lane] = o[j][dt];
+      xs[(j * 2 + 0) * 64 + lane] = run_max[j];
+      xs[(j * 2 + 1) * 64 + lane] = run_sum[j];
+    }
+  }
+  __syncthreads();
+  if (khalf == 0) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const float m1 = xs[(j * 2 + 0) * 64 + lane], l1 = xs[(j * 2 + 1) * 64 + lane];
+      const float mm = fmaxf(run_max[j], m1);
+      const float a0 = __builtin_amdgcn_exp2f(fmaxf((run_max[j] - mm) * c, -126.0f));
+      const float a1 = __builtin_amdgcn_exp2f(fmaxf((m1 - mm) * c, -126.0f));
+      const float inv = 1.0f / (run_sum[j] * a0 + l1 * a1);
+      // the context through LDS (over the query tile: every wave read its queries before the first barrier of the
+      // loop) and out in whole lines
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt) {
+        const floatx4 other = xo[(j * 4 + dt) * 64 + lane];
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          *reinterpret_cast<_Float16 *>(q_tile + (16 * dt + 4 * g + r) * kAttPitchK + (32 * qhalf + 16 * j + m) * 2) =
+              (_Float16)((o[j][dt][r] * a0 + other[r] * a1) * inv);
+      }
+    }
+  }
   __syncthreads();
   _Float16 *og = p.out + (long long)(head * kAttD) * p.ld_out + tok0 + qb * kAttQueries;
   *reinterpret_cast<uintx4 *>(og + (long long)r0 * p.ld_out + pc * 8) = *reinterpret_cast<const uintx4 *>(q_tile + l0);
@@ -345,7 +394,7 @@ bool attention_fm_applies(int batch, int heads, int seq, int head_dim, const voi
   const auto aligned = [](const void *x) { return (reinterpret_cast<uintptr_t>(x) & 15u) == 0; };
   return batch > 0 && heads > 0 && head_dim == kAttD && seq >= kAttQueries && seq % kAttQueries == 0 && seq <= kAttMaxSeq &&
          ld % 8 == 0 && ld_out % 8 == 0 && aligned(q) && aligned(k) && aligned(v) && aligned(out) &&
-         (long long)batch * heads * (seq / kAttQueries) <= 0x7fffffffLL;
+         ((long long)batch * heads + 7) * (seq / kAttQueries) <= 0x7fffffffLL;
 }
 
 hipError_t launch_attention_fm(int batch, int heads, int seq, const uint16_t *q, const uint16_t *k, const uint16_t *v,
@@ -359,8 +408,10 @@ hipError_t launch_attention_fm(int batch, int heads, int seq, const uint16_t *q,
   a.ld_out = ld_out;
   a.S = seq;
   a.heads = heads;
+  a.units = batch * heads;
   a.scale_log2e = scale * 1.4426950408889634f;
-  const unsigned blocks = (unsigned)((long long)batch * heads * (seq / kAttQueries));
+  const long long units_padded = (((long long)batch * heads + 7) / 8) * 8;
+  const unsigned blocks = (unsigned)(units_padded * (seq / kAttQueries));
   hipLaunchKernelGGL(attention_fm_kernel, dim3(blocks), dim3(kAttThreads), 0, stream, a);
   return hipGetLastError();
 }

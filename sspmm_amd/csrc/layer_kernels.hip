@@ -305,10 +305,19 @@ __global__ __launch_bounds__(kAttThreads, 3) void attention_fm_kernel(const Atte
         for (int r = 0; r < 4; ++r) mx = fmaxf(mx, s[j][kt][r]);
       mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      // The reference point of the exponentials moves only when some query's maximum has grown by more than 8 in
+      // the base-2 domain (a wave-uniform decision): until then the probabilities are at most 2^8 times too large,
+      // which fp16 holds, the running sums and the context stay consistent with the old reference point, and the
+      // rescaling of the accumulators, which after the first block is nearly always by 1, is skipped.
       const float new_max = fmaxf(run_max[j], mx);
-      const float alpha = __builtin_amdgcn_exp2f(fmaxf((run_max[j] - new_max) * c, -126.0f));
-      run_max[j] = new_max;
-      const float shift = -new_max * c;
+      if (__ballot((new_max - run_max[j]) * c > 8.0f) != 0) {
+        const float alpha = __builtin_amdgcn_exp2f(fmaxf((run_max[j] - new_max) * c, -126.0f));
+        run_max[j] = new_max;
+        run_sum[j] *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) o[j][dt] *= alpha;
+      }
+      const float shift = -run_max[j] * c;
       float part = 0.f;
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
@@ -317,9 +326,7 @@ __global__ __launch_bounds__(kAttThreads, 3) void attention_fm_kernel(const Atte
           s[j][kt][r] = __builtin_amdgcn_exp2f(fmaf(s[j][kt][r], c, shift));
           part += s[j][kt][r];
         }
-      run_sum[j] = run_sum[j] * alpha + part;
-#pragma unroll
-      for (int dt = 0; dt < 4; ++dt) o[j][dt] *= alpha;
+      run_sum[j] += part;
       pop[j].u[0] = att_pack(s[j][0][0], s[j][0][1]);
       pop[j].u[1] = att_pack(s[j][0][2], s[j][0][3]);
       pop[j].u[2] = att_pack(s[j][1][0], s[j][1][1]);

@@ -116,6 +116,25 @@ def test_feature_major_attention_matches_fp32_attention(built_library, batch, he
     assert torch.all(out[:, T:] == 7.0)
 
 
+def test_feature_major_attention_with_maxima_that_keep_growing(built_library):
+    """Keys whose norm grows along the sequence: the running maximum of a query's scores rises by many units from one
+    block of keys to the next, so the kernel moves the reference point of its exponentials again and again (it
+    skips that step while the maximum grows by little)."""
+    from sspmm_amd.layers import attention_fm
+    batch, heads, seq = 2, 2, 512
+    hidden, T = heads * 64, batch * seq
+    g = torch.Generator("cuda").manual_seed(11)
+    qkv = torch.randn(3 * hidden, T, device="cuda", generator=g)
+    growth = 1.0 + 7.0 * (torch.arange(T, device="cuda") % seq).float() / seq
+    qkv[hidden:2 * hidden] *= growth
+    qkv[:hidden] = qkv[:hidden].abs() * 2.0   # same-sign queries and keys of growing size: scores rise with the position
+    qkv[hidden:2 * hidden] = qkv[hidden:2 * hidden].abs()
+    qkv = qkv.half()
+    got = attention_fm(qkv, hidden, heads, batch, seq)
+    want = _attention_reference(qkv[:hidden], qkv[hidden:2 * hidden], qkv[2 * hidden:], batch, heads, seq, 0.125)
+    assert (got.float() - want).abs().max().item() <= 2e-3 * max(1.0, want.abs().max().item())
+
+
 def test_feature_major_attention_rejects_what_it_does_not_cover(built_library):
     from sspmm_amd import _lib
     L = _lib.lib()

@@ -281,6 +281,13 @@ def single_launch_cases(batch):
         for s in (0.7, 0.9, 0.98):
             cases["cfg2_%dx%d_v8_s%g_n256" % (M, K, s)] = dict(M=M, K=K, V=8, sparsity=s, N=256, batch=1, out_f32=True,
                                                                std=0.02, seed=2)
+    # the other points of cfg2's grid as batched launches (the headline is 2048x512 at 0.9): where the format stops
+    # paying against the dense GEMM shows here, not in the latency-bound single products
+    for (M, K) in ((2048, 512), (512, 2048)):
+        for s in (0.7, 0.9, 0.98):
+            if (M, K, s) != (2048, 512, 0.9):
+                cases["cfg2_%dx%d_v8_s%g_batched" % (M, K, s)] = dict(M=M, K=K, V=8, sparsity=s, N=256, batch=batch,
+                                                                      out_f32=True, std=0.02, seed=2)
     cases["cfg2_batched_fp16_out"] = dict(M=2048, K=512, V=8, sparsity=0.9, N=256, batch=batch, out_f32=False, std=0.02, seed=2)
     cases["cfg2_shape_v16_batched"] = dict(M=2048, K=512, V=16, sparsity=0.9, N=256, batch=batch, out_f32=True, std=0.02, seed=2)
     cases["cfg2_shape_v16_batched_fp16_out"] = dict(M=2048, K=512, V=16, sparsity=0.9, N=256, batch=batch, out_f32=False,

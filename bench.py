@@ -51,7 +51,7 @@ MEASURED_TRAFFIC = {
                                "alg_bytes": 6866100, "source": "profiles/svc_kernels_cfg4_zipf_v8_counters.txt"},
 }
 KERNEL_NAMES = {1: "spmm_generic_kernel", 2: "spmm_gather_kernel", 3: "spmm_slab_kernel<*,4>", 4: "spmm_gather_split_kernel",
-                5: "spmm_slab_kernel<*,2>", 6: "spmm_stage_kernel", 7: "spmm_balanced_kernel"}
+                5: "spmm_slab_kernel<*,2>", 6: "spmm_stage_kernel", 7: "spmm_balanced_kernel", 9: "spmm_slab_kernel<*,8>"}
 
 
 def parse_args():
@@ -72,7 +72,7 @@ def parse_args():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy (its hardware-counter readings calibrate FETCH_SIZE / "
                          "WRITE_SIZE when the run is profiled)")
-    ap.add_argument("--kernel", choices=["auto", "generic", "gather", "slab"], default="auto",
+    ap.add_argument("--kernel", choices=["auto", "generic", "gather", "slab", "slab128"], default="auto",
                     help="force one SpMM kernel (tuning); the default lets the library choose")
     return ap.parse_args()
 
@@ -710,7 +710,7 @@ def main():
     import sspmm_amd
     L = _lib.lib()
     torch.cuda.set_device(0)
-    L.sspmm_select_kernel({"auto": 0, "generic": 1, "gather": 2, "slab": 3}[args.kernel])
+    L.sspmm_select_kernel({"auto": 0, "generic": 1, "gather": 2, "slab": 3, "slab128": 9}[args.kernel])
     env = {"L": L, "torch": torch, "synth": synth, "sspmm_amd": sspmm_amd, "O": None, "st": args.steps, "wu": args.warmup,
            "batch": args.batch}
     if args.calibrate_copy:

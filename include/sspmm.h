@@ -34,7 +34,9 @@ int sspmm_version(void);
  * its preconditions hold.  0 = automatic choice (default), 1 = scalar kernel (any shape),
  * 2 = one-wave gather kernel, 3 = LDS-slab kernel, 6 = the gather kernel's staged form (rows of B
  * fetched whole and passed through LDS; the automatic choice takes it for N <= 64 only) on any
- * width, 7 = the load-balanced gather kernel (products with a plan only; others ignore it).  The setting belongs to the calling host thread (other threads keep the automatic choice).
+ * width, 7 = the load-balanced gather kernel (products with a plan only; others ignore it), 9 = the
+ * LDS-slab kernel with 128-column slabs (K up to about 570).  The setting belongs to the calling host thread
+ * (other threads keep the automatic choice).
  * Returns the previous setting, or -1 for an unknown value.
  */
 int sspmm_select_kernel(int which);
@@ -44,7 +46,7 @@ int sspmm_select_kernel(int which);
  * K > 4096 that splits long vector-rows over the waves of a workgroup (selected as 2) and
  * 5 = the LDS-slab kernel with 32-column slabs, for K too tall for 64-column ones (selected
  * as 3); the staged gather kernel reports 6 also where it was chosen automatically, the load-balanced
- * kernel 7; 0 before any
+ * kernel 7, the LDS-slab kernel with 128-column slabs 9 (chosen for fp16 outputs and dense patterns); 0 before any
  * call of this thread. */
 int sspmm_last_kernel(void);
 

@@ -69,7 +69,7 @@ extern "C" {
 int sspmm_version(void) { return (0 << 16) | 1; }
 
 int sspmm_select_kernel(int which) {
-  if (which < 0 || (which > 3 && which != 6 && which != 7)) return -1;
+  if (which < 0 || (which > 3 && which != 6 && which != 7 && which != 9)) return -1;
   return sspmm::set_kernel_override(which);
 }
 

@@ -35,7 +35,7 @@ struct SpmmArgs {
 hipError_t launch_spmm(const SpmmArgs &args, int V, bool out_f16, hipStream_t stream);
 
 // Forces a kernel where its preconditions hold: 0 automatic, 1 scalar, 2 gather, 3 LDS slab, 6 staged gather,
-// 7 load-balanced gather (calls with a plan only).
+// 7 load-balanced gather (calls with a plan only), 9 LDS slab 128 columns wide.
 // Per host thread: meant for tests and tuning.  Returns the previous value.
 int set_kernel_override(int which);
 // Kernel the latest launch_spmm of the calling thread used (1 scalar, 2 gather, 3 LDS slab; 0 before any launch).

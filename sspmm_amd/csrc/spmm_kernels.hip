@@ -576,7 +576,7 @@ __global__ __launch_bounds__(64 * kSplitWaves) void spmm_gather_split_kernel(con
 static constexpr int kSlabWaves = 16;
 static constexpr int kSlabThreads = kSlabWaves * 64;
 // A slab is NQ tiles of 16 columns wide: 4 (64 columns, 128-byte rows) where K lets it fit in LDS, 2 (32 columns,
-// 64-byte rows) for matrices up to twice as tall.
+// 64-byte rows) for matrices up to twice as tall, 8 (128 columns, 256-byte rows, one buffer) for K up to about 570.
 static constexpr int slab_row_bytes(int NQ) { return 32 * NQ; }
 // How a 64-column slab lies in LDS.  With 128-byte rows the 32-byte segments of a row are XOR-swizzled (see
 // slab_unit_dst) and every read address needs the swizzle applied in registers; where LDS allows, rows are padded
@@ -799,6 +799,21 @@ struct SlabStore<V, _Float16, 4> {
   }
 };
 
+// fp16 with a 128-column slab: two 64-column halves.
+template <int V>
+struct SlabStore<V, _Float16, 8> {
+  SlabStore<V, _Float16, 4> half_lo, half_hi;
+  __device__ __forceinline__ void init(int lane, int n0, int N) {
+    half_lo.init(lane, n0, N);
+    half_hi.init(lane, n0 + 64, N);
+  }
+  __device__ __forceinline__ void store(const floatx4 (&acc)[8], __amdgpu_buffer_rsrc_t srd, uint32_t crow) const {
+    const floatx4 a[4] = {acc[0], acc[1], acc[2], acc[3]}, b[4] = {acc[4], acc[5], acc[6], acc[7]};
+    half_lo.store(a, srd, crow);
+    half_hi.store(b, srd, crow);
+  }
+};
+
 // fp16 with a 32-column slab: after the swap a lane owns eight consecutive columns of row m, four lanes make a
 // row's 64 bytes, and one instruction writes the V rows (with V = 8 the lanes m >= 8 have nothing to write).
 template <int V>
@@ -897,6 +912,7 @@ __device__ __forceinline__ void slab_process_item(const SlabCtx<V, OutT> &x, uns
         const uint32_t c = ((int)x.slot0 + 4 * h < left) ? ld[cur].col[h] : x.zero_row;
         // row c of the slab, and the swizzle of its 32-byte segments (see slab_unit_dst)
         addr[h] = layout_pad(L) ? __umul24(c, layout_row_bytes(L, NQ)) + lane_base
+                  : NQ == 8     ? (((c << 8) + lane_base) | ((c << 5) & 0xe0u))
                   : NQ == 4     ? (((c << 7) + lane_base) | ((c << 4) & 0x60u))
                                 : (((c << 6) + lane_base) | ((c << 3) & 0x20u));
       }
@@ -964,14 +980,14 @@ __device__ __forceinline__ uint32_t slab_unit_src(const SpmmArgs &p, uint32_t u,
   return (u < units && col < (uint32_t)p.N) ? __umul24(u / kPerRow, (uint32_t)p.N * 2u) + col * 2u : b_bytes;  // b_bytes: out of bounds, reads zeros
 }
 // A 16-lane group of a slab read touches four rows at the same segment; rows 256 bytes apart share banks, so the
-// segment index is XORed with the row bits above that distance: (c >> 1) & 3 for 128-byte rows, (c >> 2) & 1 for
-// 64-byte rows.  Rows then collide only when they agree modulo 8.
+// segment index is XORed with the row bits above that distance: c & 7 for 256-byte rows, (c >> 1) & 3 for 128-byte
+// rows, (c >> 2) & 1 for 64-byte rows.  Rows then collide only when they agree modulo 8.
 template <int NQ, int L>
 __device__ __forceinline__ uint32_t slab_unit_dst(uint32_t u) {
   constexpr uint32_t kPerRow = 2u * NQ;
   const uint32_t c = u / kPerRow;
   if (layout_pad(L)) return c * layout_row_bytes(L, NQ) + (u % kPerRow) * 16u;
-  const uint32_t swz = NQ == 4 ? ((c >> 1) & 3u) : ((c >> 2) & 1u);
+  const uint32_t swz = NQ == 8 ? (c & 7u) : NQ == 4 ? ((c >> 1) & 3u) : ((c >> 2) & 1u);
   return c * slab_row_bytes(NQ) + (((u % kPerRow) * 16u) ^ (swz << 5));
 }
 
@@ -993,7 +1009,7 @@ template <int V, typename OutT, int L, int NQ>
 __global__ __launch_bounds__(kSlabThreads) void spmm_slab_kernel(const SpmmArgs p,
                                                                  const int32_t *__restrict__ row_offsets,
                                                                  const int32_t *__restrict__ row_indices) {
-  extern __shared__ __align__(128) unsigned char lds[];
+  extern __shared__ __align__(256) unsigned char lds[];
   // The hardware deals consecutive workgroup ids round-robin to the 8 XCDs, each with its own L2.
   const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3, wgs_per_xcd = gridDim.x >> 3;
   const uint32_t slabs_x = p.group_by_batch ? (((uint32_t)p.batch + 7u - xcd) / 8u) * p.n_tiles : (p.n_slabs + 7u - xcd) / 8u;
@@ -1569,7 +1585,7 @@ static hipError_t launch_slab(const SpmmArgs &a, hipStream_t stream) {
   const bool can_dbl = (uint32_t)a.K * (2u * NQ) <= (uint32_t)kSlabFetchUnits * kSlabThreads;
   int layout = kXorSingle;
   if (NQ == 4 && can_dbl && slab_lds_bytes(a.K, V, rows, kPadDouble, NQ) <= kSlabLds) layout = kPadDouble;
-  else if (can_dbl && slab_lds_bytes(a.K, V, rows, kXorDouble, NQ) <= kSlabLds) layout = kXorDouble;
+  else if (NQ != 8 && can_dbl && slab_lds_bytes(a.K, V, rows, kXorDouble, NQ) <= kSlabLds) layout = kXorDouble;
   else if (NQ == 4 && slab_lds_bytes(a.K, V, rows, kPadSingle, NQ) <= kSlabLds) layout = kPadSingle;
   while (layout == kXorSingle && slab_lds_bytes(a.K, V, rows, kXorSingle, NQ) > kSlabLds && rows > kSlabMinRows)
     rows = (rows + 1u) / 2u;  // smaller tables for a tall slab
@@ -1581,7 +1597,8 @@ static hipError_t launch_slab(const SpmmArgs &a, hipStream_t stream) {
     if (layout == kPadDouble) return launch_slab_kernel<V, OutT, kPadDouble, 4>(p, grid, lds, stream);
     if (layout == kPadSingle) return launch_slab_kernel<V, OutT, kPadSingle, 4>(p, grid, lds, stream);
   }
-  return layout == kXorDouble ? launch_slab_kernel<V, OutT, kXorDouble, NQ>(p, grid, lds, stream)
+  if (NQ == 8) return launch_slab_kernel<V, OutT, kXorSingle, NQ>(p, grid, lds, stream);  // (128-column slabs: one buffer)
+  return layout == kXorDouble ? launch_slab_kernel<V, OutT, kXorDouble, NQ == 8 ? 4 : NQ>(p, grid, lds, stream)
                               : launch_slab_kernel<V, OutT, kXorSingle, NQ>(p, grid, lds, stream);
 }
 
@@ -1590,6 +1607,7 @@ static hipError_t launch_v(const SpmmArgs &a, int which, hipStream_t stream) {
   SpmmArgs p = a;
   if (which == 3) return launch_slab<V, OutT, 4>(a, stream);
   if (which == 5) return launch_slab<V, OutT, 2>(a, stream);
+  if (which == 9) return launch_slab<V, OutT, 8>(a, stream);
   if (which == 2) {
     p.n_tiles = (uint32_t)((a.N + 127) / 128);
     p.total_work = (uint32_t)a.m_vec * p.n_tiles * (uint32_t)a.batch;
@@ -1728,8 +1746,16 @@ hipError_t launch_spmm(const SpmmArgs &a, int V, bool out_f16, hipStream_t strea
     // table entry, store set-up) outweighs it, and the gather kernels win (measured at 95 and 98 % sparsity up to 32
     // vectors per row: 1.13-1.18x; with V = 8 the two tie, and between the gather kernels the density changes nothing).
     if (which == 3 && !out_f16 && V == 16 && a.mean_row_vectors > 0 && a.mean_row_vectors <= 32) which = 2;
+    // Slabs 128 columns wide where they fit (K up to about 570, one buffer): a step then feeds eight MFMAs, and the
+    // work around them (cursor, loads, value tile, addresses) is spent once per 128 columns.  Measured on K = 256 and
+    // 512: 4-13 % on fp16 outputs from two such column tiles on, 7-15 % at 70 % sparsity whatever the output; level
+    // on fp32 outputs at 90 % and above (there the stores bound the kernel), where the double-buffered 64-column slab stays.
+    const bool wide_ok = which == 3 && slab_fits(a.K, V, 8) && a.N >= 192;
+    const bool dense_known = a.mean_row_vectors > 0 && (int64_t)a.mean_row_vectors * 5 >= (int64_t)a.K;  // 20 % and denser
+    if (wide_ok && (out_f16 || dense_known)) which = 9;
     if (g_kernel_override == 2 || g_kernel_override == 6) which = 2;
     if (g_kernel_override == 3 && slab_ok) which = 3;
+    if (g_kernel_override == 9 && slab_fits(a.K, V, 8) && c_ok && a.m_vec >= 64) which = 9;
     if (g_kernel_override == 3 && narrow_ok) which = 5;
     if (a.bias != nullptr || a.act != 0) which = 2;  // the kernels that apply the linear-layer epilogue
   }

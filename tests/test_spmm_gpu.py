@@ -102,7 +102,7 @@ def test_headline_batch_128_every_element(oracle, built_library, out_dtype):
     print("headline batch %d out=%s" % (batch, out_dtype), flush=True)
     out = sspmm_amd.bspmm(None, dev(vs.row_offsets), dev(vs.col_idx), vals, B, V, out_dtype=out_dtype)
     torch.cuda.synchronize()
-    assert _lib.lib().sspmm_last_kernel() == 3
+    assert _lib.lib().sspmm_last_kernel() == (3 if out_dtype == torch.float32 else 9)  # (fp16 C: 128-column slabs)
     out, vals_h, B_h = out.cpu().numpy(), vals.cpu().numpy(), B.cpu().numpy()
     tol = TIGHT_F32 if out_dtype == torch.float32 else TIGHT_F16
     for b in range(batch):
@@ -482,3 +482,67 @@ def test_probe_gather_runs_and_leaves_its_sink_alone(built_library):
     assert rc == 0
     torch.cuda.synchronize()
     assert torch.all(sink == 123)
+
+
+@pytest.mark.parametrize("V", [8, 16])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
+@pytest.mark.parametrize("N", [128, 136, 200, 256, 520])
+def test_wide_slab_kernel(oracle, built_library, V, out_dtype, N):
+    """The 128-column slab: column tails inside the first and the second half of a slab, ragged and empty rows,
+    unsorted columns, row_indices, a batch whose row blocks share slabs, and the automatic choice for fp16 outputs."""
+    from sspmm_amd import _lib
+    L = _lib.lib()
+    rng = np.random.default_rng(700 + V + N)
+    K, m_vec = 512, 150
+    lens = rng.integers(0, 90, m_vec)
+    lens[[0, 9, 33, 149]] = [0, 512, 31, 33]
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cols = np.concatenate([rng.permutation(K)[:n] for n in lens]).astype(np.int32)
+    vs = synth.VectorSparse(m_vec * V, K, V, m_vec, off, cols,
+                            (rng.standard_normal(cols.size * V) * 0.1).astype(np.float16), cols.size * V)
+    B = synth.dense_rhs(K, N, seed=N)
+    L.sspmm_select_kernel(9)
+    try:
+        got, _ = check(oracle, vs, B, out_dtype)
+        assert L.sspmm_last_kernel() == 9
+        assert not got[:V].any()
+        perm = rng.permutation(m_vec).astype(np.int32)
+        assert np.array_equal(run(vs, B, out_dtype, dev(perm)), got)
+        vals9 = (rng.standard_normal((9, cols.size * V)) * 0.1).astype(np.float16)
+        B9 = np.stack([synth.dense_rhs(K, N, seed=40 + b) for b in range(9)])
+        out = sspmm_amd.bspmm(None, dev(vs.row_offsets), dev(vs.col_idx), dev(vals9), dev(B9), V, out_dtype=out_dtype)
+        torch.cuda.synchronize()
+        assert L.sspmm_last_kernel() == 9
+        for b in range(9):
+            want = oracle.spmm(vs.m_vec, V, N, K, vs.row_offsets, vs.col_idx, vals9[b], B9[b], threads=8)
+            assert max_rel_err(out[b].cpu().numpy(), want) <= (TIGHT_F32 if out_dtype == torch.float32 else TIGHT_F16)
+    finally:
+        L.sspmm_select_kernel(0)
+    # K beyond what a 128-column slab leaves room for: the forced choice is ignored
+    tall = synth.vector_sparse(80 * V, 700, V, 0.9, seed=5)
+    L.sspmm_select_kernel(9)
+    try:
+        check(oracle, tall, synth.dense_rhs(700, 256, seed=6), out_dtype)
+        assert L.sspmm_last_kernel() != 9
+    finally:
+        L.sspmm_select_kernel(0)
+
+
+def test_wide_slab_is_the_choice_for_fp16_outputs_of_large_batches(oracle, built_library):
+    from sspmm_amd import _lib
+    L = _lib.lib()
+    V, K, N, batch = 8, 512, 256, 64
+    vs = synth.vector_sparse(2048, K, V, 0.9, seed=2, std=0.02)
+    g = torch.Generator("cuda").manual_seed(1)
+    vals = (torch.randn(batch, vs.col_idx.size * V, device="cuda", generator=g) * 0.02).half()
+    B = torch.randn(batch, K, N, device="cuda", generator=g).half()
+    ro, ci = dev(vs.row_offsets), dev(vs.col_idx)
+    out16 = sspmm_amd.bspmm(None, ro, ci, vals, B, V, out_dtype=torch.float16)
+    assert L.sspmm_last_kernel() == 9
+    out32 = sspmm_amd.bspmm(None, ro, ci, vals, B, V, out_dtype=torch.float32)
+    assert L.sspmm_last_kernel() == 3
+    torch.cuda.synchronize()
+    for b in (0, 7, 8, 63):
+        want = oracle.spmm(vs.m_vec, V, N, K, vs.row_offsets, vs.col_idx, vals[b].cpu().numpy(), B[b].cpu().numpy(), threads=8)
+        assert max_rel_err(out16[b].cpu().numpy(), want) <= TIGHT_F16
+        assert max_rel_err(out32[b].cpu().numpy(), want) <= TIGHT_F32

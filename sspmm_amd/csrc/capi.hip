@@ -279,6 +279,7 @@ static int svc_args(int M, int K, int V, const int32_t *row_ptr, const int32_t *
   a->M = M;
   a->K = K;
   a->V = V;
+  a->nnz = nnz;
   a->row_ptr = row_ptr;
   a->col_ind = col_ind;
   a->tmp_cols = reinterpret_cast<int32_t *>(w);

@@ -126,8 +126,15 @@ static hipError_t launch_ln(int H, int T, const uint16_t *x, const uint16_t *a, 
   const size_t lds = (size_t)H * TOK * 2 + (size_t)(THREADS / 64) * (TOK / 4) * 16;
   auto kern = add_layernorm_kernel<TOK, THREADS, TRIP, NT>;
   if (lds > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return e;
+    // the runtime is told once per device and size
+    static int raised[16] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) dev = -1;
+    if (dev < 0 || raised[dev] < (int)lds) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) return e;
+      if (dev >= 0) raised[dev] = (int)lds;
+    }
   }
   const int line_groups = (T + 63) / 64;
   const int blocks = ((line_groups + 7) / 8) * 8 * (64 / TOK);

@@ -10,6 +10,7 @@ namespace sspmm {
 
 struct SvcArgs {
   int M, K, V;
+  long long nnz;                 // entries of col_ind
   const int32_t *row_ptr;
   const int32_t *col_ind;
   int32_t *vec_row_ptr;          // svc_count output

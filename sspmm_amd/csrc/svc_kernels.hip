@@ -222,12 +222,34 @@ __global__ __launch_bounds__(THREADS) void svc_count_distinct_kernel(const SvcAr
   if (threadIdx.x == 0) a.vec_row_ptr[grp + 1] = total;
 }
 
+// The first entries of a group's member rows, fetched once: lane j of every wave holds the start of member row j
+// (the end of the last row behind them), and a uniform index reads it back without touching memory again.
+// Groups of 64 rows, one boundary more than a wave has lanes, read the row pointer each time.
+struct RowBounds {
+  const int32_t *row_ptr;
+  int r0, count;  // first row, number of rows
+  int mine;
+  bool in_lanes;
+  __device__ __forceinline__ RowBounds(const SvcArgs &a, int first, int last) : row_ptr(a.row_ptr), r0(first), count(last - first) {
+    in_lanes = count < 64;
+    mine = a.row_ptr[first + min((int)(threadIdx.x & 63), count)];
+  }
+  __device__ __forceinline__ int start(int j) const {  // j uniform, 0 .. count
+    return in_lanes ? __builtin_amdgcn_readlane(mine, j) : row_ptr[r0 + j];
+  }
+  __device__ __forceinline__ int row_of(int idx) const {  // member row (0-based) of entry idx of the group
+    int r = 0;
+    for (int j = 1; j < count; ++j) r += idx >= start(j) ? 1 : 0;
+    return r;
+  }
+};
+
 // Direct mode: a group's ordered columns and value vectors go to their final place.  list[0 .. n) are the
 // ordered columns; position_of(column) is the column's index in that list.  The group owns
 // scanned[grp + 1] - scanned[grp] vectors; n equals that count unless a CSR row repeats a column (invalid
 // input), in which case surplus vectors stay zero with column 0.
 template <int THREADS, typename PositionOf>
-__device__ __forceinline__ void write_group_output(const SvcArgs &a, int grp, int r0, int r1, const int *list, int n,
+__device__ __forceinline__ void write_group_output(const SvcArgs &a, int grp, const RowBounds &rows, const int *list, int n,
                                                    PositionOf position_of) {
   const int v0 = a.scanned[grp], n_out = a.scanned[grp + 1] - v0;
   if (a.vec_col)
@@ -248,13 +270,15 @@ __device__ __forceinline__ void write_group_output(const SvcArgs &a, int grp, in
   }
   __syncthreads();
   if (n == 0) return;
-  for (int r = r0; r < r1; ++r) {
-    const int b = a.row_ptr[r], e = a.row_ptr[r + 1];
-    for (int idx = b + (int)threadIdx.x; idx < e; idx += THREADS) {
-      const uint32_t c = (uint32_t)a.col_ind[idx];
-      const int p = c < (uint32_t)a.K ? position_of(c) : -1;
-      if (p >= 0 && p < n_out) out[(int64_t)p * a.V + (r - r0)] = a.csr_val[idx];
-    }
+  // the member rows' entries are one contiguous run of the CSR arrays: one pass over it, the row found from the
+  // boundaries in registers, so that no load waits for another
+  const int e_end = rows.start(rows.count);
+  for (int idx = rows.start(0) + (int)threadIdx.x; idx < e_end; idx += THREADS) {
+    const uint32_t c = (uint32_t)a.col_ind[idx];
+    const uint16_t value = a.csr_val[idx];
+    const int r = rows.row_of(idx);
+    const int p = c < (uint32_t)a.K ? position_of(c) : -1;
+    if (p >= 0 && p < n_out) out[(int64_t)p * a.V + r] = value;
   }
 }
 
@@ -310,7 +334,7 @@ __global__ __launch_bounds__(THREADS) void svc_merge_cpython_kernel(const SvcArg
   }
 
   if (listed) {
-    write_group_output<THREADS>(a, grp, r0, r1, list, n, [&](uint32_t key) {
+    write_group_output<THREADS>(a, grp, RowBounds(a, r0, r1), list, n, [&](uint32_t key) {
       const int s = find_slot(table, slots - 1u, key);
       return s >= 0 ? (int)(table[s] >> 32) : -1;
     });
@@ -397,8 +421,17 @@ __device__ __forceinline__ void list_store(int *list, int idx, int v) {
 // Writes the keys of a table to list[] in slot order and returns their number; with `final`, the
 // table entries are rewritten as (rank, key).  wcount: slots / 64 + 1 words of LDS.  Contains
 // barriers; the table must be complete (a barrier behind the last insert) on entry.
+// check (optional): compares the new order with the list as it was (the construction's input) and with the input
+// of the construction before (check->before, if kept), and leaves the old list there for the next comparison.
+struct OrderCheck {
+  bool on;            // off: nothing is compared or kept (both answers "no")
+  int *before;        // LDS copy of the previous construction's input, or null
+  bool same_as_input;   // out: every key landed on the list entry that already held it
+  bool same_as_before;  // out: ... on the entry of `before` that held it (meaningful when `before` was that input)
+};
 template <int THREADS, bool LIST_IN_LDS>
-__device__ __forceinline__ int compact_table32(const Table32 &t, uint32_t slots, uint32_t *wcount, int *list, bool final) {
+__device__ __forceinline__ int compact_table32(const Table32 &t, uint32_t slots, uint32_t *wcount, int *list, bool final,
+                                               OrderCheck *check = nullptr) {
   constexpr int WAVES = THREADS / 64;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const uint32_t words = slots >= 64u ? slots / 64u : 1u;
@@ -434,6 +467,7 @@ __device__ __forceinline__ int compact_table32(const Table32 &t, uint32_t slots,
     if (lane == 0) wcount[words] = carry;  // number of keys in the table
   }
   __syncthreads();
+  int moved = 0, moved_before = 0;
   for (uint32_t w0 = wave; w0 < words; w0 += 4 * WAVES) {
     uint32_t x[4], before[4];
 #pragma unroll
@@ -450,13 +484,27 @@ __device__ __forceinline__ int compact_table32(const Table32 &t, uint32_t slots,
       const unsigned long long m = __ballot(occ);
       const uint32_t rank = before[j] + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
       if (occ) {
+        // (entry `rank` of either list is written by this thread alone, so what it reads here is the old content)
+        if (check) {
+          const int key = (int)(x[j] & t.key_mask), was = list_load<LIST_IN_LDS>(list, (int)rank);
+          moved |= was != key;
+          if (check->before) {
+            moved_before |= check->before[rank] != key;
+            check->before[rank] = was;
+          }
+        }
         list_store<LIST_IN_LDS>(list, (int)rank, (int)(x[j] & t.key_mask));
         if (final) t.slots[s] = (rank << t.key_bits) | (x[j] & t.key_mask);
       }
     }
   }
   const int kept = (int)wcount[words];
-  __syncthreads();
+  if (check) {
+    check->same_as_input = __syncthreads_or(moved) == 0;
+    check->same_as_before = check->before != nullptr && __syncthreads_or(moved_before) == 0;
+  } else {
+    __syncthreads();
+  }
   return kept;
 }
 
@@ -513,14 +561,17 @@ __device__ __forceinline__ void phase_insert(const Table32 &t, uint32_t mask, co
 // is the old table first compacted into the list.  The phases of the smallest tables (a few dozen
 // keys) are run by the first wave alone, without workgroup barriers.
 static constexpr uint32_t kSoloSlots = 128;
+// check: see compact_table32; both answers are "no" when the list was rewritten between phases, and
+// check.before is then cleared (what it would receive is not the input).
 template <int THREADS, bool LIST_IN_LDS>
-__device__ __forceinline__ uint32_t rebuild_set32(Table32 &t, const TableRegions &reg, int *list, int &n) {
+__device__ __forceinline__ uint32_t rebuild_set32(Table32 &t, const TableRegions &reg, int *list, int &n, OrderCheck &check) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   uint32_t slots = 8, old_slots = 0;
   uint32_t *cur = nullptr;
   int prev_cnt = 0;
   bool solo_pending = false;  // the first wave ran phases on its own that the others have not waited for yet
+  bool list_rewritten = false;  // a compaction between phases already replaced the head of the list
   // the largest table must land in region a: start so that the alternation ends there
   uint32_t phases_to_max = 0;
   for (uint32_t s8 = 8; s8 < reg.cap_a; s8 <<= 2) ++phases_to_max;
@@ -541,6 +592,7 @@ __device__ __forceinline__ uint32_t rebuild_set32(Table32 &t, const TableRegions
       Table32 old = t;
       old.slots = cur;
       prev_cnt = 0;
+      list_rewritten = true;
       compact_table32<THREADS, LIST_IN_LDS>(old, old_slots, nt, list, false);
       nt = cur;
       cur = nullptr;
@@ -565,7 +617,9 @@ __device__ __forceinline__ uint32_t rebuild_set32(Table32 &t, const TableRegions
     }
     if (n < (int)thr) {
       if (solo_pending) __syncthreads();
-      n = compact_table32<THREADS, LIST_IN_LDS>(t, slots, other, list, true);
+      if (list_rewritten || !check.on) check.before = nullptr;
+      n = compact_table32<THREADS, LIST_IN_LDS>(t, slots, other, list, true, check.on ? &check : nullptr);
+      if (list_rewritten || !check.on) check.same_as_input = check.same_as_before = false;
       return slots;
     }
     cur = nt;
@@ -578,7 +632,8 @@ __device__ __forceinline__ uint32_t rebuild_set32(Table32 &t, const TableRegions
 
 template <int THREADS, bool LIST_IN_LDS>
 __global__ __launch_bounds__(THREADS) void svc_merge_fast_kernel(const SvcArgs a, int cls, int cls_last,
-                                                                 uint32_t key_bits, uint32_t max_slots, uint32_t small_slots) {
+                                                                 uint32_t key_bits, uint32_t max_slots, uint32_t small_slots,
+                                                                 int list_cap) {
   extern __shared__ __align__(16) unsigned char smem[];
   // direct mode only: the groups of this launch's classes are listed, and a group's column count is known.
   // A launch takes the classes cls, cls - 1, ..., cls_last (largest groups first).
@@ -604,12 +659,33 @@ __global__ __launch_bounds__(THREADS) void svc_merge_fast_kernel(const SvcArgs a
   reg.b = t.slots + max_slots;
   reg.cap_b = small_slots;
   int *list = LIST_IN_LDS ? reinterpret_cast<int *>(smem + 128 + ((size_t)max_slots + small_slots) * 4) : a.tmp_cols + e0;
+  int *const list_before = LIST_IN_LDS ? list + list_cap : nullptr;  // the input of the latest construction
   const int cap = count;
 
   int n = 0;
   uint32_t slots = 0;
+  const RowBounds rows(a, r0, r1);
+  // CPython rebuilds the set for every member row, also for one that brings nothing new (an empty row, a row of
+  // known columns); the order may still change then, because the keys go in in the previous table's slot order.
+  // Two cases need no construction.  period == 1: the latest construction returned its keys in the order it got
+  // them, so every further one without new keys does too.  period == 2: it returned the order that went into the
+  // construction before it, so further ones alternate between the two orders: they are counted (`owed`, modulo 2)
+  // and at most one of them is carried out, when new keys arrive or at the end.
+  // The comparisons cost a few per cent of a construction, so they are made where they can pay: when the row
+  // brought nothing new itself, or when the row behind it is empty.
+  int period = 0, owed = 0;
+  bool before_is_input = false;  // list_before holds the input of the construction that produced the list
+  OrderCheck check;
+  auto construct = [&](bool without_new_keys, bool compare) {
+    const bool had_input = before_is_input;
+    check.on = compare;
+    check.before = list_before;
+    slots = rebuild_set32<THREADS, LIST_IN_LDS>(t, reg, list, n, check);
+    period = check.same_as_input ? 1 : (without_new_keys && had_input && check.same_as_before) ? 2 : 0;
+    before_is_input = check.before != nullptr;
+  };
   for (int row = r0; row < r1; ++row) {
-    const int b = a.row_ptr[row], e = a.row_ptr[row + 1];
+    const int b = rows.start(row - r0), e = rows.start(row - r0 + 1);
     // acc + row: append the row's columns that are not in acc yet, in row order
     int appended = 0;
     for (int base = b; base < e; base += THREADS) {
@@ -625,12 +701,27 @@ __global__ __launch_bounds__(THREADS) void svc_merge_fast_kernel(const SvcArgs a
       if (is_new && n + appended + rank < cap) list_store<LIST_IN_LDS>(list, n + appended + rank, (int)k);
       appended += total;
     }
-    n = min(n + appended, cap);  // the cap only bites for invalid input (a row that repeats a column)
+    appended = min(appended, cap - n);  // the cap only bites for invalid input (a row that repeats a column)
     __syncthreads();
-    slots = rebuild_set32<THREADS, LIST_IN_LDS>(t, reg, list, n);
+    if (appended == 0 && slots != 0) {
+      if (period == 1) continue;
+      if (period == 2) {
+        owed ^= 1;
+        continue;
+      }
+      construct(true, true);
+      continue;
+    }
+    if (owed) {  // the order the new keys go behind is the other one of the pair (the new keys wait behind list[n])
+      construct(true, false);
+      owed = 0;
+    }
+    n += appended;
+    construct(false, row + 1 < r1 && rows.start(row - r0 + 1) == rows.start(row - r0 + 2));
   }
+  if (owed) construct(true, false);
 
-  write_group_output<THREADS>(a, grp, r0, r1, list, n, [&](uint32_t key) {
+  write_group_output<THREADS>(a, grp, rows, list, n, [&](uint32_t key) {
     const int sl = find_slot32(t, slots - 1u, key);
     return sl >= 0 ? (int)(t.slots[sl] >> key_bits) : -1;
   });
@@ -766,6 +857,18 @@ __global__ __launch_bounds__(THREADS) void svc_fill_kernel(const SvcArgs a, cons
 
 static size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
+// Lets a kernel ask for `lds` bytes of dynamic LDS; the runtime is only told when a kernel's need grows
+// (`raised`: the limit in force per device, one array per kernel).
+static constexpr int kMaxDevices = 16;
+static hipError_t raise_lds_limit(const void *kern, size_t lds, int (&raised)[kMaxDevices]) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) dev = -1;
+  if (dev >= 0 && raised[dev] >= (int)lds) return hipSuccess;
+  const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (e == hipSuccess && dev >= 0) raised[dev] = (int)lds;
+  return e;
+}
+
 size_t svc_workspace_layout(int64_t nnz, int m_vec, size_t *off_pos, size_t *off_tables, size_t *off_lists) {
   const size_t n = (size_t)(nnz > 0 ? nnz : 1);
   const size_t cols = align256(n * 4);
@@ -785,8 +888,8 @@ static hipError_t launch_lds_class(const SvcArgs &base, int m_vec, int lo, int h
   const size_t lds = 128 + (size_t)slots * 8 + (size_t)hi * 4;
   auto kern = svc_merge_cpython_kernel<THREADS, true>;
   if (lds > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    static int raised[kMaxDevices] = {};
+    const hipError_t e = raise_lds_limit(reinterpret_cast<const void *>(kern), lds, raised);
     if (e != hipSuccess) return e;
   }
   hipLaunchKernelGGL(kern, dim3(m_vec), dim3(THREADS), lds, stream, a, lo, hi, hi);
@@ -799,17 +902,19 @@ static hipError_t launch_fast_class(const SvcArgs &a, int grid, int cls, int cls
   // second table region: a quarter of the first (what the phase before the largest needs), less where LDS is short;
   // it also serves as the running-count array of the compaction of a table in the first region (slots / 64 + 1 words)
   uint32_t small_slots = slots / 4u;
-  while (128 + ((size_t)slots + small_slots) * 4 + (LIST_IN_LDS ? (size_t)hi * 4 : 0) > 160 * 1024) small_slots /= 4u;
+  // (a key list in LDS has a second copy behind it: the input of the latest construction)
+  const size_t list_bytes = LIST_IN_LDS ? (size_t)hi * 8 : 0;
+  while (128 + ((size_t)slots + small_slots) * 4 + list_bytes > 160 * 1024) small_slots /= 4u;
   if (small_slots < slots / 64u + 1u) return hipErrorInvalidValue;
-  size_t lds = 128 + ((size_t)slots + small_slots) * 4 + (LIST_IN_LDS ? (size_t)hi * 4 : 0);
+  size_t lds = 128 + ((size_t)slots + small_slots) * 4 + list_bytes;
   if (lds < min_lds) lds = min_lds;  // asking for more than half of a CU's LDS keeps a workgroup alone on its CU
   auto kern = svc_merge_fast_kernel<THREADS, LIST_IN_LDS>;
   if (lds > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    static int raised[kMaxDevices] = {};
+    const hipError_t e = raise_lds_limit(reinterpret_cast<const void *>(kern), lds, raised);
     if (e != hipSuccess) return e;
   }
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(THREADS), lds, stream, a, cls, cls_last, key_bits, slots, small_slots);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(THREADS), lds, stream, a, cls, cls_last, key_bits, slots, small_slots, hi);
   return hipGetLastError();
 }
 
@@ -921,9 +1026,8 @@ hipError_t launch_svc_count(const SvcArgs &a, int order, hipStream_t stream) {
     if (lds > 160 * 1024) return hipErrorInvalidValue;
     auto kern = svc_merge_sorted_kernel<256>;
     if (lds > 64 * 1024) {
-      e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              (int)lds);
-      if (e != hipSuccess) return e;
+      static int raised[kMaxDevices] = {};
+      if ((e = raise_lds_limit(reinterpret_cast<const void *>(kern), lds, raised)) != hipSuccess) return e;
     }
     hipLaunchKernelGGL(kern, dim3(m_vec), dim3(256), lds, stream, a);
     if ((e = hipGetLastError()) != hipSuccess) return e;
@@ -954,29 +1058,47 @@ hipError_t launch_svc_fill(const SvcArgs &args, int order, const uint16_t *csr_v
   a.vec_val = csr_val ? vec_val : nullptr;
   a.csr_val = csr_val;
   const uint32_t key_bits = bits_of(a.K);
-  hipError_t e;
+  // A group cannot hold more distinct columns than the matrix has columns or entries: the launches of the classes
+  // above that bound are left out (each would cost a launch's latency to find its list empty).
+  const long long bound = a.nnz < a.K ? a.nnz : (long long)a.K;
+  const bool medium = bound > kSmallKeys, large = bound > kMediumKeys, xlarge = bound > kLargeKeys, beyond = bound > kXLargeKeys;
+  const int cus = 256;
+  hipError_t e = hipSuccess;
+  // Grids: what the chip holds at once for the class's workgroup size and LDS, at most one workgroup per group.
+  // The two classes of 1229 .. 4914 and 307 .. 1228 columns share a launch on the caller's stream (1024 threads
+  // and 8192-slot tables for both): with one such workgroup per CU resident every group (up to the number of CUs) of either
+  // class starts at once, and nothing that could outlast the largest group waits on a helper stream to begin.
+  // These workgroups are chains of LDS round trips: each gets a CU to itself (by asking for more than half its LDS).
+  auto rare_classes = [&](hipStream_t s) {
+    if (e == hipSuccess && xlarge) e = launch_fast_class<1024, false>(a, min(m_vec, cus), 3, 3, kXLargeKeys, 32768, key_bits, s);
+    if (e == hipSuccess && beyond) {
+      // more columns than a 32768-slot table takes: 64-bit entries in the workspace
+      hipLaunchKernelGGL((svc_merge_cpython_kernel<1024, false>), dim3(min(m_vec, cus)), dim3(1024), 128, s, a, 0, 0, 0);
+      e = hipGetLastError();
+    }
+  };
+  if (!medium || m_vec <= cus) {
+    // Everything on the caller's stream: either no group can be larger than the small class, or the matrix has so
+    // few groups that each gets a CU of its own in one launch of the wide workgroups (which then also take the
+    // small groups); a fork and a join of a helper stream would cost more than they hide.
+    if (!medium)
+      e = launch_fast_class<64, true>(a, min(m_vec, 32 * cus), 0, 0, kSmallKeys, 512, key_bits, stream);
+    else
+      e = launch_fast_class<1024, true>(a, m_vec, large ? 2 : 1, 0, kLargeKeys, 8192, key_bits, stream, 81 * 1024);
+    rare_classes(stream);
+    return e;
+  }
+  // The many small groups, and the two classes that are nearly always empty, follow each other on one helper
+  // stream: one fork and one join.
   SideStreams *ss = side_streams_for(stream);
   std::unique_lock<std::mutex> sequence;
   if (ss) sequence = std::unique_lock<std::mutex>(ss->in_use);
   hipStream_t st[4];
   if ((e = fork_streams(ss, stream, st, 1)) != hipSuccess) return e;
   // (from here on the helper is joined back into the caller's stream whatever happens)
-  // Grids: what the chip holds at once for the class's workgroup size and LDS, at most one workgroup per group.
-  // The two classes of 1229 .. 4914 and 307 .. 1228 columns share a launch on the caller's stream (1024 threads
-  // and 8192-slot tables for both): with one such workgroup per CU resident every group (up to the number of CUs) of either
-  // class starts at once, and nothing that could outlast the largest group waits on a helper stream to begin.
-  // These workgroups are chains of LDS round trips: each gets a CU to itself (by asking for more than half its LDS).
-  // The many small groups, and the two classes that are nearly always empty, follow each other on one helper
-  // stream: one fork and one join.
-  const int cus = 256;
-  e = launch_fast_class<1024, true>(a, min(m_vec, cus), 2, 1, kLargeKeys, 8192, key_bits, st[0], 81 * 1024);
+  e = launch_fast_class<1024, true>(a, min(m_vec, cus), large ? 2 : 1, 1, kLargeKeys, 8192, key_bits, st[0], 81 * 1024);
   if (e == hipSuccess) e = launch_fast_class<64, true>(a, min(m_vec, 32 * cus), 0, 0, kSmallKeys, 512, key_bits, st[1]);
-  if (e == hipSuccess) e = launch_fast_class<1024, false>(a, min(m_vec, cus), 3, 3, kXLargeKeys, 32768, key_bits, st[1]);
-  if (e == hipSuccess) {
-    // more columns than a 32768-slot table takes: 64-bit entries in the workspace
-    hipLaunchKernelGGL((svc_merge_cpython_kernel<1024, false>), dim3(min(m_vec, cus)), dim3(1024), 128, st[1], a, 0, 0, 0);
-    e = hipGetLastError();
-  }
+  rare_classes(st[1]);
   const hipError_t ej = join_streams(ss, stream, 1);
   return e != hipSuccess ? e : ej;
 }

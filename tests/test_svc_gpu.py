@@ -114,6 +114,40 @@ def test_a_groups_class_comes_from_its_distinct_columns(oracle, built_library, d
     assert vrp[2] - vrp[1] == distinct
 
 
+@pytest.mark.parametrize("keys", [5, 40, 200, 700, 2500, 4000])
+def test_member_rows_that_bring_nothing_new(oracle, built_library, keys):
+    """CPython rebuilds the set for every member row, also for an empty row and for a row whose columns are all
+    known; the order can change each time, settle, or alternate between two orders.  The kernels skip
+    constructions whose result they know: groups whose empty and repeated rows come singly, in runs of even and
+    odd length, at the start, between rows with new columns and at the end, in every size class, against the
+    Python runtime's own set."""
+    rng = np.random.default_rng(keys)
+    V, K = 8, 16384
+    layouts = ["n.......", "nr......", "n.n.....", "n..n....", "n...n...", "n....n..", ".n.....n", "..n..r.n",
+               "nrrrrrrr", "n.r.r.r.", "nn....nn", "n.....rn", "........", "...n....", "n......r", "nr.n.r.n"]
+    rows = []
+    for layout in layouts:
+        seen = np.empty(0, np.int64)
+        for ch in layout:
+            if ch == "n":    # new columns (and a few known ones)
+                fresh = rng.choice(np.setdiff1d(np.arange(K), seen), keys, replace=False)
+                again = rng.choice(seen, min(seen.size, 3), replace=False) if seen.size else seen
+                row = np.sort(np.concatenate([fresh, again]))
+                seen = np.union1d(seen, fresh)
+            elif ch == "r":  # only known columns
+                row = np.sort(rng.choice(seen, max(1, seen.size // 2), replace=False)) if seen.size else seen
+            else:
+                row = np.empty(0, np.int64)
+            rows.append(row)
+    lens = np.array([r.size for r in rows])
+    ptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cols = np.concatenate(rows).astype(np.int32)
+    csr = synth.Csr(len(rows), K, ptr, cols, rng.standard_normal(cols.size).astype(np.float16))
+    vrp, vcol, _ = _compare_with_oracle(oracle, csr, V)
+    want_ptr, want_cols = oracle.rowmerge_python(csr.M, V, oracle.csr_col_lists(csr.M, csr.row_ptr, csr.col_ind))
+    assert vrp.tolist() == want_ptr and vcol.tolist() == want_cols
+
+
 def test_more_groups_of_a_class_than_workgroups_in_its_launch(oracle, built_library):
     """V = 1 makes every row a group: 9000 short rows (the launch of the smallest class has 8192 workgroups),
     and 300 + 260 + 270 rows of 1300, 400 and 5000 columns (one workgroup per CU for those classes), so that

@@ -37,7 +37,7 @@ struct ScheduleItem {
 };
 
 static constexpr int kScheduleMinBudget = 8;      // steps: shorter panels are all overhead
-static constexpr int kScheduleTargetItems = 1024;  // panels of cut rows wanted at most (before the memory cap)
+static constexpr int kScheduleTargetItems = 512;   // panels of cut rows wanted at most (before the memory cap)
 
 // A partial tile: the accumulators of one wave (V rows x 64 columns, fp32) as they lie in its registers,
 // 4 x (lanes that hold rows) x 16 bytes.

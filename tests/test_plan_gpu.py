@@ -32,7 +32,7 @@ def expected_info(lens, panel_steps=0):
     """The schedule's figures restated from the row lengths (steps of 32 vectors; an empty row is one step)."""
     steps = steps_of(lens)
     total, m_vec = int(steps.sum()), len(steps)
-    budget = panel_steps or max(8, -(-total // 1024), -(-2 * total // m_vec))
+    budget = panel_steps or max(8, -(-total // 512), -(-2 * total // m_vec))
     cut = steps > budget
     panels = int((-(-steps[cut] // budget)).sum())
     return dict(num_vec=int(np.sum(lens)), longest_row_steps=int(steps.max()), total_steps=total, panel_steps=budget,

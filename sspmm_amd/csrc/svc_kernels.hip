@@ -383,18 +383,23 @@ __device__ __forceinline__ int find_slot32(const Table32 &t, uint32_t mask, uint
 }
 
 // First-come-first-served placement of one key, as in place() above, on 32-bit entries.
-__device__ __forceinline__ void place32(const Table32 &t, uint32_t mask, uint32_t key, uint32_t order) {
-  uint32_t mine = (order << t.key_bits) | key;
+// A function of its own on purpose: inlined into the eight-fold unrolled loops of every phase variant it made the
+// merge kernels 150 KB of code, more than twice the instruction cache that two CUs share, and a construction is
+// a walk through all of it.  The table comes as an LDS pointer so that the atomic stays an LDS instruction.
+typedef __attribute__((address_space(3))) uint32_t lds_u32;
+__device__ __attribute__((noinline)) void place32_lds(lds_u32 *slots, uint32_t key_bits, uint32_t mask, uint32_t key, uint32_t order) {
+  const uint32_t key_mask = (1u << key_bits) - 1u;
+  uint32_t mine = (order << key_bits) | key;
   uint32_t i, perturb, lin;
   probe_start(key, mask, i, perturb, lin);
   for (;;) {
     const uint32_t s0 = i + lin;
-    const uint32_t old = atomicMin(&t.slots[s0], mine);
-    if (old == kEmpty32 || ((old ^ mine) & t.key_mask) == 0) return;  // placed, or a repeated key (invalid row)
+    const uint32_t old = __hip_atomic_fetch_min(slots + s0, mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (old == kEmpty32 || ((old ^ mine) & key_mask) == 0) return;  // placed, or a repeated key (invalid row)
     if (old > mine) {
       // a later entry sat here: carry it on from this slot of its own probe sequence
       mine = old;
-      probe_start(old & t.key_mask, mask, i, perturb, lin);
+      probe_start(old & key_mask, mask, i, perturb, lin);
       // nearly always it lost a slot of its first window: no walk needed then
       const uint32_t d = s0 - i;
       if ((d <= 9u) & ((i + 9u <= mask) | (d == 0u)))
@@ -404,6 +409,9 @@ __device__ __forceinline__ void place32(const Table32 &t, uint32_t mask, uint32_
     }
     probe_next(mask, i, perturb, lin);
   }
+}
+__device__ __forceinline__ void place32(const Table32 &t, uint32_t mask, uint32_t key, uint32_t order) {
+  place32_lds((lds_u32 *)t.slots, t.key_bits, mask, key, order);
 }
 
 // The key list lives in LDS, or in the workspace where other waves of the group wrote it: those

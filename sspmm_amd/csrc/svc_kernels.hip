@@ -545,6 +545,9 @@ __device__ __forceinline__ void phase_insert(const Table32 &t, uint32_t mask, co
     }
   }
   const uint32_t first_index = old_table != nullptr ? old_slots : 0u;
+  // the list's keys start with the thread behind the last one that holds a slot of the previous table, so that as few
+  // threads as possible have a key of both kinds to place one after the other
+  me = (me + STRIDE - (int)(first_index % (uint32_t)STRIDE)) % STRIDE;
   for (int base = prev_cnt + me; base < cnt; base += 8 * STRIDE) {
     int k8[8];
 #pragma unroll

@@ -18,6 +18,7 @@ struct SddmmArgs {
   uint16_t *out;        // [batch][nvec*V]
   int64_t stride_lhs, stride_rhs, stride_out;  // per-batch strides in elements
   uint32_t total_work, per_xcd;                // filled by the launcher
+  int pair_stores;                             // filled by the launcher: out and stride_out allow 16-byte stores
 };
 
 struct SoftmaxArgs {

@@ -134,7 +134,8 @@ __global__ __launch_bounds__(64) void sddmm_kernel(const SddmmArgs p) {
     for (int i = 0; i < NC; ++i)
       if (ld_ok[i]) *reinterpret_cast<uintx4 *>(st + ld_dst[i]) = b.d[i];
   };
-  auto finish = [&](const unsigned char *st, int kc) {
+  // the group's 16 x V products: lane (m, g) gets rows 4g .. 4g+3 of stored vector kc + m, as four halfs
+  auto products = [&](const unsigned char *st) {
     floatx4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
@@ -142,11 +143,23 @@ __global__ __launch_bounds__(64) void sddmm_kernel(const SddmmArgs p) {
       if (op_ok[c]) b = *reinterpret_cast<const half8 *>(st + op_off[c]);
       acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[c], b, acc, 0, 0, 0);
     }
-    if (kc + m < end && 4 * g < V) {
-      const half4 h = {(_Float16)acc[0], (_Float16)acc[1], (_Float16)acc[2], (_Float16)acc[3]};  // round to nearest even
-      *reinterpret_cast<half4 *>(out + ((int64_t)(kc + m) * V + 4 * g)) = h;
-    }
+    const half4 h = {(_Float16)acc[0], (_Float16)acc[1], (_Float16)acc[2], (_Float16)acc[3]};  // round to nearest even
+    return __builtin_bit_cast(uintx2, h);
   };
+  auto store_group = [&](uintx2 h, int kc) {
+    if (kc + m < end && 4 * g < V) *reinterpret_cast<uintx2 *>(out + ((int64_t)(kc + m) * V + 4 * g)) = h;
+  };
+  // Two groups in one store instruction (a store costs the address unit the same sixteen cycles whether its lanes
+  // carry 8 or 16 bytes, and this kernel is bound by that unit): the lane groups g and g + 1 exchange halves, so
+  // that g even holds rows 8 (g / 2) .. + 7 of vector kc + m and g odd those of vector kc + 16 + m.
+  auto store_two_groups = [&](uintx2 first, uintx2 second, int kc) {
+    const auto w0 = __builtin_amdgcn_permlane16_swap(first[0], second[0], false, false);
+    const auto w1 = __builtin_amdgcn_permlane16_swap(first[1], second[1], false, false);
+    const uintx4 v = {(uint32_t)w0[0], (uint32_t)w1[0], (uint32_t)w0[1], (uint32_t)w1[1]};
+    const int vec = kc + m + 16 * (g & 1);
+    if (vec < end && 8 * (g >> 1) < V) *reinterpret_cast<uintx4 *>(out + ((int64_t)vec * V + 8 * (g >> 1))) = v;
+  };
+  const bool pair_stores = p.pair_stores != 0;
 
   // The LDS operations of a wave execute in order, so a stage can be rewritten right after the reads of the group
   // that used it have been issued; no barrier is involved (one wave per workgroup).
@@ -159,21 +172,26 @@ __global__ __launch_bounds__(64) void sddmm_kernel(const SddmmArgs p) {
   for (;;) {
     // stage[0] holds group kc; c_next the columns of group kc + 16
     if (kc + 16 >= end) {
-      finish(stage[0], kc);
+      store_group(products(stage[0]), kc);
       break;
     }
     Cols c_after = load_cols(kc + 32);
     load_rows(b1, c_next);
-    finish(stage[0], kc);
+    const uintx2 first = products(stage[0]);
+    if (!pair_stores) store_group(first, kc);
     to_stage(b1, stage[1]);
     kc += 16;
     if (kc + 16 >= end) {
-      finish(stage[1], kc);
+      const uintx2 second = products(stage[1]);
+      if (pair_stores) store_two_groups(first, second, kc - 16);
+      else store_group(second, kc);
       break;
     }
     c_next = load_cols(kc + 32);
     load_rows(b0, c_after);
-    finish(stage[1], kc);
+    const uintx2 second = products(stage[1]);
+    if (pair_stores) store_two_groups(first, second, kc - 16);
+    else store_group(second, kc);
     to_stage(b0, stage[0]);
     kc += 16;
   }
@@ -182,6 +200,7 @@ __global__ __launch_bounds__(64) void sddmm_kernel(const SddmmArgs p) {
 template <int V, int NC>
 static hipError_t launch_sddmm_nc(const SddmmArgs &a, hipStream_t stream) {
   SddmmArgs p = a;
+  p.pair_stores = reinterpret_cast<uintptr_t>(a.out) % 16 == 0 && a.stride_out % 8 == 0;
   p.total_work = (uint32_t)a.m_vec * (uint32_t)a.batch;
   p.per_xcd = (p.total_work + 7u) / 8u;
   if (p.total_work == 0) return hipSuccess;

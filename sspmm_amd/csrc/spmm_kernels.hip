@@ -1742,6 +1742,11 @@ hipError_t launch_spmm(const SpmmArgs &a, int V, bool out_f16, hipStream_t strea
     }
     which = (slab_ok && a.m_vec >= 64 && weighted >= enough) ? 3 : 2;
     if (narrow_ok && V == 8 && a.m_vec >= 256 && 2u * blocks >= 1024) which = 5;
+    // (known to be at least 30 % dense, a slab's rows are used often enough from half as many vector-rows on:
+    // 1.3-1.45x over the gather kernel on 1024 x 2048 at 50 and 70 % sparsity, level at 80 %)
+    if (narrow_ok && V == 8 && a.m_vec >= 128 && 2u * blocks >= 1024 && a.mean_row_vectors > 0 &&
+        (int64_t)a.mean_row_vectors * 10 >= (int64_t)a.K * 3)
+      which = 5;
     // Very sparse patterns with V = 16 and fp32 C: a vector-row is one step, the slab kernel's per-row work (claim,
     // table entry, store set-up) outweighs it, and the gather kernels win (measured at 95 and 98 % sparsity up to 32
     // vectors per row: 1.13-1.18x; with V = 8 the two tie, and between the gather kernels the density changes nothing).

@@ -255,6 +255,7 @@ def test_plan_argument_checks(built_library):
     (2048, 1024, 16, 0.98, 256, 128, 3, 2),  # one step per row: a gather kernel in place of the slab kernel
     (3072, 768, 8, 0.7, 64, 16, 6, 3),       # dense for this format: the slab kernel from fewer blocks on
     (2048, 512, 8, 0.9, 256, 128, 3, 3),     # the density the thresholds were measured at: no change
+    (1024, 2048, 8, 0.7, 256, 32, 2, 5),     # tall and dense: the 32-column slab from half as many vector-rows on
 ])
 def test_plan_of_an_even_pattern_picks_the_kernel_by_density(oracle, built_library, M, K, V, sparsity, N, batch, want_plain,
                                                              want_planned):

@@ -172,7 +172,7 @@ struct SlabVals<16> {
 // indices of chunk s + 2 are in flight.
 template <int V>
 struct ChunkHead {   // stage 1: what does not depend on other loads
-  uintx4 c0, c1;     // column indices of k slots 8g .. 8g+7
+  uint32_t cols;     // column index of k slot lane % 32 (the lanes that need it fetch it from there)
   typename SlabVals<V>::type vraw;  // the lane's share of the chunk's 32 x V values, as they lie in memory
   int kc;            // first vector of the chunk
 };
@@ -202,11 +202,11 @@ struct Chunk {
 template <int V>
 __device__ __forceinline__ void load_head(ChunkHead<V> &h, int kc, int g, __amdgpu_buffer_rsrc_t srd_cols,
                                           __amdgpu_buffer_rsrc_t srd_vals, uint32_t vals_lane_off) {
-  const int kb = kc + 8 * g;
   h.kc = kc;
   // srd_cols / srd_vals end at this vector-row's last vector: slots past it read as zero.
-  h.c0 = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_cols, kb * 4, 0, 0));
-  h.c1 = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_cols, kb * 4 + 16, 0, 0));
+  // One dword per lane, 128 distinct bytes per instruction (the address unit takes sixteen cycles for an instruction
+  // of a wave whatever it carries: the eight indices a lane needs, fetched by the lane itself, cost two of them).
+  h.cols = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(srd_cols, (kc + (int)(threadIdx.x & 31)) * 4, 0, 0);
   // one coalesced load of the chunk's values (vals_lane_off = lane * V bytes); vectors past the row read as zero
   h.vraw = SlabVals<V>::load(srd_vals, (uint32_t)kc * (V * 2) + vals_lane_off);
 }
@@ -220,7 +220,7 @@ __device__ __forceinline__ void load_body(Chunk<CPL> &c, const ChunkHead<V> &h, 
   uint32_t off[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
-    const uint32_t col = j < 4 ? h.c0[j] : h.c1[j - 4];
+    const uint32_t col = (uint32_t)__builtin_amdgcn_ds_bpermute((8 * g + j) * 4, (int)h.cols);
     off[j] = __umul24(col, lane_n2) + lane_col_off;
   }
   if (h.kc + 32 > end) {  // wave-uniform: only the last chunk of a vector-row can be partial

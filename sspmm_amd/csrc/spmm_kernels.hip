@@ -170,9 +170,15 @@ struct SlabVals<16> {
 // memory round trips (column indices, then the rows of B they name), so they are issued in two
 // stages, one step apart: while chunk s is contracted, the gathers of chunk s + 1 and the column
 // indices of chunk s + 2 are in flight.
-template <int V>
+// SHARED_COLS: the column indices come as one dword per lane and the lanes that need one fetch it from there with a
+// lane permute (the address unit takes sixteen cycles for a load instruction of a wave whatever it carries: the
+// eight indices a lane needs, loaded by the lane itself, cost two of them).  Pays where that unit bounds the kernel
+// (one wave per vector-row, many in flight); where a single long row is the critical path (the split-row kernel)
+// the permutes' latency costs more than the instruction saves.
+template <int V, bool SHARED_COLS = true>
 struct ChunkHead {   // stage 1: what does not depend on other loads
-  uint32_t cols;     // column index of k slot lane % 32 (the lanes that need it fetch it from there)
+  uint32_t cols;     // SHARED_COLS: column index of k slot lane % 32
+  uintx4 c0, c1;     // otherwise: column indices of k slots 8g .. 8g+7
   typename SlabVals<V>::type vraw;  // the lane's share of the chunk's 32 x V values, as they lie in memory
   int kc;            // first vector of the chunk
 };
@@ -199,28 +205,33 @@ struct Chunk {
   typename ChunkRaw<CPL>::type raw[8];  // raw[j] = CPL halfs (columns n0+CPL*m..) of the row of B named by k slot 8g+j
 };
 
-template <int V>
-__device__ __forceinline__ void load_head(ChunkHead<V> &h, int kc, int g, __amdgpu_buffer_rsrc_t srd_cols,
+template <int V, bool SHARED_COLS>
+__device__ __forceinline__ void load_head(ChunkHead<V, SHARED_COLS> &h, int kc, int g, __amdgpu_buffer_rsrc_t srd_cols,
                                           __amdgpu_buffer_rsrc_t srd_vals, uint32_t vals_lane_off) {
   h.kc = kc;
   // srd_cols / srd_vals end at this vector-row's last vector: slots past it read as zero.
-  // One dword per lane, 128 distinct bytes per instruction (the address unit takes sixteen cycles for an instruction
-  // of a wave whatever it carries: the eight indices a lane needs, fetched by the lane itself, cost two of them).
-  h.cols = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(srd_cols, (kc + (int)(threadIdx.x & 31)) * 4, 0, 0);
+  if (SHARED_COLS) {
+    h.cols = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(srd_cols, (kc + (int)(threadIdx.x & 31)) * 4, 0, 0);
+  } else {
+    const int kb = kc + 8 * g;
+    h.c0 = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_cols, kb * 4, 0, 0));
+    h.c1 = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_cols, kb * 4 + 16, 0, 0));
+  }
   // one coalesced load of the chunk's values (vals_lane_off = lane * V bytes); vectors past the row read as zero
   h.vraw = SlabVals<V>::load(srd_vals, (uint32_t)kc * (V * 2) + vals_lane_off);
 }
 
 // (also sends the chunk's values to the value tile `tile_lane` points into: the lane's slot of the tile)
-template <int CPL, int V>
-__device__ __forceinline__ void load_body(Chunk<CPL> &c, const ChunkHead<V> &h, int end, int g, __amdgpu_buffer_rsrc_t srd_b,
+template <int CPL, int V, bool SHARED_COLS>
+__device__ __forceinline__ void load_body(Chunk<CPL> &c, const ChunkHead<V, SHARED_COLS> &h, int end, int g, __amdgpu_buffer_rsrc_t srd_b,
                                           uint32_t lane_n2, uint32_t lane_col_off, uint32_t b_bytes,
                                           unsigned char *tile_lane) {
   const int kb = h.kc + 8 * g;
   uint32_t off[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
-    const uint32_t col = (uint32_t)__builtin_amdgcn_ds_bpermute((8 * g + j) * 4, (int)h.cols);
+    const uint32_t col = SHARED_COLS ? (uint32_t)__builtin_amdgcn_ds_bpermute((8 * g + j) * 4, (int)h.cols)
+                                     : (j < 4 ? h.c0[j] : h.c1[j - 4]);
     off[j] = __umul24(col, lane_n2) + lane_col_off;
   }
   if (h.kc + 32 > end) {  // wave-uniform: only the last chunk of a vector-row can be partial
@@ -334,8 +345,8 @@ __global__ __launch_bounds__(64) void spmm_gather_kernel(const SpmmArgs p) {
     // A head past the end of the row reads zeros and is never turned into a body.
     ChunkHead<V> h0, h1;
     Chunk<CPL> c0, c1;
-    load_head<V>(h0, beg, g, srd_cols, srd_vals, vals_lane_off);
-    load_head<V>(h1, beg + 32, g, srd_cols, srd_vals, vals_lane_off);
+    load_head(h0, beg, g, srd_cols, srd_vals, vals_lane_off);
+    load_head(h1, beg + 32, g, srd_cols, srd_vals, vals_lane_off);
     load_body(c0, h0, end, g, srd_b, lane_n2, lane_col_off, b_bytes, tw0);
     int kc = beg + 32;  // first vector of the chunk whose body is loaded next
     for (;;) {
@@ -343,7 +354,7 @@ __global__ __launch_bounds__(64) void spmm_gather_kernel(const SpmmArgs p) {
         mac_chunk<CPL, V>(c0, acc, tr0);
         break;
       }
-      load_head<V>(h0, kc + 32, g, srd_cols, srd_vals, vals_lane_off);
+      load_head(h0, kc + 32, g, srd_cols, srd_vals, vals_lane_off);
       load_body(c1, h1, end, g, srd_b, lane_n2, lane_col_off, b_bytes, tw1);
       mac_chunk<CPL, V>(c0, acc, tr0);
       kc += 32;
@@ -351,7 +362,7 @@ __global__ __launch_bounds__(64) void spmm_gather_kernel(const SpmmArgs p) {
         mac_chunk<CPL, V>(c1, acc, tr1);
         break;
       }
-      load_head<V>(h1, kc + 32, g, srd_cols, srd_vals, vals_lane_off);
+      load_head(h1, kc + 32, g, srd_cols, srd_vals, vals_lane_off);
       load_body(c0, h0, end, g, srd_b, lane_n2, lane_col_off, b_bytes, tw0);
       mac_chunk<CPL, V>(c1, acc, tr1);
       kc += 32;
@@ -421,10 +432,10 @@ __device__ __forceinline__ void gather_accumulate(floatx4 (&acc)[8], const SpmmA
 #pragma unroll
   for (int q = 0; q < 8; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
   if (beg >= sub_end) return;
-  ChunkHead<V> h0, h1;
+  ChunkHead<V, false> h0, h1;
   Chunk<8> c0, c1;
-  load_head<V>(h0, beg, g, srd_cols, srd_vals, vals_lane_off);
-  load_head<V>(h1, beg + 32, g, srd_cols, srd_vals, vals_lane_off);
+  load_head(h0, beg, g, srd_cols, srd_vals, vals_lane_off);
+  load_head(h1, beg + 32, g, srd_cols, srd_vals, vals_lane_off);
   load_body(c0, h0, end, g, srd_b, lane_n2, lane_col_off, b_bytes, tw0);
   int kc = beg + 32;  // first vector of the chunk whose body is loaded next
   for (;;) {
@@ -432,7 +443,7 @@ __device__ __forceinline__ void gather_accumulate(floatx4 (&acc)[8], const SpmmA
       mac_chunk<8, V>(c0, acc, tr0);
       break;
     }
-    load_head<V>(h0, kc + 32, g, srd_cols, srd_vals, vals_lane_off);
+    load_head(h0, kc + 32, g, srd_cols, srd_vals, vals_lane_off);
     load_body(c1, h1, end, g, srd_b, lane_n2, lane_col_off, b_bytes, tw1);
     mac_chunk<8, V>(c0, acc, tr0);
     kc += 32;
@@ -440,7 +451,7 @@ __device__ __forceinline__ void gather_accumulate(floatx4 (&acc)[8], const SpmmA
       mac_chunk<8, V>(c1, acc, tr1);
       break;
     }
-    load_head<V>(h1, kc + 32, g, srd_cols, srd_vals, vals_lane_off);
+    load_head(h1, kc + 32, g, srd_cols, srd_vals, vals_lane_off);
     load_body(c0, h0, end, g, srd_b, lane_n2, lane_col_off, b_bytes, tw0);
     mac_chunk<8, V>(c1, acc, tr1);
     kc += 32;

@@ -62,7 +62,7 @@ hipError_t launch_schedule_fill(int m_vec, const int32_t *row_offsets, const Sch
                                 int64_t counters_to_clear, int64_t counters_per_cut_row, hipStream_t stream);
 
 // launch_schedule_measure (budget chosen from the pattern) and launch_schedule_fill (clearing the counters of the
-// cut rows) as one launch.
+// cut rows) as one launch; up to 4096 vector-rows by a kernel of its own that writes the same schedule sooner.
 hipError_t launch_schedule_build(int m_vec, const int32_t *row_offsets, int64_t slot_cap, const ScheduleView &view,
                                  int64_t item_cap, int64_t counters_per_cut_row, hipStream_t stream);
 

@@ -199,6 +199,248 @@ __global__ __launch_bounds__(kBuildThreads) void schedule_build_kernel(int m_vec
   schedule_fill(m_vec, row_offsets, header, items, item_cap, counters, -1, counters_per_cut_row, scratch);
 }
 
+// ------------------------------------------------------------------------------------------
+// The same schedule for patterns of at most kSmallRows vector-rows, which is what a call that rebuilds
+// its schedule every time usually brings.  One workgroup again, arranged for the latency of its one CU:
+// every thread keeps its rows' offsets in registers (row offsets are read from memory once instead of
+// once per pass); the header reaches the other threads as values every thread computes alike instead
+// of through memory; the places of all items come from one scan that carries a value per block of
+// 512 rows; a thread's rows are 512 apart, so that the items of rows that stay whole leave the wave
+// as contiguous stores; and the panels of cut rows are written one per thread from a list in LDS (a
+// loop over a row's panels would make its whole wave wait for the longest row).
+// Writes exactly what schedule_measure + schedule_fill write.
+static constexpr int kSmallThreads = 512;  // 8 waves: 256 registers per thread (the scans hold many words at once)
+static constexpr int kSmallRowsPerThread = 8;
+static constexpr int kSmallRows = kSmallRowsPerThread * kSmallThreads;
+static constexpr int kSmallCutRows = 2048;  // cut rows whose panels are written one per thread (five words of LDS each)
+
+// What a row adds to the running sums, in one word: its panels in bits 0-31 and 1 in bit 32 if it is cut
+// (bits 32-47: cut rows), else 1 in bit 48 (bits 48-63: rows that stay whole; at most kSmallRows = 2^12 rows).
+__device__ __forceinline__ unsigned long long row_word(int steps, int pcs) {
+  return steps == 0 ? 0ull : pcs ? (unsigned long long)(unsigned)pcs + (1ull << 32) : (1ull << 48);
+}
+
+// Lane moves inside the vector unit (a permute through the LDS pipe costs this kernel, which has one wave or two
+// per SIMD and nothing to hide a latency behind, some 70 cycles each).  CTRL: 0x110 + n = from the lane n below in
+// the same row of 16 lanes, 0x142 / 0x143 = lane 15 of the row below / lane 31, to the rows ROW_MASK names; lanes
+// without a source, and rows not named, get 0.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ int lanes_below(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, ROW_MASK, 0xf, true);
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ unsigned long long lanes_below(unsigned long long v) {
+  const unsigned lo = (unsigned)lanes_below<CTRL, ROW_MASK>((int)(unsigned)v);
+  const unsigned hi = (unsigned)lanes_below<CTRL, ROW_MASK>((int)(unsigned)(v >> 32));
+  return ((unsigned long long)hi << 32) | lo;
+}
+// Sum of v over lanes 0 .. own lane of the wave (all 64 lanes active).
+__device__ __forceinline__ unsigned long long wave_inclusive_sum(unsigned long long v) {
+  v += lanes_below<0x111, 0xf>(v);
+  v += lanes_below<0x112, 0xf>(v);
+  v += lanes_below<0x114, 0xf>(v);
+  v += lanes_below<0x118, 0xf>(v);
+  v += lanes_below<0x142, 0xa>(v);  // rows 1 and 3 take the sum of the row below
+  v += lanes_below<0x143, 0xc>(v);  // rows 2 and 3 take the sum of rows 0 and 1
+  return v;
+}
+// Maximum of v (not negative) over lanes 0 .. own lane.
+__device__ __forceinline__ int wave_inclusive_max(int v) {
+  v = max(v, lanes_below<0x111, 0xf>(v));
+  v = max(v, lanes_below<0x112, 0xf>(v));
+  v = max(v, lanes_below<0x114, 0xf>(v));
+  v = max(v, lanes_below<0x118, 0xf>(v));
+  v = max(v, lanes_below<0x142, 0xa>(v));
+  v = max(v, lanes_below<0x143, 0xc>(v));
+  return v;
+}
+
+// Sum over the workgroup of a 64-bit value per thread and maximum of an int per thread.  One barrier; `scratch`
+// (2 x kSmallThreads / 64 words) must not be in use by an earlier step that some wave may still be reading.
+__device__ __forceinline__ unsigned long long small_sum_max(unsigned long long a, int m, int *m_out,
+                                                            unsigned long long *scratch) {
+  constexpr int W = kSmallThreads / 64;
+  a = wave_inclusive_sum(a);
+  m = wave_inclusive_max(m);
+  if ((threadIdx.x & 63) == 63) {
+    scratch[threadIdx.x >> 6] = a;
+    scratch[W + (threadIdx.x >> 6)] = (unsigned long long)(unsigned)m;
+  }
+  __syncthreads();
+  unsigned long long s = 0;
+  int mm = 0;
+#pragma unroll
+  for (int w = 0; w < W; ++w) {
+    s += scratch[w];
+    mm = max(mm, (int)scratch[W + w]);
+  }
+  *m_out = mm;
+  return s;
+}
+
+// R exclusive prefix sums at once, each over the workgroup's threads: x[i] becomes the sum of the x[i] of the
+// threads before this one, total[i] the sum over all threads; only for i < n, the others (whose x[i] is 0
+// in every thread) get 0.  One barrier; same rule for `scratch` (R x kSmallThreads / 64 words).
+template <int R>
+__device__ __forceinline__ void small_exclusive_scans(unsigned long long (&x)[R], unsigned long long (&total)[R], int n,
+                                                      unsigned long long *scratch) {
+  constexpr int W = kSmallThreads / 64;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  unsigned long long incl[R];
+#pragma unroll
+  for (int i = 0; i < R; ++i) incl[i] = x[i];
+#pragma unroll
+  for (int i = 0; i < R; ++i)
+    if (i < n) incl[i] = wave_inclusive_sum(incl[i]);  // (uniform)
+  if (lane == 63) {
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+      if (i < n) scratch[i * W + wave] = incl[i];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    unsigned long long base = 0, sum = 0;
+    if (i < n) {
+#pragma unroll
+      for (int w = 0; w < W; ++w) {
+        const unsigned long long t = scratch[i * W + w];
+        if (w < wave) base += t;
+        sum += t;
+      }
+    }
+    total[i] = sum;
+    x[i] = base + incl[i] - x[i];
+  }
+}
+
+__device__ __forceinline__ void store_item(ScheduleItem *__restrict__ at, int row, int kbeg, int kend, int split_id,
+                                           int first_slot, int pieces, int piece) {
+  ScheduleItem it;
+  it.row = row;
+  it.kbeg = kbeg;
+  it.kend = kend;
+  it.split_id = split_id;
+  it.first_slot = first_slot;
+  it.pieces = pieces;
+  it.piece = piece;
+  it.pad = 0;
+  *at = it;
+}
+
+__global__ __launch_bounds__(kSmallThreads) void schedule_build_small_kernel(int m_vec, const int32_t *__restrict__ row_offsets,
+                                                                             long long slot_cap, int32_t *__restrict__ header,
+                                                                             ScheduleItem *__restrict__ items, long long item_cap,
+                                                                             int32_t *__restrict__ counters,
+                                                                             long long counters_per_cut_row) {
+  constexpr int R = kSmallRowsPerThread, W = kSmallThreads / 64;
+  // The sum and the scans of successive budgets each have words of their own: a wave may still be reading the
+  // previous step's.  (A wave that writes the words of two steps ago again has passed the barrier in between.)
+  __shared__ unsigned long long scratch_sum[2 * W], scratch_scan[2][R * W];
+  __shared__ int cut_first[kSmallCutRows], cut_row[kSmallCutRows], cut_beg[kSmallCutRows], cut_end[kSmallCutRows],
+      cut_pieces[kSmallCutRows];
+  int beg[R], end[R], steps[R];  // of row i * kSmallThreads + threadIdx.x; steps 0: no such row
+  unsigned long long steps_sum = 0;
+  int steps_max = 0;
+  int nvec = 0;  // (thread 0 only; fetched with the rows so that nothing waits for it later)
+  if (threadIdx.x == 0) nvec = row_offsets[m_vec];
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    const int r = i * kSmallThreads + (int)threadIdx.x;
+    beg[i] = row_offsets[min(r, m_vec)];
+    end[i] = row_offsets[min(r + 1, m_vec)];
+  }
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    steps[i] = i * kSmallThreads + (int)threadIdx.x < m_vec ? steps_of(end[i] - beg[i]) : 0;
+    steps_sum += (unsigned long long)steps[i];
+    steps_max = max(steps_max, steps[i]);
+  }
+  int longest;
+  const unsigned long long total = small_sum_max(steps_sum, steps_max, &longest, scratch_sum);
+  const long long by_items = (long long)((total + kScheduleTargetItems - 1) / kScheduleTargetItems);
+  const long long by_mean = (long long)((2 * total + (unsigned long long)m_vec - 1) / (unsigned long long)m_vec);
+  long long budget = max((long long)kScheduleMinBudget, max(by_items, by_mean));
+  const int blocks = (m_vec + kSmallThreads - 1) / kSmallThreads;  // blocks of rows that hold rows
+  int budget_i, pcs[R];
+  unsigned long long before[R], in_block[R];  // row words of the rows before this one in its block; of the whole block
+  unsigned long long all = 0;
+  for (int turn = 0;; turn ^= 1) {
+    budget_i = (int)min(budget, (long long)0x7fffffff);
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      pcs[i] = i < blocks ? pieces_of(steps[i], budget_i) : 0;  // (uniform: a wave skips the division)
+      before[i] = row_word(steps[i], pcs[i]);
+    }
+    small_exclusive_scans<R>(before, in_block, blocks, scratch_scan[turn]);
+    all = 0;
+#pragma unroll
+    for (int i = 0; i < R; ++i) all += in_block[i];
+    if ((long long)(all & 0xffffffffull) <= slot_cap || budget >= longest) break;
+    budget *= 2;
+  }
+  const long long slots = (long long)(all & 0xffffffffull);
+  const int split_rows = (int)((all >> 32) & 0xffffull);
+  if (threadIdx.x == 0) {
+    header[kHdrItems] = (int)(slots + (long long)(m_vec - split_rows));
+    header[kHdrSplitRows] = split_rows;
+    header[kHdrSlots] = (int)slots;
+    header[kHdrBudget] = budget_i;
+    header[kHdrNvec] = nvec;
+    header[kHdrMaxSteps] = longest;
+    header[kHdrTotalSteps] = (int)min(total, (unsigned long long)0x7fffffff);
+    header[7] = 0;
+  }
+  const long long counters_to_clear = (long long)split_rows * counters_per_cut_row;
+  for (long long i = threadIdx.x; i < counters_to_clear; i += kSmallThreads) counters[i] = 0;
+  const bool listed = split_rows <= kSmallCutRows;  // (uniform)
+  unsigned long long blocks_before = 0;
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    if (i >= blocks) break;  // (uniform)
+    const unsigned long long at = blocks_before + before[i];
+    blocks_before += in_block[i];
+    if (!steps[i]) continue;
+    const int r = i * kSmallThreads + (int)threadIdx.x;
+    if (pcs[i]) {
+      const long long first_slot = (long long)(at & 0xffffffffull);
+      const int split_id = (int)((at >> 32) & 0xffffull);
+      if (listed) {
+        cut_first[split_id] = (int)first_slot;
+        cut_row[split_id] = r;
+        cut_beg[split_id] = beg[i];
+        cut_end[split_id] = end[i];
+        cut_pieces[split_id] = pcs[i];
+      } else {
+        const int per = (steps[i] + pcs[i] - 1) / pcs[i];  // steps per panel: the panels of a row are even
+        for (int pc = 0; pc < pcs[i] && first_slot + pc < item_cap; ++pc) {
+          const int kbeg = min(end[i], beg[i] + pc * per * 32);
+          store_item(items + first_slot + pc, r, kbeg, min(end[i], kbeg + per * 32), split_id, (int)first_slot, pcs[i], pc);
+        }
+      }
+    } else {
+      const long long whole_at = slots + (long long)(at >> 48);
+      if (whole_at < item_cap) store_item(items + whole_at, r, beg[i], end[i], -1, 0, 0, 0);
+    }
+  }
+  if (!listed || slots == 0) return;  // (uniform)
+  __syncthreads();
+  for (long long slot = threadIdx.x; slot < slots && slot < item_cap; slot += kSmallThreads) {
+    int lo = 0, hi = split_rows - 1;  // the last cut row whose first panel is at or before this one
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (cut_first[mid] <= (int)slot)
+        lo = mid;
+      else
+        hi = mid - 1;
+    }
+    const int b = cut_beg[lo], e = cut_end[lo], p = cut_pieces[lo], first_slot = cut_first[lo], pc = (int)slot - first_slot;
+    const int per = (steps_of(e - b) + p - 1) / p;  // steps per panel: the panels of a row are even
+    const int kbeg = min(e, b + pc * per * 32);
+    store_item(items + slot, cut_row[lo], kbeg, min(e, kbeg + per * 32), lo, first_slot, p, pc);
+  }
+}
+
 hipError_t launch_schedule_measure(int m_vec, const int32_t *row_offsets, int budget, int64_t slot_cap, int32_t *header,
                                    hipStream_t stream) {
   hipLaunchKernelGGL(schedule_measure_kernel, dim3(1), dim3(kBuildThreads), 0, stream, m_vec, row_offsets, budget,
@@ -216,8 +458,13 @@ hipError_t launch_schedule_fill(int m_vec, const int32_t *row_offsets, const Sch
 
 hipError_t launch_schedule_build(int m_vec, const int32_t *row_offsets, int64_t slot_cap, const ScheduleView &view,
                                  int64_t item_cap, int64_t counters_per_cut_row, hipStream_t stream) {
-  hipLaunchKernelGGL(schedule_build_kernel, dim3(1), dim3(kBuildThreads), 0, stream, m_vec, row_offsets, (long long)slot_cap,
-                     view.header, view.items, (long long)item_cap, view.counters, (long long)counters_per_cut_row);
+  if (m_vec > 0 && m_vec <= kSmallRows)
+    hipLaunchKernelGGL(schedule_build_small_kernel, dim3(1), dim3(kSmallThreads), 0, stream, m_vec, row_offsets,
+                       (long long)slot_cap, view.header, view.items, (long long)item_cap, view.counters,
+                       (long long)counters_per_cut_row);
+  else
+    hipLaunchKernelGGL(schedule_build_kernel, dim3(1), dim3(kBuildThreads), 0, stream, m_vec, row_offsets, (long long)slot_cap,
+                       view.header, view.items, (long long)item_cap, view.counters, (long long)counters_per_cut_row);
   return hipGetLastError();
 }
 

@@ -65,6 +65,39 @@ def test_two_calls_in_a_row_the_second_smaller(oracle, built_library, V):
     assert not got2[:V].any()  # the empty first vector-row is written as zeros
 
 
+@pytest.mark.parametrize("m_vec", [64, 511, 513, 1025, 2049, 4096, 4097, 6000])
+def test_row_counts_either_side_of_the_schedule_builders(oracle, built_library, m_vec):
+    """Up to 4096 vector-rows the schedule is built from row offsets kept in registers (512 threads x 8), beyond
+    that by passes over memory; blocks of 512 or 1024 rows are scanned one after the other."""
+    L = _lib.lib()
+    vs = _pattern(m_vec, 2500, 8, seed=m_vec, long_rows=19)
+    B = synth.dense_rhs(2500, 64, seed=5)
+    got, want, cut = _both(L, vs, B, 64)
+    assert cut > 0
+    assert torch.equal(got, want)
+    ref = oracle.spmm(vs.m_vec, 8, 64, 2500, vs.row_offsets, vs.col_idx, vs.values, B, threads=8)
+    assert max_rel_err(got.cpu().numpy(), ref) <= TIGHT_F32
+
+
+def test_budget_doubled_until_the_panels_fit_the_static_scratch(oracle, built_library):
+    """With 64 column tiles the static scratch holds 64 partial tiles per column tile: 40 rows of 32 steps in a
+    pattern of 200 ask for 3 panels each (120), then 2 (80), and are then left whole."""
+    L = _lib.lib()
+    rng = np.random.default_rng(77)
+    lens = rng.integers(1, 33, 200)
+    lens[rng.choice(200, 40, replace=False)] = rng.integers(993, 1025, 40)
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cols = np.concatenate([rng.permutation(1500)[:n] for n in lens]).astype(np.int32)
+    vals = (rng.standard_normal(cols.size * 8) * 0.1).astype(np.float16)
+    vs = synth.VectorSparse(1600, 1500, 8, 200, off, cols, vals, cols.size * 8)
+    B = synth.dense_rhs(1500, 4096, seed=6)
+    got, want, cut = _both(L, vs, B, 4096)
+    assert cut == 40  # the plan has room for all 120 panels ...
+    ref = oracle.spmm(200, 8, 4096, 1500, off, cols, vals, B, threads=8)
+    assert max_rel_err(got.cpu().numpy(), ref) <= TIGHT_F32  # ... so the sums differ in their order, not in value
+    assert max_rel_err(want.cpu().numpy(), ref) <= TIGHT_F32
+
+
 def test_sizes_beyond_the_static_scratch_are_rejected(built_library):
     L = _lib.lib()
     one = 1  # rejected calls never dereference their pointers

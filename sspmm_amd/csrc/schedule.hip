@@ -5,6 +5,8 @@
 // MB; the work is bound by the latency of a dozen workgroup barriers, not by bytes).
 #include "schedule.h"
 
+#include "lane_ops.h"
+
 namespace sspmm {
 
 static constexpr int kBuildThreads = 1024;
@@ -220,48 +222,13 @@ __device__ __forceinline__ unsigned long long row_word(int steps, int pcs) {
   return steps == 0 ? 0ull : pcs ? (unsigned long long)(unsigned)pcs + (1ull << 32) : (1ull << 48);
 }
 
-// Lane moves inside the vector unit (a permute through the LDS pipe costs this kernel, which has one wave or two
-// per SIMD and nothing to hide a latency behind, some 70 cycles each).  CTRL: 0x110 + n = from the lane n below in
-// the same row of 16 lanes, 0x142 / 0x143 = lane 15 of the row below / lane 31, to the rows ROW_MASK names; lanes
-// without a source, and rows not named, get 0.
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ int lanes_below(int v) {
-  return __builtin_amdgcn_update_dpp(0, v, CTRL, ROW_MASK, 0xf, true);
-}
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ unsigned long long lanes_below(unsigned long long v) {
-  const unsigned lo = (unsigned)lanes_below<CTRL, ROW_MASK>((int)(unsigned)v);
-  const unsigned hi = (unsigned)lanes_below<CTRL, ROW_MASK>((int)(unsigned)(v >> 32));
-  return ((unsigned long long)hi << 32) | lo;
-}
-// Sum of v over lanes 0 .. own lane of the wave (all 64 lanes active).
-__device__ __forceinline__ unsigned long long wave_inclusive_sum(unsigned long long v) {
-  v += lanes_below<0x111, 0xf>(v);
-  v += lanes_below<0x112, 0xf>(v);
-  v += lanes_below<0x114, 0xf>(v);
-  v += lanes_below<0x118, 0xf>(v);
-  v += lanes_below<0x142, 0xa>(v);  // rows 1 and 3 take the sum of the row below
-  v += lanes_below<0x143, 0xc>(v);  // rows 2 and 3 take the sum of rows 0 and 1
-  return v;
-}
-// Maximum of v (not negative) over lanes 0 .. own lane.
-__device__ __forceinline__ int wave_inclusive_max(int v) {
-  v = max(v, lanes_below<0x111, 0xf>(v));
-  v = max(v, lanes_below<0x112, 0xf>(v));
-  v = max(v, lanes_below<0x114, 0xf>(v));
-  v = max(v, lanes_below<0x118, 0xf>(v));
-  v = max(v, lanes_below<0x142, 0xa>(v));
-  v = max(v, lanes_below<0x143, 0xc>(v));
-  return v;
-}
-
 // Sum over the workgroup of a 64-bit value per thread and maximum of an int per thread.  One barrier; `scratch`
 // (2 x kSmallThreads / 64 words) must not be in use by an earlier step that some wave may still be reading.
 __device__ __forceinline__ unsigned long long small_sum_max(unsigned long long a, int m, int *m_out,
                                                             unsigned long long *scratch) {
   constexpr int W = kSmallThreads / 64;
   a = wave_inclusive_sum(a);
-  m = wave_inclusive_max(m);
+  m = (int)wave_inclusive_max((uint32_t)m);  // (not negative)
   if ((threadIdx.x & 63) == 63) {
     scratch[threadIdx.x >> 6] = a;
     scratch[W + (threadIdx.x >> 6)] = (unsigned long long)(unsigned)m;

@@ -42,6 +42,7 @@
 
 #include <mutex>
 
+#include "lane_ops.h"
 #include "svc_kernels.h"
 
 namespace sspmm {
@@ -113,15 +114,10 @@ __device__ __forceinline__ void place(u64 *table, uint32_t mask, uint32_t key, u
 template <int THREADS>
 __device__ __forceinline__ int block_exclusive_scan(int x, int *total, int *scratch) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  int incl = x;
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const int y = __shfl_up(incl, d, 64);
-    if (lane >= d) incl += y;
-  }
+  const int incl = (int)wave_inclusive_sum((uint32_t)x);
   constexpr int WAVES = THREADS / 64;
   if (WAVES == 1) {
-    *total = __shfl(incl, 63, 64);
+    *total = (int)from_last_lane((uint32_t)incl);
     return incl - x;
   }
   __syncthreads();  // scratch may still be read from a previous call
@@ -136,6 +132,35 @@ __device__ __forceinline__ int block_exclusive_scan(int x, int *total, int *scra
   }
   *total = sum;
   return base + incl - x;
+}
+
+// The same for a flag per thread, for loops that call it every trip: the rank comes from the wave's ballot, and
+// consecutive calls alternate between two halves of `scratch` (2 x THREADS / 64 ints; `turn` is the caller's
+// counter, starting anywhere), so that one barrier per call is enough: a wave that comes round to a half again
+// has passed the barrier of the call in between, which every wave reaches only after it has read that half.
+template <int THREADS>
+__device__ __forceinline__ int block_rank_of_flag(bool flag, int *total, int *scratch, int &turn) {
+  constexpr int WAVES = THREADS / 64;
+  const unsigned long long m = __ballot(flag);
+  const int in_wave = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+  if (WAVES == 1) {
+    *total = (int)__popcll(m);
+    return in_wave;
+  }
+  const int wave = threadIdx.x >> 6;
+  int *mine = scratch + (turn & 1) * WAVES;
+  ++turn;
+  if ((threadIdx.x & 63) == 0) mine[wave] = (int)__popcll(m);
+  __syncthreads();
+  int base = 0, sum = 0;
+#pragma unroll
+  for (int wv = 0; wv < WAVES; ++wv) {
+    const int t = mine[wv];
+    if (wv < wave) base += t;
+    sum += t;
+  }
+  *total = sum;
+  return base + in_wave;
 }
 
 __device__ __forceinline__ uint32_t resize_threshold(uint32_t slots) { return (3u * (slots - 1u) + 4u) / 5u; }
@@ -434,6 +459,7 @@ __device__ __forceinline__ void list_store(int *list, int idx, int v) {
 struct OrderCheck {
   bool on;            // off: nothing is compared or kept (both answers "no")
   int *before;        // LDS copy of the previous construction's input, or null
+  int *wave_words;    // LDS, one int per wave, free between the barriers inside a compaction
   bool same_as_input;   // out: every key landed on the list entry that already held it
   bool same_as_before;  // out: ... on the entry of `before` that held it (meaningful when `before` was that input)
 };
@@ -463,14 +489,9 @@ __device__ __forceinline__ int compact_table32(const Table32 &t, uint32_t slots,
     for (uint32_t w0 = 0; w0 < words; w0 += 64) {
       const uint32_t w = w0 + lane;
       const uint32_t c = w < words ? wcount[w] : 0u;
-      uint32_t incl = c;
-#pragma unroll
-      for (int d = 1; d < 64; d <<= 1) {
-        const uint32_t y = __shfl_up(incl, d, 64);
-        if (lane >= d) incl += y;
-      }
+      const uint32_t incl = wave_inclusive_sum(c);
       if (w < words) wcount[w] = carry + incl - c;
-      carry += __shfl(incl, 63, 64);
+      carry += from_last_lane(incl);
     }
     if (lane == 0) wcount[words] = carry;  // number of keys in the table
   }
@@ -508,11 +529,17 @@ __device__ __forceinline__ int compact_table32(const Table32 &t, uint32_t slots,
   }
   const int kept = (int)wcount[words];
   if (check) {
-    check->same_as_input = __syncthreads_or(moved) == 0;
-    check->same_as_before = check->before != nullptr && __syncthreads_or(moved_before) == 0;
-  } else {
+    // both answers through one word per wave (the library's workgroup-wide "or" is three barriers per answer)
+    const int mine = (__ballot(moved) != 0 ? 1 : 0) | (__ballot(moved_before) != 0 ? 2 : 0);
+    if (lane == 0) check->wave_words[wave] = mine;
     __syncthreads();
+    int any = 0;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) any |= check->wave_words[w];
+    check->same_as_input = (any & 1) == 0;
+    check->same_as_before = check->before != nullptr && (any & 2) == 0;
   }
+  __syncthreads();  // (also: the wave words may be written again)
   return kept;
 }
 
@@ -684,9 +711,10 @@ __global__ __launch_bounds__(THREADS) void svc_merge_fast_kernel(const SvcArgs a
   // and at most one of them is carried out, when new keys arrive or at the end.
   // The comparisons cost a few per cent of a construction, so they are made where they can pay: when the row
   // brought nothing new itself, or when the row behind it is empty.
-  int period = 0, owed = 0;
+  int period = 0, owed = 0, scan_turn = 0;
   bool before_is_input = false;  // list_before holds the input of the construction that produced the list
   OrderCheck check;
+  check.wave_words = scratch;
   auto construct = [&](bool without_new_keys, bool compare) {
     const bool had_input = before_is_input;
     check.on = compare;
@@ -708,7 +736,7 @@ __global__ __launch_bounds__(THREADS) void svc_merge_fast_kernel(const SvcArgs a
         is_new = k < (uint32_t)a.K && ((slots == 0) || find_slot32(t, slots - 1u, k) < 0);
       }
       int total;
-      const int rank = block_exclusive_scan<THREADS>(is_new ? 1 : 0, &total, scratch);
+      const int rank = block_rank_of_flag<THREADS>(is_new, &total, scratch, scan_turn);
       if (is_new && n + appended + rank < cap) list_store<LIST_IN_LDS>(list, n + appended + rank, (int)k);
       appended += total;
     }

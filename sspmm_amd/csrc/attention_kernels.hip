@@ -12,6 +12,7 @@
 #include <stdint.h>
 
 #include "attention_kernels.h"
+#include "lane_ops.h"
 
 namespace sspmm {
 
@@ -224,16 +225,8 @@ hipError_t launch_sddmm(const SddmmArgs &a, int V, hipStream_t stream) {
 // ---------------------------------------------------------------------------------- softmax
 namespace {
 
-__device__ __forceinline__ float wave_max(float x) {
-#pragma unroll
-  for (int d = 32; d >= 1; d >>= 1) x = fmaxf(x, __shfl_xor(x, d, 64));
-  return x;
-}
-__device__ __forceinline__ float wave_sum(float x) {
-#pragma unroll
-  for (int d = 32; d >= 1; d >>= 1) x += __shfl_xor(x, d, 64);
-  return x;
-}
+__device__ __forceinline__ float wave_max(float x) { return wave_max_all(x); }
+__device__ __forceinline__ float wave_sum(float x) { return wave_sum_all(x); }
 
 template <int V>
 struct VecLoad;  // the V halfs of one stored vector

@@ -48,6 +48,31 @@ __device__ __forceinline__ uint32_t wave_inclusive_max(uint32_t v) {
   return v;
 }
 
+// The same moves for floats, with what a lane without a source (or a row not named) gets instead given by the caller.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float lanes_below_or(float v, float otherwise) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(otherwise), __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
+}
+// Maximum / sum of x over all 64 lanes, in every lane (the running value reaches lane 63, which is then read out).
+__device__ __forceinline__ float wave_max_all(float x) {
+  x = fmaxf(x, lanes_below_or<0x111, 0xf>(x, x));
+  x = fmaxf(x, lanes_below_or<0x112, 0xf>(x, x));
+  x = fmaxf(x, lanes_below_or<0x114, 0xf>(x, x));
+  x = fmaxf(x, lanes_below_or<0x118, 0xf>(x, x));
+  x = fmaxf(x, lanes_below_or<0x142, 0xa>(x, x));
+  x = fmaxf(x, lanes_below_or<0x143, 0xc>(x, x));
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), 63));
+}
+__device__ __forceinline__ float wave_sum_all(float x) {
+  x += lanes_below_or<0x111, 0xf>(x, 0.f);
+  x += lanes_below_or<0x112, 0xf>(x, 0.f);
+  x += lanes_below_or<0x114, 0xf>(x, 0.f);
+  x += lanes_below_or<0x118, 0xf>(x, 0.f);
+  x += lanes_below_or<0x142, 0xa>(x, 0.f);
+  x += lanes_below_or<0x143, 0xc>(x, 0.f);
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), 63));
+}
+
 // The value lane 63 holds, in every lane.
 __device__ __forceinline__ uint32_t from_last_lane(uint32_t v) { return (uint32_t)__builtin_amdgcn_readlane((int)v, 63); }
 

@@ -438,6 +438,28 @@ __device__ __attribute__((noinline)) void place32_lds(lds_u32 *slots, uint32_t k
 __device__ __forceinline__ void place32(const Table32 &t, uint32_t mask, uint32_t key, uint32_t order) {
   place32_lds((lds_u32 *)t.slots, t.key_bits, mask, key, order);
 }
+// The same placement inlined, for the phases one wave runs on its own: alone on its SIMD a wave pays every
+// instruction in full, the call and its register shuffling included, and those phases have two call sites.
+__device__ __forceinline__ void place32_inline(const Table32 &t, uint32_t mask, uint32_t key, uint32_t order) {
+  uint32_t mine = (order << t.key_bits) | key;
+  uint32_t i, perturb, lin;
+  probe_start(key, mask, i, perturb, lin);
+  for (;;) {
+    const uint32_t s0 = i + lin;
+    const uint32_t old = __hip_atomic_fetch_min(t.slots + s0, mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (old == kEmpty32 || ((old ^ mine) & t.key_mask) == 0) return;
+    if (old > mine) {
+      mine = old;
+      probe_start(old & t.key_mask, mask, i, perturb, lin);
+      const uint32_t d = s0 - i;
+      if ((d <= 9u) & ((i + 9u <= mask) | (d == 0u)))
+        lin = d;
+      else
+        while (i + lin != s0) probe_next(mask, i, perturb, lin);
+    }
+    probe_next(mask, i, perturb, lin);
+  }
+}
 
 // The key list lives in LDS, or in the workspace where other waves of the group wrote it: those
 // accesses go past the L1.
@@ -558,6 +580,23 @@ struct TableRegions {
 template <int STRIDE, bool LIST_IN_LDS>
 __device__ __forceinline__ void phase_insert(const Table32 &t, uint32_t mask, const int *list, int cnt, const uint32_t *old_table,
                                              uint32_t old_slots, int prev_cnt, int me) {
+  if (LIST_IN_LDS) {
+    // every key comes from LDS: nothing to fetch ahead, and two inlined placements instead of sixteen calls
+    uint32_t first = 0;
+    if (old_table != nullptr) {
+      first = old_slots;
+#pragma unroll 1
+      for (uint32_t s = me; s < old_slots; s += STRIDE) {
+        const uint32_t x = old_table[s];
+        if (x != kEmpty32) place32_inline(t, mask, x & t.key_mask, s);
+      }
+    }
+    me = (me + STRIDE - (int)(first % (uint32_t)STRIDE)) % STRIDE;
+#pragma unroll 1
+    for (int idx = prev_cnt + me; idx < cnt; idx += STRIDE)
+      place32_inline(t, mask, (uint32_t)list[idx], first + (uint32_t)(idx - prev_cnt));
+    return;
+  }
   if (old_table != nullptr) {
     for (uint32_t base = me; base < old_slots; base += 8 * STRIDE) {
       uint32_t x8[8];
@@ -588,6 +627,25 @@ __device__ __forceinline__ void phase_insert(const Table32 &t, uint32_t mask, co
       if (idx < cnt) place32(t, mask, (uint32_t)k8[j], first_index + (uint32_t)(idx - prev_cnt));
     }
   }
+}
+
+// The same inserts by one wave on its own (tables of up to kSoloSlots slots: a lane has a key or two).
+template <bool LIST_IN_LDS>
+__device__ __forceinline__ void phase_insert_solo(const Table32 &t, uint32_t mask, const int *list, int cnt,
+                                                  const uint32_t *old_table, uint32_t old_slots, int prev_cnt, int lane) {
+  uint32_t first_index = 0;
+  if (old_table != nullptr) {
+    first_index = old_slots;
+#pragma unroll 1
+    for (uint32_t s = lane; s < old_slots; s += 64) {
+      const uint32_t x = old_table[s];
+      if (x != kEmpty32) place32_inline(t, mask, x & t.key_mask, s);
+    }
+  }
+  const int me = (lane + 64 - (int)(first_index % 64u)) % 64;
+#pragma unroll 1
+  for (int idx = prev_cnt + me; idx < cnt; idx += 64)
+    place32_inline(t, mask, (uint32_t)list_load<LIST_IN_LDS>(list, idx), first_index + (uint32_t)(idx - prev_cnt));
 }
 
 // One `set(list)` of CPython on the keys list[0 .. n): leaves the final table in t (entries
@@ -642,7 +700,7 @@ __device__ __forceinline__ uint32_t rebuild_set32(Table32 &t, const TableRegions
         for (uint32_t s = lane; s < slots; s += 64) nt[s] = kEmpty32;
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");  // the wave's LDS operations execute in order
         __builtin_amdgcn_wave_barrier();
-        phase_insert<64, LIST_IN_LDS>(t, mask, list, cnt, cur, old_slots, prev_cnt, lane);
+        phase_insert_solo<LIST_IN_LDS>(t, mask, list, cnt, cur, old_slots, prev_cnt, lane);
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
         __builtin_amdgcn_wave_barrier();
       }
@@ -833,7 +891,7 @@ __global__ __launch_bounds__(1024) void svc_scan_classify_kernel(int m_vec, int3
       if (members == 0) continue;  // uniform over the wave
       int at = 0;
       if (lane == 0) at = atomicAdd(&filed[c], __popcll(members));
-      at = __shfl(at, 0, 64);
+      at = __builtin_amdgcn_readfirstlane(at);
       if (cls == c) class_lists[(int64_t)c * list_stride + at + __popcll(members & ((1ull << lane) - 1ull))] = i;
     }
   }

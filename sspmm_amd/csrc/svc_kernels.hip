@@ -438,17 +438,31 @@ __device__ __attribute__((noinline)) void place32_lds(lds_u32 *slots, uint32_t k
 __device__ __forceinline__ void place32(const Table32 &t, uint32_t mask, uint32_t key, uint32_t order) {
   place32_lds((lds_u32 *)t.slots, t.key_bits, mask, key, order);
 }
-// The same placement inlined, for the phases one wave runs on its own: alone on its SIMD a wave pays every
-// instruction in full, the call and its register shuffling included, and those phases have two call sites.
-__device__ __forceinline__ void place32_inline(const Table32 &t, uint32_t mask, uint32_t key, uint32_t order) {
+// The same placement inlined, for keys that come from LDS (two call sites per phase): alone on its SIMD a wave
+// pays every instruction in full, the call and its register shuffling included, and with four waves per SIMD a round
+// of placements is bound by the instructions the waves issue, not by the LDS.
+//
+// Together with its attempt on a slot a key reads the three slots behind it: an entry only ever gets smaller
+// (atomic min), so a slot that holds an earlier key now is lost to this key for good and can be passed without an
+// atomic; if the attempt fails, the next one goes to the first of the three that is free or holds a later key, or to
+// the slot behind them.  The reads are in flight with the atomic and add nothing to the round trip; rounds, and
+// with them the wave-rounds a phase costs, come down to about half.  Passing over slots unseen would also pass
+// over an earlier copy of the same key, which only a row that repeats a column (invalid input) can bring:
+// `safe` = true switches the passing off and the test for the same key on (the caller falls back to it when a
+// group turns out to hold more keys than distinct columns).
+__device__ __forceinline__ void place32_inline(const Table32 &t, uint32_t mask, uint32_t key, uint32_t order, bool safe) {
   uint32_t mine = (order << t.key_bits) | key;
   uint32_t i, perturb, lin;
   probe_start(key, mask, i, perturb, lin);
   for (;;) {
     const uint32_t s0 = i + lin;
     const uint32_t old = __hip_atomic_fetch_min(t.slots + s0, mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    if (old == kEmpty32 || ((old ^ mine) & t.key_mask) == 0) return;
+    // (slots behind the table's end are read and not used: every table is followed by other LDS of the group)
+    const uint32_t x1 = t.slots[s0 + 1u], x2 = t.slots[s0 + 2u], x3 = t.slots[s0 + 3u];
+    if (old == kEmpty32) return;
+    if (safe && ((old ^ mine) & t.key_mask) == 0) return;  // a repeated key (invalid row)
     if (old > mine) {
+      // a later entry sat here: carry it on from this slot of its own probe sequence
       mine = old;
       probe_start(old & t.key_mask, mask, i, perturb, lin);
       const uint32_t d = s0 - i;
@@ -457,6 +471,13 @@ __device__ __forceinline__ void place32_inline(const Table32 &t, uint32_t mask, 
       else
         while (i + lin != s0) probe_next(mask, i, perturb, lin);
     }
+    // slots s0 + 1 .. s0 + 3 are the next three of the sequence, and the one behind them the fourth, if they are
+    // inside the window of ten
+    const bool can = (lin <= 5u) & (i + 9u <= mask) & !safe;
+    uint32_t k = x3 < mine ? 3u : 2u;
+    k = x2 < mine ? k : 1u;
+    k = x1 < mine ? k : 0u;
+    lin += can ? k : 0u;
     probe_next(mask, i, perturb, lin);
   }
 }
@@ -579,7 +600,7 @@ struct TableRegions {
 // arrives before an earlier one; keys are fetched eight at a time ahead of the inserts.
 template <int STRIDE, bool LIST_IN_LDS>
 __device__ __forceinline__ void phase_insert(const Table32 &t, uint32_t mask, const int *list, int cnt, const uint32_t *old_table,
-                                             uint32_t old_slots, int prev_cnt, int me) {
+                                             uint32_t old_slots, int prev_cnt, int me, bool safe) {
   if (LIST_IN_LDS) {
     // every key comes from LDS: nothing to fetch ahead, and two inlined placements instead of sixteen calls
     uint32_t first = 0;
@@ -588,13 +609,13 @@ __device__ __forceinline__ void phase_insert(const Table32 &t, uint32_t mask, co
 #pragma unroll 1
       for (uint32_t s = me; s < old_slots; s += STRIDE) {
         const uint32_t x = old_table[s];
-        if (x != kEmpty32) place32_inline(t, mask, x & t.key_mask, s);
+        if (x != kEmpty32) place32_inline(t, mask, x & t.key_mask, s, safe);
       }
     }
     me = (me + STRIDE - (int)(first % (uint32_t)STRIDE)) % STRIDE;
 #pragma unroll 1
     for (int idx = prev_cnt + me; idx < cnt; idx += STRIDE)
-      place32_inline(t, mask, (uint32_t)list[idx], first + (uint32_t)(idx - prev_cnt));
+      place32_inline(t, mask, (uint32_t)list[idx], first + (uint32_t)(idx - prev_cnt), safe);
     return;
   }
   if (old_table != nullptr) {
@@ -632,20 +653,21 @@ __device__ __forceinline__ void phase_insert(const Table32 &t, uint32_t mask, co
 // The same inserts by one wave on its own (tables of up to kSoloSlots slots: a lane has a key or two).
 template <bool LIST_IN_LDS>
 __device__ __forceinline__ void phase_insert_solo(const Table32 &t, uint32_t mask, const int *list, int cnt,
-                                                  const uint32_t *old_table, uint32_t old_slots, int prev_cnt, int lane) {
+                                                  const uint32_t *old_table, uint32_t old_slots, int prev_cnt, int lane,
+                                                  bool safe) {
   uint32_t first_index = 0;
   if (old_table != nullptr) {
     first_index = old_slots;
 #pragma unroll 1
     for (uint32_t s = lane; s < old_slots; s += 64) {
       const uint32_t x = old_table[s];
-      if (x != kEmpty32) place32_inline(t, mask, x & t.key_mask, s);
+      if (x != kEmpty32) place32_inline(t, mask, x & t.key_mask, s, safe);
     }
   }
   const int me = (lane + 64 - (int)(first_index % 64u)) % 64;
 #pragma unroll 1
   for (int idx = prev_cnt + me; idx < cnt; idx += 64)
-    place32_inline(t, mask, (uint32_t)list_load<LIST_IN_LDS>(list, idx), first_index + (uint32_t)(idx - prev_cnt));
+    place32_inline(t, mask, (uint32_t)list_load<LIST_IN_LDS>(list, idx), first_index + (uint32_t)(idx - prev_cnt), safe);
 }
 
 // One `set(list)` of CPython on the keys list[0 .. n): leaves the final table in t (entries
@@ -660,7 +682,8 @@ static constexpr uint32_t kSoloSlots = 128;
 // check: see compact_table32; both answers are "no" when the list was rewritten between phases, and
 // check.before is then cleared (what it would receive is not the input).
 template <int THREADS, bool LIST_IN_LDS>
-__device__ __forceinline__ uint32_t rebuild_set32(Table32 &t, const TableRegions &reg, int *list, int &n, OrderCheck &check) {
+__device__ __forceinline__ uint32_t rebuild_set32(Table32 &t, const TableRegions &reg, int *list, int &n, OrderCheck &check,
+                                                  bool safe) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   uint32_t slots = 8, old_slots = 0;
@@ -700,7 +723,7 @@ __device__ __forceinline__ uint32_t rebuild_set32(Table32 &t, const TableRegions
         for (uint32_t s = lane; s < slots; s += 64) nt[s] = kEmpty32;
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");  // the wave's LDS operations execute in order
         __builtin_amdgcn_wave_barrier();
-        phase_insert_solo<LIST_IN_LDS>(t, mask, list, cnt, cur, old_slots, prev_cnt, lane);
+        phase_insert_solo<LIST_IN_LDS>(t, mask, list, cnt, cur, old_slots, prev_cnt, lane, safe);
         __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
         __builtin_amdgcn_wave_barrier();
       }
@@ -708,7 +731,7 @@ __device__ __forceinline__ uint32_t rebuild_set32(Table32 &t, const TableRegions
     } else {
       for (uint32_t s = tid; s < slots; s += THREADS) nt[s] = kEmpty32;
       __syncthreads();
-      phase_insert<THREADS, LIST_IN_LDS>(t, mask, list, cnt, cur, old_slots, prev_cnt, tid);
+      phase_insert<THREADS, LIST_IN_LDS>(t, mask, list, cnt, cur, old_slots, prev_cnt, tid, safe);
       __syncthreads();
     }
     if (n < (int)thr) {
@@ -771,16 +794,26 @@ __global__ __launch_bounds__(THREADS) void svc_merge_fast_kernel(const SvcArgs a
   // brought nothing new itself, or when the row behind it is empty.
   int period = 0, owed = 0, scan_turn = 0;
   bool before_is_input = false;  // list_before holds the input of the construction that produced the list
+  // The placements pass over slots without looking for their own key there (place32_inline), which is right as long
+  // as no row repeats a column.  A row that does makes the group's keys outnumber its distinct columns sooner or
+  // later (`cap`, counted beforehand): the group is then done again with the placements that look.
+  bool safe = false;
   OrderCheck check;
   check.wave_words = scratch;
   auto construct = [&](bool without_new_keys, bool compare) {
     const bool had_input = before_is_input;
     check.on = compare;
     check.before = list_before;
-    slots = rebuild_set32<THREADS, LIST_IN_LDS>(t, reg, list, n, check);
+    slots = rebuild_set32<THREADS, LIST_IN_LDS>(t, reg, list, n, check, safe);
     period = check.same_as_input ? 1 : (without_new_keys && had_input && check.same_as_before) ? 2 : 0;
     before_is_input = check.before != nullptr;
   };
+  for (;;) {
+  bool overfull = false;
+  n = 0;
+  slots = 0;
+  period = owed = 0;
+  before_is_input = false;
   for (int row = r0; row < r1; ++row) {
     const int b = rows.start(row - r0), e = rows.start(row - r0 + 1);
     // acc + row: append the row's columns that are not in acc yet, in row order
@@ -798,8 +831,10 @@ __global__ __launch_bounds__(THREADS) void svc_merge_fast_kernel(const SvcArgs a
       if (is_new && n + appended + rank < cap) list_store<LIST_IN_LDS>(list, n + appended + rank, (int)k);
       appended += total;
     }
+    overfull = appended > cap - n;
     appended = min(appended, cap - n);  // the cap only bites for invalid input (a row that repeats a column)
     __syncthreads();
+    if (overfull && !safe) break;
     if (appended == 0 && slots != 0) {
       if (period == 1) continue;
       if (period == 2) {
@@ -815,6 +850,9 @@ __global__ __launch_bounds__(THREADS) void svc_merge_fast_kernel(const SvcArgs a
     }
     n += appended;
     construct(false, row + 1 < r1 && rows.start(row - r0 + 1) == rows.start(row - r0 + 2));
+  }
+  if (!overfull || safe) break;
+  safe = true;
   }
   if (owed) construct(true, false);
 
@@ -1001,9 +1039,11 @@ static hipError_t launch_fast_class(const SvcArgs &a, int grid, int cls, int cls
   uint32_t small_slots = slots / 4u;
   // (a key list in LDS has a second copy behind it: the input of the latest construction)
   const size_t list_bytes = LIST_IN_LDS ? (size_t)hi * 8 : 0;
-  while (128 + ((size_t)slots + small_slots) * 4 + list_bytes > 160 * 1024) small_slots /= 4u;
+  // (16 bytes behind everything: a placement reads up to three slots past the end of its table)
+  constexpr size_t kTail = 16;
+  while (128 + ((size_t)slots + small_slots) * 4 + list_bytes + kTail > 160 * 1024) small_slots /= 4u;
   if (small_slots < slots / 64u + 1u) return hipErrorInvalidValue;
-  size_t lds = 128 + ((size_t)slots + small_slots) * 4 + list_bytes;
+  size_t lds = 128 + ((size_t)slots + small_slots) * 4 + list_bytes + kTail;
   if (lds < min_lds) lds = min_lds;  // asking for more than half of a CU's LDS keeps a workgroup alone on its CU
   auto kern = svc_merge_fast_kernel<THREADS, LIST_IN_LDS>;
   if (lds > 64 * 1024) {

@@ -386,9 +386,10 @@ __global__ __launch_bounds__(THREADS) void svc_merge_cpython_kernel(const SvcArg
 // bits of insertion index: enough for 19 660 keys, the largest set CPython keeps in a 32 768-slot
 // table.  Halving the entries brings groups of up to 19 660 keys into LDS (a 128 KB table; their
 // key list stays in the workspace) and makes the atomics 32-bit.  The compaction of a phase is done
-// one 64-slot word per wave iteration: a ballot gives the occupancy mask, a first pass leaves the
-// population of every word, wave 0 turns them into running counts, and a second pass writes
-// list[count[word] + rank in word] = key, so nothing is scanned per thread.
+// one 64-slot word per wave iteration: a ballot gives the occupancy mask; every wave takes a contiguous
+// run of words and counts its keys in a first pass, the counts of the waves before it give its starting
+// rank (one barrier), and a second pass writes list[running count + rank in word] = key, so nothing
+// is scanned per thread.
 static constexpr uint32_t kEmpty32 = 0xffffffffu;
 
 struct Table32 {
@@ -495,7 +496,7 @@ __device__ __forceinline__ void list_store(int *list, int idx, int v) {
 }
 
 // Writes the keys of a table to list[] in slot order and returns their number; with `final`, the
-// table entries are rewritten as (rank, key).  wcount: slots / 64 + 1 words of LDS.  Contains
+// table entries are rewritten as (rank, key).  wcount: one word of LDS per wave.  Contains
 // barriers; the table must be complete (a barrier behind the last insert) on entry.
 // check (optional): compares the new order with the list as it was (the construction's input) and with the input
 // of the construction before (check->before, if kept), and leaves the old list there for the next comparison.
@@ -510,51 +511,52 @@ template <int THREADS, bool LIST_IN_LDS>
 __device__ __forceinline__ int compact_table32(const Table32 &t, uint32_t slots, uint32_t *wcount, int *list, bool final,
                                                OrderCheck *check = nullptr) {
   constexpr int WAVES = THREADS / 64;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const uint32_t words = slots >= 64u ? slots / 64u : 1u;
+  // A wave takes a contiguous run of 64-slot words, so that the number of keys before its first word is a sum over
+  // the waves before it: one barrier, and no wave scans the words' counts for the others.
+  const uint32_t per_wave = (words + WAVES - 1u) / WAVES;
+  const uint32_t w_beg = min(words, (uint32_t)wave * per_wave), w_end = min(words, w_beg + per_wave);
   // (four words per trip, their loads in flight together: these passes are chains of LDS round trips)
-  for (uint32_t w0 = wave; w0 < words; w0 += 4 * WAVES) {
+  uint32_t in_wave = 0;
+  for (uint32_t w0 = w_beg; w0 < w_end; w0 += 4) {
     uint32_t x[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const uint32_t s = (w0 + j * WAVES) * 64u + lane;
-      x[j] = s < slots ? t.slots[s] : kEmpty32;
+      const uint32_t s = (w0 + j) * 64u + lane;
+      x[j] = (w0 + j < w_end && s < slots) ? t.slots[s] : kEmpty32;
     }
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const unsigned long long m = __ballot(x[j] != kEmpty32);
-      if (lane == 0 && w0 + j * WAVES < words) wcount[w0 + j * WAVES] = (uint32_t)__popcll(m);
+    for (int j = 0; j < 4; ++j) in_wave += (uint32_t)__popcll(__ballot(x[j] != kEmpty32));
+  }
+  uint32_t running = 0, kept_u = in_wave;  // keys before this wave's words; keys in the table
+  if (WAVES > 1) {
+    if (lane == 0) wcount[wave] = in_wave;
+    __syncthreads();
+    kept_u = 0;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+      const uint32_t c = wcount[w];
+      if (w < wave) running += c;
+      kept_u += c;
     }
   }
-  __syncthreads();
-  if (wave == 0) {  // running counts over the words
-    uint32_t carry = 0;
-    for (uint32_t w0 = 0; w0 < words; w0 += 64) {
-      const uint32_t w = w0 + lane;
-      const uint32_t c = w < words ? wcount[w] : 0u;
-      const uint32_t incl = wave_inclusive_sum(c);
-      if (w < words) wcount[w] = carry + incl - c;
-      carry += from_last_lane(incl);
-    }
-    if (lane == 0) wcount[words] = carry;  // number of keys in the table
-  }
-  __syncthreads();
   int moved = 0, moved_before = 0;
-  for (uint32_t w0 = wave; w0 < words; w0 += 4 * WAVES) {
-    uint32_t x[4], before[4];
+  for (uint32_t w0 = w_beg; w0 < w_end; w0 += 4) {
+    uint32_t x[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const uint32_t w = w0 + j * WAVES;
-      const uint32_t s = w * 64u + lane;
-      x[j] = s < slots ? t.slots[s] : kEmpty32;
-      before[j] = w < words ? wcount[w] : 0u;
+      const uint32_t s = (w0 + j) * 64u + lane;
+      x[j] = (w0 + j < w_end && s < slots) ? t.slots[s] : kEmpty32;
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const uint32_t s = (w0 + j * WAVES) * 64u + lane;
+      const uint32_t s = (w0 + j) * 64u + lane;
       const bool occ = x[j] != kEmpty32;
       const unsigned long long m = __ballot(occ);
-      const uint32_t rank = before[j] + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+      const uint32_t rank = running + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+      running += (uint32_t)__popcll(m);
       if (occ) {
         // (entry `rank` of either list is written by this thread alone, so what it reads here is the old content)
         if (check) {
@@ -570,7 +572,7 @@ __device__ __forceinline__ int compact_table32(const Table32 &t, uint32_t slots,
       }
     }
   }
-  const int kept = (int)wcount[words];
+  const int kept = (int)kept_u;
   if (check) {
     // both answers through one word per wave (the library's workgroup-wide "or" is three barriers per answer)
     const int mine = (__ballot(moved) != 0 ? 1 : 0) | (__ballot(moved_before) != 0 ? 2 : 0);

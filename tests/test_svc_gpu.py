@@ -179,6 +179,33 @@ def test_a_row_that_repeats_a_column_stays_inside_its_group(built_library):
     assert ((vcol >= 0) & (vcol < K)).all() and np.isin(vval, [0.0, 1.0]).all()
 
 
+@pytest.mark.parametrize("sizes", [[5, 300, 0, 1500, 40, 2, 9, 700], [3, 12, 0, 25, 7, 1, 30, 16], [2400, 0, 0, 4, 0, 1100, 0, 600],
+                                   [9000, 0, 40, 3000, 0, 0, 2, 0]])
+def test_a_repeated_column_is_kept_once(built_library, sizes):
+    """Invalid input again: whatever the order, a group's vectors are its distinct columns, each once, and every
+    non-zero lands in the vector of its column (the placements that pass over slots unseen are given up for the
+    group as soon as it holds more keys than distinct columns, and the group is done again with those that look)."""
+    rng = np.random.default_rng(sum(sizes))
+    K, V = 16384, 8
+    rows = []
+    for g in range(3):
+        for n in sizes:
+            c = rng.choice(K, n, replace=False)
+            rows.append(np.concatenate([c, c[: (len(c) + 1) // 2]]) if g != 1 else c)  # the middle group is valid
+    lens = np.array([len(r) for r in rows])
+    ptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    cols = np.concatenate(rows).astype(np.int32)
+    vals = np.ones(cols.size, np.float16)
+    vrp, vcol, vval, nvec = gpu_svc(len(rows), K, V, ptr, cols, vals)
+    for g in range(0, len(rows), V):
+        distinct = np.unique(cols[ptr[g]:ptr[g + V]])
+        got = vcol[vrp[g // V]:vrp[g // V + 1]]
+        assert np.array_equal(np.sort(got), distinct)
+        block = vval[vrp[g // V] * V:vrp[g // V + 1] * V].reshape(-1, V)
+        for r in range(V):
+            assert np.array_equal(np.sort(got[block[:, r] != 0]), np.unique(rows[g + r]))
+
+
 @pytest.mark.parametrize("K,order", [(4096, "cpython"), (4096, "sorted"), (300000, "cpython")])
 def test_columns_outside_the_matrix_are_ignored(oracle, built_library, K, order):
     """Invalid input (the contract wants 0 <= column < K): such non-zeros are dropped, nothing else changes, and

@@ -35,10 +35,10 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 MEASURED_TRAFFIC = {
     # HBM bytes per launch from rocprofv3 counters (FETCH_SIZE and WRITE_SIZE, each scaled by its reading of a plain
     # 256 MiB copy), keyed by benchmark entry; measured in runs of their own, not in this one.
-    "headline_batch128": {"kernel": "spmm_slab_kernel<8,float,*,4>", "bytes": 65.9e6 + 268.4e6, "alg_bytes": 328781828,
+    "headline_batch128": {"kernel": "spmm_slab_kernel<8,float,*,4>", "bytes": 66.1e6 + 268.4e6, "alg_bytes": 328781828,
                           "source": "profiles/spmm_slab_v8_f32_cfg2_batch128_hbm_traffic.txt"},
     "cfg3_1024x2304_v16_s0.8_n3136": {"kernel": "spmm_gather_kernel<16,float,8>", "bytes": 27.0e6 + 12.8e6,
-                                      "alg_bytes": 28358148, "l2_request_bytes": 224.0e6,
+                                      "alg_bytes": 28358148, "l2_request_bytes": 220.8e6,
                                       "source": "profiles/spmm_gather_v16_f32_cfg3_1024x2304_s0.8_n3136_counters.txt"},
     "cfg4_spmm_on_svc_output_with_plan": {"kernel": "spmm_balanced_kernel<8,float,false>", "bytes": 44.0e6 + 20.1e6,
                                           "alg_bytes": 30393520, "l2_request_bytes": 204.4e6,
@@ -47,7 +47,7 @@ MEASURED_TRAFFIC = {
                                 "alg_bytes": 30393520, "l2_request_bytes": 186.5e6,
                                 "source": "profiles/spmm_balanced_v8_f32_cfg4_zipf_n256_counters.txt"},
     "svc_cfg4_zipf_16384_v8": {"kernel": "svc_count_distinct + svc_scan_classify + the svc_merge kernels",
-                               "bytes": (1.708 + 0.012 + 2.009 + 1.540 + 0.030) * 1e6 + (0.044 + 0.011 + 3.145 + 0.918) * 1e6,
+                               "bytes": (1.705 + 0.012 + 1.906 + 1.366 + 0.026) * 1e6 + (0.044 + 0.011 + 3.145 + 0.918) * 1e6,
                                "alg_bytes": 6866100, "source": "profiles/svc_kernels_cfg4_zipf_v8_counters.txt"},
 }
 KERNEL_NAMES = {1: "spmm_generic_kernel", 2: "spmm_gather_kernel", 3: "spmm_slab_kernel<*,4>", 4: "spmm_gather_split_kernel",

@@ -238,8 +238,9 @@ int sspmm_softmax_batched_f16(int batch, int m_vec, int V, const int32_t *row_in
  * iteration order of CPython's set in `list(set(acc + row))`), bit for bit;
  * SVC_ORDER_SORTED stores each vector-row's columns ascending.
  * Column indices must lie in [0, K) and a CSR row must not repeat a column; a non-zero that breaks
- * the first rule is ignored, rows that break the second give an unspecified column order, and
- * neither makes the kernels touch memory outside the arrays named here.
+ * the first rule is ignored, rows that break the second give an unspecified column order (every
+ * distinct column of the group still once), and neither makes the kernels touch memory outside the
+ * arrays named here.
  * ---------------------------------------------------------------------------------------- */
 #define SVC_ORDER_CPYTHON 0
 #define SVC_ORDER_SORTED 1

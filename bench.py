@@ -3,7 +3,8 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-Prints ONE JSON line.  A "step" is one pass of the SpMM over one batch of synthetic inputs
+Prints ONE short JSON line (the contract keys, roofline, cpu_baseline and a dozen scalars) and writes every figure of
+the run to bench_extra.json in the working directory (--extras-file).  A "step" is one pass of the SpMM over one batch of synthetic inputs
 already resident in HBM: the FFN-shaped configuration (A 2048x512 fp16, V=8, 90 % vector
 sparsity, B 512x256 fp16, C fp32), run bspmm-style over a batch of independent value / B / C
 sets that share the pattern, so that one launch moves more bytes than the last-level cache
@@ -30,26 +31,34 @@ import numpy as np
 
 HBM_PEAK_GBPS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
-# HBM bytes per launch from hardware counters (FETCH_SIZE and WRITE_SIZE in separate runs, each scaled by its
-# reading for a plain 256 MiB device copy), keyed by kernel and workload; `source` names the summary it comes from.
-MEASURED_TRAFFIC = {
-    # HBM bytes per launch from rocprofv3 counters (FETCH_SIZE and WRITE_SIZE, each scaled by its reading of a plain
-    # 256 MiB copy), keyed by benchmark entry; measured in runs of their own, not in this one.
-    "headline_batch128": {"kernel": "spmm_slab_kernel<8,float,*,4>", "bytes": 66.1e6 + 268.4e6, "alg_bytes": 328781828,
-                          "source": "profiles/spmm_slab_v8_f32_cfg2_batch128_hbm_traffic.txt"},
-    "cfg3_1024x2304_v16_s0.8_n3136": {"kernel": "spmm_gather_kernel<16,float,8>", "bytes": 27.0e6 + 12.8e6,
-                                      "alg_bytes": 28358148, "l2_request_bytes": 220.8e6,
-                                      "source": "profiles/spmm_gather_v16_f32_cfg3_1024x2304_s0.8_n3136_counters.txt"},
-    "cfg4_spmm_on_svc_output_with_plan": {"kernel": "spmm_balanced_kernel<8,float,false>", "bytes": 44.0e6 + 20.1e6,
-                                          "alg_bytes": 30393520, "l2_request_bytes": 204.4e6,
-                                          "source": "profiles/spmm_balanced_v8_f32_cfg4_zipf_n256_counters.txt"},
-    "cfg4_spmm_on_svc_output": {"kernel": "spmm_gather_split_kernel<8,float>", "bytes": 51.3e6 + 16.8e6,
-                                "alg_bytes": 30393520, "l2_request_bytes": 186.5e6,
-                                "source": "profiles/spmm_balanced_v8_f32_cfg4_zipf_n256_counters.txt"},
-    "svc_cfg4_zipf_16384_v8": {"kernel": "svc_count_distinct + svc_scan_classify + the svc_merge kernels",
-                               "bytes": (1.705 + 0.012 + 1.906 + 1.366 + 0.026) * 1e6 + (0.044 + 0.011 + 3.145 + 0.918) * 1e6,
-                               "alg_bytes": 6866100, "source": "profiles/svc_kernels_cfg4_zipf_v8_counters.txt"},
-}
+def measured_traffic(profiles_dir=None):
+    """HBM bytes per launch from hardware counters, read from the summaries under profiles/: every line of the form
+        traffic: entry=<benchmark entry> kernel=<kernel> fetch_mb=<F> write_mb=<W> [l2_request_mb=<R>] alg_mb=<A>
+    (FETCH_SIZE and WRITE_SIZE of separate rocprofv3 runs, each scaled by its reading of a plain 256 MiB copy; measured
+    in runs of their own, not in this one).  Returns entry -> {kernel, bytes, alg_bytes, l2_request_bytes, source}."""
+    d = profiles_dir or os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles")
+    table = {}
+    if not os.path.isdir(d):
+        return table
+    for fn in sorted(os.listdir(d)):
+        if not fn.endswith(".txt"):
+            continue
+        with open(os.path.join(d, fn)) as f:
+            for ln in f:
+                if not ln.startswith("traffic:"):
+                    continue
+                kv = dict(p.split("=", 1) for p in ln[len("traffic:"):].split() if "=" in p)
+                try:
+                    row = {"kernel": kv["kernel"], "bytes": (float(kv["fetch_mb"]) + float(kv["write_mb"])) * 1e6,
+                           "alg_bytes": float(kv["alg_mb"]) * 1e6, "source": "profiles/" + fn}
+                    if "l2_request_mb" in kv:
+                        row["l2_request_bytes"] = float(kv["l2_request_mb"]) * 1e6
+                    table[kv["entry"]] = row
+                except (KeyError, ValueError):
+                    continue
+    return table
+
+
 KERNEL_NAMES = {1: "spmm_generic_kernel", 2: "spmm_gather_kernel", 3: "spmm_slab_kernel<*,4>", 4: "spmm_gather_split_kernel",
                 5: "spmm_slab_kernel<*,2>", 6: "spmm_stage_kernel", 7: "spmm_balanced_kernel", 9: "spmm_slab_kernel<*,8>"}
 
@@ -72,6 +81,8 @@ def parse_args():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy (its hardware-counter readings calibrate FETCH_SIZE / "
                          "WRITE_SIZE when the run is profiled)")
+    ap.add_argument("--extras-file", default="bench_extra.json",
+                    help="where the full dictionary of figures is written (the line on stdout is a short summary of it)")
     ap.add_argument("--kernel", choices=["auto", "generic", "gather", "slab", "slab128"], default="auto",
                     help="force one SpMM kernel (tuning); the default lets the library choose")
     return ap.parse_args()
@@ -139,33 +150,6 @@ def graph_time(fn, launches=20, replays=20):
     return start.elapsed_time(end) / (launches * replays)
 
 
-_PROBE = {}
-
-
-def gather_probe(L, torch, waves_per_cu, rows=2304, row_bytes=6144, steps=32):
-    """TB/s at which the device serves the gather kernels' access pattern (16 lanes read 256 contiguous bytes of a random
-    row of a matrix that fits the caches, eight 16-byte loads per lane in flight) with waves_per_cu waves on each of
-    the 256 CUs: sspmm_probe_gather of the C ABI, a loop of loads and nothing else."""
-    mat = torch.ones(rows * row_bytes // 2, dtype=torch.float16, device="cuda")
-    waves = 256 * waves_per_cu
-    sink = torch.empty(waves * 4, dtype=torch.int32, device="cuda")
-
-    def run():
-        rc = L.sspmm_probe_gather(mat.data_ptr(), rows, row_bytes, waves, steps, sink.data_ptr(), torch.cuda.current_stream().cuda_stream)
-        if rc:
-            raise RuntimeError("sspmm_probe_gather failed: %d" % rc)
-
-    ms = time_launches(run, 50, 10)
-    return waves * steps * 8192 / ms / 1e9
-
-
-def gather_probe_rate(L, torch):
-    """The probe's rate at full occupancy (32 waves per CU), measured once per process."""
-    if "tbps" not in _PROBE:
-        _PROBE["tbps"] = gather_probe(L, torch, 32)
-    return _PROBE["tbps"]
-
-
 def figures(ms, alg_bytes, flops):
     return {"ms": ms, "useful_tflops": flops / ms / 1e9, "alg_bytes": alg_bytes, "hbm_gbps": alg_bytes / ms / 1e6,
             "hbm_frac": alg_bytes / ms / 1e6 / HBM_PEAK_GBPS}
@@ -224,8 +208,6 @@ def spmm_case(L, torch, synth, M, K, V, sparsity, N, batch, out_f32, std, seed, 
         cms = graph_time(lambda s_: dst.copy_(src))
         out["plain_copy_of_the_same_bytes_ms_in_a_graph"] = cms
         out["time_vs_plain_copy_of_the_same_bytes_in_a_graph"] = gms / cms
-        # and what the gathers alone cost at the rate the device serves this access pattern from its caches
-        out["gather_bytes_at_the_probe_rate_ms"] = out["gather_bytes_no_reuse"] / gather_probe_rate(L, torch) / 1e9
         del src, dst
     if dense:
         A = torch.zeros(vs.m_vec * V, K, dtype=torch.float16, device="cuda")
@@ -773,8 +755,6 @@ def main():
         ceilings = {"device_copy_1GiB_gbps": 2 * src.numel() * 4 / copy_ms / 1e6,
                     "device_fill_1GiB_gbps": src.numel() * 4 / fill_ms / 1e6}
         ceilings["frac_of_device_copy"] = main_res["hbm_gbps"] / ceilings["device_copy_1GiB_gbps"]
-        # the caches' side: the gather kernels' access pattern with nothing else in the loop, at 4, 8, 16 and 32 waves per CU
-        ceilings["cache_to_cu_gather_tbps_by_waves_per_cu"] = {str(w): gather_probe(L, torch, w) for w in (4, 8, 16, 32)}
         del src, dst
 
     # parity of batch elements spread over the launch (first, last, and one per way the batch is dealt to the XCDs)
@@ -835,29 +815,106 @@ def main():
     if not args.quick:
         for name in list(single_launch_cases(args.batch)) + GROUPS:
             extra.update(run_extra(name, env))
-        extra["measured_hbm_traffic"] = MEASURED_TRAFFIC
+    traffic = measured_traffic()
+    if not args.quick:
+        extra["measured_hbm_traffic"] = traffic
+    head_traffic = traffic.get("headline_batch128") if (args.kernel == "auto" and args.batch == 128) else None
 
-    line = {
+    roofline = {"bound": "hbm", "achieved": main_res["hbm_gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                "frac": main_res["hbm_frac"], "traffic": head_traffic["bytes"] if head_traffic else None,
+                "kernel": main_kernel, "alg_bytes_per_launch": main_res["alg_bytes"]}
+    dense = {k: main_res[k] for k in main_res if k.startswith("dense") or k.startswith("speedup")}
+    contract = {
         "metric": "SpMM useful TFLOP/s (2*nnz*N/t), V=8 @90% sparsity, fp16 in / fp32 accumulate",
         "value": main_res["useful_tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": main_res["ms"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": main_res["workload"] + " (one launch, pattern shared by the batch)",
                    "hbm_gbps": main_res["hbm_gbps"]},
-        "roofline": {"bound": "hbm", "achieved": main_res["hbm_gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": main_res["hbm_frac"],
-                     "traffic": MEASURED_TRAFFIC["headline_batch128"]["bytes"] if (args.kernel == "auto" and args.batch == 128) else None,
-                     "traffic_source": MEASURED_TRAFFIC["headline_batch128"]["source"],
-                     "kernel": main_kernel, "alg_bytes_per_launch": main_res["alg_bytes"],
-                     "operands": "warm: the same 329 MB of operands every launch (the cold rotation of two sets is "
-                                 "extra.headline_batched_cold)",
-                     "measured_stream_rates": ceilings},
-        "cpu_baseline": cpu,
-        "parity_max_rel_err": parity,
-        "dense_gemm": {k: main_res[k] for k in main_res if k.startswith("dense") or k.startswith("speedup")},
-        "extra": extra,
     }
-    print(json.dumps(line))
+
+    # Every figure of the run goes to a file; the line on stdout carries the contract and a dozen scalars.
+    full = dict(contract)
+    full["roofline"] = dict(roofline, traffic_source=head_traffic["source"] if head_traffic else None,
+                            operands="warm: the same 329 MB of operands every launch (the cold rotation of two sets is "
+                                     "extra.headline_batched_cold)", measured_stream_rates=ceilings)
+    full.update({"cpu_baseline": cpu, "parity_max_rel_err": parity, "dense_gemm": dense, "extra": extra})
+    try:
+        with open(args.extras_file, "w") as f:
+            json.dump(full, f, indent=1)
+            f.write("\n")
+    except OSError as e:
+        print("bench.py: could not write %s: %s" % (args.extras_file, e), file=sys.stderr)
+
+    # an entry whose result was compared with the host loop and disagrees fails the run, whichever entry it is
+    bad = parity_failures(extra)
+    if bad:
+        print("bench.py: entries that disagree with the host loop (max relative error > %g): %r" % (PARITY_BAR, bad),
+              file=sys.stderr)
+        sys.exit(3)
+
+    line = dict(contract)
+    line["roofline"] = roofline
+    line["cpu_baseline"] = {k: cpu[k] for k in ("value", "unit", "cores", "kind", "sample")} if cpu else None
+    line["parity_max_rel_err"] = parity
+    line["dense_gemm"] = dense
+    line["extra"] = short_extra(extra)
+    line["extra_file"] = args.extras_file
+    text = json.dumps(line)
+    assert len(text) < 4096, "the benchmark line must stay short (%d bytes)" % len(text)
+    print(text)
+
+
+PARITY_BAR = 1e-2
+
+
+def parity_failures(tree, path=""):
+    """Every '...max_rel_err...' figure of the nested result dictionary that exceeds the bar, and every
+    '...bit_exact...' flag that is false."""
+    bad = {}
+    if isinstance(tree, dict):
+        for k, v in tree.items():
+            p = path + "/" + str(k) if path else str(k)
+            if isinstance(v, dict):
+                bad.update(parity_failures(v, p))
+            elif "max_rel_err" in str(k) and isinstance(v, (int, float)) and not v <= PARITY_BAR:
+                bad[p] = v
+            elif "bit_exact" in str(k) and v is False:
+                bad[p] = v
+    return bad
+
+
+def short_extra(extra):
+    """At most a dozen scalars of the full result dictionary for the line on stdout (single-launch fractions of the
+    HBM peak, SVC speed-ups over the Python RowMerge); absent entries are left out."""
+    def get(*keys):
+        node = extra
+        for k in keys:
+            if not isinstance(node, dict) or k not in node:
+                return None
+            node = node[k]
+        return round(node, 4) if isinstance(node, float) else node
+
+    picks = {
+        "headline_cold_hbm_frac": ("headline_batched_cold", "hbm_frac"),
+        "cfg3_1024x2304_s0.8_n3136_hbm_frac": ("cfg3_1024x2304_v16_s0.8_n3136", "hbm_frac"),
+        "cfg3_1024x2304_s0.8_n3136_ms": ("cfg3_1024x2304_v16_s0.8_n3136", "ms"),
+        "cfg3_2048x1024_s0.95_n3136_hbm_frac": ("cfg3_2048x1024_v16_s0.95_n3136", "hbm_frac"),
+        "cfg5_ffn1_hbm_frac": ("cfg5_ffn1_3072x768_v16_s0.9_n4096", "hbm_frac"),
+        "cfg5_ffn2_hbm_frac": ("cfg5_ffn2_768x3072_v16_s0.9_n4096", "hbm_frac"),
+        "cfg4_spmm_with_plan_hbm_frac": ("cfg4_spmm_on_svc_output_with_plan", "hbm_frac"),
+        "cfg4_spmm_with_plan_ms": ("cfg4_spmm_on_svc_output_with_plan", "ms"),
+        "svc_cfg4_speedup_vs_python": ("svc_cfg4_zipf_16384_v8", "speedup_vs_python"),
+        "svc_batched_dlmc_shapes_speedup_vs_python": ("svc_batched_dlmc_shapes", "speedup_vs_python"),
+        "cfg5_layer_speedup_vs_dense_in_a_graph": ("cfg5_encoder_layer_v16_s0.9_tokens4096", "speedup_vs_dense_layer_in_a_graph"),
+        "sparse_attention_forward_seq4096_ms": ("sparse_attention_forward_seq4096_h4_e256_s0.9_b2_l4", "ms"),
+    }
+    out = {}
+    for name, keys in picks.items():
+        v = get(*keys)
+        if v is not None:
+            out[name] = v
+    return out
 
 
 if __name__ == "__main__":

@@ -307,17 +307,6 @@ int sspmm_attention_fm_f16(int batch, int heads, int seq, int head_dim, const ss
                            const sspmm_half_t *v, int64_t ld, sspmm_half_t *out, int64_t ld_out, float scale, void *hip_stream);
 
 /* ------------------------------------------------------------------------------------------
- * Diagnostic, no counterpart in the reference: the rate at which the device serves the gather kernels'
- * access pattern with nothing else in the loop.  `waves` wavefronts each issue `steps` rounds of eight
- * 16-byte loads per lane; a 16-lane group reads 256 contiguous bytes of a pseudo-random row of the
- * [rows x row_bytes] matrix (row_bytes a multiple of 256, 16-byte aligned pointers).  The launch moves
- * waves * steps * 8192 bytes from the caches to the compute units; the benchmark times it and reports the
- * rate beside the SpMM kernels'.  sink: device memory of at least 16 bytes per wave (not written in
- * practice: it keeps the loads alive).
- * ---------------------------------------------------------------------------------------- */
-int sspmm_probe_gather(const void *matrix, int rows, int row_bytes, int waves, int steps, void *sink, void *hip_stream);
-
-/* ------------------------------------------------------------------------------------------
  * Coordinate list -> CSR, the step between a Matrix Market file and the RowMerge in the
  * reference's SuiteSparse path: `csr = self.coo.tocsr()` in suite_matrix.coo2csr, reference
  * RowMerge/suit_sparse_matrix.py:109-111 (scipy: rows ascending, inside a row the columns

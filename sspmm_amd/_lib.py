@@ -37,7 +37,6 @@ SIGNATURES = {
     "svc_count": (_int, [_int, _int, _int, _vp, _vp, _i64, _int, _vp, _vp, _vp]),
     "svc_fill": (_int, [_int, _int, _int, _vp, _vp, _vp, _i64, _int, _vp, _vp, _vp, _vp, _vp]),
     "sspmm_add_layernorm_f16": (_int, [_int, _int, _vp, _vp, _vp, _vp, ctypes.c_float, _vp, _vp]),
-    "sspmm_probe_gather": (_int, [_vp, _int, _int, _int, _int, _vp, _vp]),
     "sspmm_linear_f16": (_int, [_int, _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _int, _vp, _vp]),
     "sspmm_attention_fm_f16": (_int, [_int, _int, _int, _int, _vp, _vp, _vp, ctypes.c_int64, _vp, ctypes.c_int64, ctypes.c_float, _vp]),
     "svc_coo_workspace_bytes": (ctypes.c_size_t, [_i64]),

@@ -7,7 +7,6 @@
 #include "coo_kernels.h"
 #include "layer_kernels.h"
 #include "plan.h"
-#include "probe.h"
 #include "reorder_kernels.h"
 #include "spmm_kernels.h"
 #include "svc_kernels.h"
@@ -356,12 +355,6 @@ int sspmm_attention_fm_f16(int batch, int heads, int seq, int head_dim, const ss
   if (!q || !k || !v || !out || ld < (int64_t)batch * seq || ld_out < (int64_t)batch * seq) return kInvalid;
   if (!sspmm::attention_fm_applies(batch, heads, seq, head_dim, q, k, v, ld, out, ld_out)) return kInvalid;
   return (int)sspmm::launch_attention_fm(batch, heads, seq, q, k, v, ld, out, ld_out, scale, static_cast<hipStream_t>(hip_stream));
-}
-
-int sspmm_probe_gather(const void *matrix, int rows, int row_bytes, int waves, int steps, void *sink, void *hip_stream) {
-  if (!matrix || !sink || rows <= 0 || row_bytes <= 0 || row_bytes % 256 != 0 || waves <= 0 || steps < 0) return kInvalid;
-  if (reinterpret_cast<uintptr_t>(matrix) % 16 != 0 || reinterpret_cast<uintptr_t>(sink) % 16 != 0) return kInvalid;
-  return (int)sspmm::launch_probe_gather(matrix, rows, row_bytes, waves, steps, sink, static_cast<hipStream_t>(hip_stream));
 }
 
 size_t svc_coo_workspace_bytes(int64_t n) { return sspmm::coo_workspace_bytes(n); }

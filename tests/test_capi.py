@@ -59,15 +59,13 @@ def test_argument_errors_without_device_work(built_library):
     assert L.sspmm_plan_destroy(None) == 0
     assert L.sspmm_plan_info(None, None) == 1
     assert L.sspmm_plan_batched_f16_f32(None, 1, 64, one, one, one, 0, one, 0, one, 0, None) == 1
-    # the linear-layer, attention and probe entry points reject what they do not cover before touching the device
+    # the linear-layer and attention entry points reject what they do not cover before touching the device
     assert L.sspmm_linear_f16(4, 8, 64, 64, one, one, one, one, None, 7, one, None) == 1       # unknown activation
     assert L.sspmm_linear_f16(4, 4, 64, 64, one, one, one, one, None, 0, one, None) == 1       # unsupported V
     assert L.sspmm_linear_f16(0, 8, 64, 64, None, None, None, None, None, 1, None, None) == 0  # nothing to do
     assert L.sspmm_attention_fm_f16(1, 1, 64, 32, 16, 16, 16, 64, 16, 64, 0.125, None) == 1    # head size
     assert L.sspmm_attention_fm_f16(1, 1, 96, 64, 16, 16, 16, 96, 16, 96, 0.125, None) == 1    # sequence not a multiple of 64
     assert L.sspmm_attention_fm_f16(0, 1, 64, 64, None, None, None, 0, None, 0, 0.125, None) == 0
-    assert L.sspmm_probe_gather(None, 16, 256, 4, 1, 16, None) == 1
-    assert L.sspmm_probe_gather(16, 16, 200, 4, 1, 16, None) == 1                              # rows of 256-byte pieces
     assert L.svc_workspace_bytes(16, 100, 8) >= 100 * 8
     assert b"invalid" in L.sspmm_error_string(1)
     assert L.sspmm_error_string(0) == b"success"

@@ -471,19 +471,6 @@ def test_row_swizzle_matches_oracle(oracle, built_library):
         assert np.array_equal(got, oracle.sorted_row_swizzle(off))
 
 
-def test_probe_gather_runs_and_leaves_its_sink_alone(built_library):
-    """The diagnostic loop of gathers (bench.py times it): launches, returns success, writes nothing."""
-    from sspmm_amd import _lib
-    L = _lib.lib()
-    rows, row_bytes, waves, steps = 300, 1024, 64, 5
-    mat = torch.ones(rows * row_bytes // 2, dtype=torch.float16, device="cuda")
-    sink = torch.full((waves * 4,), 123, dtype=torch.int32, device="cuda")
-    rc = L.sspmm_probe_gather(mat.data_ptr(), rows, row_bytes, waves, steps, sink.data_ptr(), torch.cuda.current_stream().cuda_stream)
-    assert rc == 0
-    torch.cuda.synchronize()
-    assert torch.all(sink == 123)
-
-
 @pytest.mark.parametrize("V", [8, 16])
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("N", [128, 136, 200, 256, 520])

@@ -170,8 +170,10 @@ int sspmm_plan_batched_f16_f16(const sspmm_plan_t *plan, int batch, int N, const
  *   SSPMM_ERROR_STATIC_SCRATCH_TOO_SMALL and does nothing.  Other arguments as sspmm_f16_f32.
  *   All calls on one GPU share the array: two calls that overlap on a GPU (different streams,
  *   or threads) race and give wrong results; calls on one stream are safe.
- *   The first call on a device looks the array's address up and should not be made inside a
- *   capture.  Same results as sspmm_plan_batched_f16_f32 with a plan of the same pattern, bit
+ *   The first call on a device looks the array's address up and must come before any capture:
+ *   made on a capturing stream it returns hipErrorInvalidValue and records nothing.  Patterns that
+ *   the load-balanced kernel does not cover (N not a multiple of 8, unaligned pointers) take the
+ *   kernels of sspmm_f16_f32 and use no scratch.  Same results as sspmm_plan_batched_f16_f32 with a plan of the same pattern, bit
  *   for bit, as long as the plan's panels also fit 8 MB of partial tiles.
  */
 #define SSPMM_ERROR_STATIC_SCRATCH_TOO_SMALL 9001
@@ -301,7 +303,8 @@ int sspmm_add_layernorm_f16(int H, int T, const sspmm_half_t *x, const sspmm_hal
  *             t = b * seq + s (they may be three row ranges of one fused projection)
  *   out       fp16, same layout with ld_out
  * Supported: head_dim = 64, seq a multiple of 64 up to 16384, ld and ld_out multiples of 8 and at
- * least batch * seq, 16-byte aligned pointers; anything else returns hipErrorInvalidValue.
+ * least batch * seq, 16-byte aligned pointers, scale positive and finite; anything else returns
+ * hipErrorInvalidValue.
  * ---------------------------------------------------------------------------------------- */
 int sspmm_attention_fm_f16(int batch, int heads, int seq, int head_dim, const sspmm_half_t *q, const sspmm_half_t *k,
                            const sspmm_half_t *v, int64_t ld, sspmm_half_t *out, int64_t ld_out, float scale, void *hip_stream);

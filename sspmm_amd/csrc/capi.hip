@@ -352,6 +352,8 @@ int sspmm_attention_fm_f16(int batch, int heads, int seq, int head_dim, const ss
                            const sspmm_half_t *v, int64_t ld, sspmm_half_t *out, int64_t ld_out, float scale, void *hip_stream) {
   if (batch < 0 || heads < 0 || seq < 0 || head_dim <= 0) return kInvalid;
   if (batch == 0 || heads == 0 || seq == 0) return 0;
+  // (the kernel's running maximum is taken of the unscaled scores, which orders the scaled ones only for scale > 0)
+  if (!(scale > 0.0f) || !(scale <= 3.0e38f)) return kInvalid;
   if (!q || !k || !v || !out || ld < (int64_t)batch * seq || ld_out < (int64_t)batch * seq) return kInvalid;
   if (!sspmm::attention_fm_applies(batch, heads, seq, head_dim, q, k, v, ld, out, ld_out)) return kInvalid;
   return (int)sspmm::launch_attention_fm(batch, heads, seq, q, k, v, ld, out, ld_out, scale, static_cast<hipStream_t>(hip_stream));

@@ -13,6 +13,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <mutex>
+
 #include "layer_kernels.h"
 
 namespace sspmm {
@@ -128,6 +130,8 @@ static hipError_t launch_ln(int H, int T, const uint16_t *x, const uint16_t *a, 
   if (lds > 64 * 1024) {
     // the runtime is told once per device and size
     static int raised[16] = {};
+    static std::mutex raised_mutex;
+    std::lock_guard<std::mutex> lock(raised_mutex);
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) dev = -1;
     if (dev < 0 || raised[dev] < (int)lds) {

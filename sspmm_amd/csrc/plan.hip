@@ -136,13 +136,18 @@ static constexpr int kStaticMaxDevices = 64;
 static unsigned char *g_scratch_ptr[kStaticMaxDevices] = {};
 static std::mutex g_scratch_mutex;
 
-static hipError_t static_scratch(unsigned char **ptr) {
+static hipError_t static_scratch(unsigned char **ptr, hipStream_t stream) {
   int dev = -1;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return e;
   if (dev < 0 || dev >= kStaticMaxDevices) return hipErrorInvalidDevice;
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
   if (!g_scratch_ptr[dev]) {
+    // The look-up is not a call to make while a stream records a graph: the first use on a device has to come
+    // before the capture (any call of the entry point outside a capture will do).
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (stream && hipStreamIsCapturing(stream, &cap) == hipSuccess && cap != hipStreamCaptureStatusNone)
+      return hipErrorInvalidValue;
     void *p = nullptr;
     if ((e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch))) != hipSuccess) return e;
     g_scratch_ptr[dev] = static_cast<unsigned char *>(p);
@@ -156,7 +161,7 @@ bool static_spmm_fits(int m_vec, int N) { return m_vec <= kStaticMaxRows && N <=
 hipError_t launch_spmm_static(const SpmmArgs &a, int V, bool out_f16, hipStream_t stream) {
   if (!balanced_kernel_applies(a, V, out_f16)) return launch_spmm(a, V, out_f16, stream);  // (needs no scratch)
   unsigned char *base = nullptr;
-  hipError_t e = static_scratch(&base);
+  hipError_t e = static_scratch(&base, stream);
   if (e != hipSuccess) return e;
   ScheduleView view;
   view.header = reinterpret_cast<int32_t *>(base);

@@ -82,6 +82,24 @@ class SparseLinear(torch.nn.Module):
         r = svc(row_ptr, col_ind, weight[mask].contiguous(), out_features, in_features, vec_length, order=order)
         return cls(in_features, out_features, vec_length, r.vec_row_ptr, r.vec_col, r.vec_val, bias, **kw)
 
+    def rows(self, first, last):
+        """The layer of output features first .. last-1 (multiples of vec_length) as a layer of its own whose arrays
+        are views of this one's: nothing is copied, and the view is not registered anywhere."""
+        V = self.vec_length
+        if first % V or last % V or not 0 <= first <= last <= self.out_features:
+            raise ValueError("row range must be multiples of vec_length inside [0, out_features]")
+        off = self.row_offsets[first // V:last // V + 1]
+        lo, hi = int(off[0]), int(off[-1])
+        return SparseLinear(self.in_features, last - first, V, (off - lo).to(torch.int32), self.column_indices[lo:hi],
+                            self.values[lo * V:hi * V], None if self.bias is None else self.bias[first:last],
+                            out_dtype=self.out_dtype, activation=self.activation)
+
+    def _apply(self, fn, *args, **kw):
+        # a plan lives on the device it was built on and describes the row offsets it was built from: when the
+        # buffers are moved or converted it is dropped, and make_plan has to be called again
+        self.plan = None
+        return super()._apply(fn, *args, **kw)
+
     def make_plan(self, max_tokens):
         """Builds the pattern's plan (sspmm_amd.Plan) for inputs of up to max_tokens columns; later calls of the
         layer use it.  Worth it for weights whose merged rows are uneven (unstructured pruning through RowMerge)."""
@@ -89,22 +107,24 @@ class SparseLinear(torch.nn.Module):
         self.plan = Plan(self.row_offsets, self.vec_length, self.in_features, max_N=max_tokens)
         return self.plan
 
-    def forward(self, x):
+    def forward(self, x, activation="layer"):
+        """activation: "layer" applies the layer's own (self.activation); None or "gelu" override it for this call."""
+        act = self.activation if activation == "layer" else activation
         if x.dim() != 2 or x.size(0) != self.in_features:
             raise ValueError("x must be [in_features, tokens] = [%d, *], got %s" % (self.in_features, tuple(x.shape)))
         plan = getattr(self, "plan", None)
         if plan is not None and x.size(1) > plan.max_N:
             plan = None
         fuse = plan is None and self.out_dtype == torch.float16 and (self.bias is None or self.bias.dtype == torch.float16)
-        if fuse and (self.bias is not None or self.activation is not None):
+        if fuse and (self.bias is not None or act is not None):
             # bias and activation in the product's epilogue: one launch, the output written once
             return linear_op(self.row_offsets, self.column_indices, self.values, x.contiguous(), self.vec_length,
-                             bias=self.bias, activation=self.activation)
+                             bias=self.bias, activation=act)
         y = spmm(None, self.row_offsets, self.column_indices, self.values, x.contiguous(), self.vec_length,
                  out_dtype=self.out_dtype, plan=plan)
         if self.bias is not None:
             y = y + self.bias[:, None].to(y.dtype)
-        if self.activation == "gelu":
+        if act == "gelu":
             y = torch.nn.functional.gelu(y)
         return y
 
@@ -170,14 +190,34 @@ class SparseEncoderLayer(torch.nn.Module):
     def __init__(self, hidden, heads, ffn, q, k, v, o, ffn1, ffn2):
         super().__init__()
         self.hidden, self.heads, self.ffn = hidden, heads, ffn
-        self.q, self.k, self.v, self.o, self.ffn1, self.ffn2 = q, k, v, o, ffn1, ffn2
-        # query, key and value projections as one SpMM over the three patterns stacked along M
+        self.o, self.ffn1, self.ffn2 = o, ffn1, ffn2
+        # query, key and value projections as one SpMM over the three patterns stacked along M.  The fused layer is
+        # the only copy the module keeps (q, k and v below are views of its arrays), so the weights are held once and
+        # state_dict names them once.
         self.qkv = SparseLinear.concat([q, k, v])
-        # the first feed-forward product with its GELU in the product's epilogue (shares ffn1's arrays)
-        self.ffn1_gelu = SparseLinear(ffn1.in_features, ffn1.out_features, ffn1.vec_length, ffn1.row_offsets, ffn1.column_indices,
-                                      ffn1.values, ffn1.bias, out_dtype=ffn1.out_dtype, activation="gelu")
+        self._qkv_rows = (0, q.out_features, q.out_features + k.out_features,
+                          q.out_features + k.out_features + v.out_features)
         self.ln1 = torch.nn.LayerNorm(hidden)
         self.ln2 = torch.nn.LayerNorm(hidden)
+
+    q = property(lambda self: self.qkv.rows(self._qkv_rows[0], self._qkv_rows[1]))
+    k = property(lambda self: self.qkv.rows(self._qkv_rows[1], self._qkv_rows[2]))
+    v = property(lambda self: self.qkv.rows(self._qkv_rows[2], self._qkv_rows[3]))
+
+    @property
+    def ffn1_gelu(self):
+        """The first feed-forward product with its GELU in the product's epilogue: ffn1 itself, called with the
+        activation (no second module, no second copy of the arrays)."""
+        ffn1 = self.ffn1
+
+        class _WithGelu:
+            in_features, out_features = ffn1.in_features, ffn1.out_features
+            dense_weight = staticmethod(ffn1.dense_weight)
+
+            def __call__(self, x):
+                return ffn1(x, activation="gelu")
+
+        return _WithGelu()
 
     def _attention(self, qkv, batch, seq):
         """qkv: [3 * hidden, batch*seq] feature-major; returns the context [hidden, batch*seq].  One HIP kernel that

@@ -66,6 +66,8 @@ def test_argument_errors_without_device_work(built_library):
     assert L.sspmm_attention_fm_f16(1, 1, 64, 32, 16, 16, 16, 64, 16, 64, 0.125, None) == 1    # head size
     assert L.sspmm_attention_fm_f16(1, 1, 96, 64, 16, 16, 16, 96, 16, 96, 0.125, None) == 1    # sequence not a multiple of 64
     assert L.sspmm_attention_fm_f16(0, 1, 64, 64, None, None, None, 0, None, 0, 0.125, None) == 0
+    for bad_scale in (0.0, -0.125, float("nan"), float("inf")):
+        assert L.sspmm_attention_fm_f16(1, 1, 64, 64, 16, 16, 16, 64, 16, 64, bad_scale, None) == 1
     assert L.svc_workspace_bytes(16, 100, 8) >= 100 * 8
     assert b"invalid" in L.sspmm_error_string(1)
     assert L.sspmm_error_string(0) == b"success"

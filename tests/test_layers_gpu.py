@@ -169,6 +169,40 @@ def test_encoder_layer_at_the_benchmark_shape_takes_the_attention_kernel(built_l
     assert max_rel_err(got.float().cpu().numpy(), want.float().cpu().numpy()) <= 1e-2
 
 
+def test_encoder_layer_at_the_benchmark_shape_matches_dense_products(built_library):
+    """hidden 768, 12 heads, FFN 3072, 8 x 512 tokens, six weights V = 16 at 90 %: the layer against the same layer whose
+    four products are dense fp32 matmuls on the densified weights (an independent check of the sparse products at the
+    full shape: nothing of this library computes the comparison's products)."""
+    hidden, heads, ffn, V, batch, seq = 768, 12, 3072, 16, 8, 512
+    mk = lambda o, i, s: _vector_sparse_linear(o, i, V, 0.9, seed=s)
+    layer = SparseEncoderLayer(hidden, heads, ffn, mk(hidden, hidden, 1), mk(hidden, hidden, 2), mk(hidden, hidden, 3),
+                               mk(hidden, hidden, 4), mk(ffn, hidden, 5), mk(hidden, ffn, 6)).cuda().half()
+    x = torch.randn(hidden, batch * seq, device="cuda", generator=torch.Generator("cuda").manual_seed(6)).half()
+    dense = {n: getattr(layer, n).dense_weight().float() for n in ("qkv", "o", "ffn1", "ffn2")}
+    assert torch.equal(dense["qkv"], torch.cat([layer.q.dense_weight(), layer.k.dense_weight(), layer.v.dense_weight()]).float())
+    # the weights are held once: q, k and v are views of the fused layer's arrays, and state_dict names them once
+    assert layer.q.values.data_ptr() == layer.qkv.values.data_ptr()
+    assert not any(key.startswith(("q.", "k.", "v.", "ffn1_gelu.")) for key in layer.state_dict())
+    gelu = torch.nn.functional.gelu
+    with torch.no_grad():
+        got = layer(x, batch, seq)
+        want = layer(x, batch, seq, linear=lambda name, lin, t: (
+            gelu(dense["ffn1"] @ t.float()) if name == "ffn1_gelu" else dense[name] @ t.float()).half())
+    assert got.shape == (hidden, batch * seq)
+    assert max_rel_err(got.float().cpu().numpy(), want.float().cpu().numpy()) <= 1e-2
+
+
+def test_sparse_linear_drops_its_plan_when_the_buffers_move(built_library):
+    lin = _vector_sparse_linear(256, 192, 16, 0.8, seed=72)
+    lin.make_plan(64)
+    assert lin.plan is not None
+    lin = lin.half()   # any conversion or move goes through _apply
+    assert lin.plan is None
+    x = torch.randn(192, 64, device="cuda", generator=torch.Generator("cuda").manual_seed(7)).half()
+    want = lin.dense_weight().float() @ x.float()
+    assert max_rel_err(lin(x).float().cpu().numpy(), want.cpu().numpy()) <= 2e-3
+
+
 @pytest.mark.parametrize("V,out_f,in_f,N", [(16, 3072, 768, 4096), (8, 64, 100, 72), (16, 128, 5000, 64), (8, 256, 96, 33)])
 @pytest.mark.parametrize("activation", [None, "gelu"])
 @pytest.mark.parametrize("with_bias", [False, True])

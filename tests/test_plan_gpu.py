@@ -279,3 +279,35 @@ def test_plan_of_an_even_pattern_picks_the_kernel_by_density(oracle, built_libra
         assert max_rel_err(planned[b].cpu().numpy(), want) <= TIGHT_F32
         assert max_rel_err(plain[b].cpu().numpy(), want) <= TIGHT_F32
     plan.destroy()
+
+
+def test_many_panels_give_the_same_bits_twenty_times_in_a_row(oracle, built_library):
+    """More than 1000 panels over 9 column tiles and 2 batch elements (their partial tiles just fit the plan's 64 MB): the cut rows are added up by whichever wave
+    counts itself in last, on whichever XCD it runs, so a hand-over that lets a wave read a partial tile before it
+    has arrived shows as a run that differs from the first.  Twenty consecutive products are compared bit for bit
+    and the test stops at the first mismatch."""
+    V, K, N, batch = 8, 12000, 520, 2
+    rng = np.random.default_rng(901)
+    lens = rng.integers(0, 40, 600)
+    long_rows = rng.choice(600, 150, replace=False)
+    lens[long_rows] = rng.integers(900, 3000, 150)
+    vs = ragged(len(lens), K, V, lens, seed=902)
+    vals = (rng.standard_normal((batch, vs.values.size)) * 0.1).astype(np.float16)
+    B = rng.standard_normal((batch, K, N)).astype(np.float16)
+    ro, ci, dv, dB = dev(vs.row_offsets), dev(vs.col_idx), dev(vals), dev(B)
+    plan = Plan(ro, V, K, max_N=N, max_batch=batch, panel_steps=8)
+    info = plan.info()
+    assert info.panels >= 1000 and info.cut_rows >= 100, info
+    first = None
+    for it in range(20):
+        out = sspmm_amd.bspmm(None, ro, ci, dv, dB, V, out_dtype=torch.float32, plan=plan)
+        torch.cuda.synchronize()
+        assert _lib.lib().sspmm_last_kernel() == BALANCED
+        if first is None:
+            first = out.clone()
+        else:
+            assert torch.equal(out, first), "run %d differs from the first in %d elements" % (it, int((out != first).sum()))
+    # and the first is right: one batch element against the oracle
+    want = oracle.spmm(vs.m_vec, V, N, K, vs.row_offsets, vs.col_idx, vals[1], B[1], threads=8)
+    assert max_rel_err(first[1].cpu().numpy(), want) <= TIGHT_F32
+    plan.destroy()

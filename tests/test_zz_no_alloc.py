@@ -107,3 +107,43 @@ def test_sizes_beyond_the_static_scratch_are_rejected(built_library):
     assert b"static scratch" in L.sspmm_error_string(too_small)
     assert L.sspmm_noalloc_f16_f32(64, 4, 64, 64, one, one, one, one, one, None) == 1
     assert L.sspmm_noalloc_f16_f32(0, 8, 64, 64, None, None, None, None, None, None) == 0
+
+
+def test_two_patterns_recorded_into_one_graph(built_library):
+    """The entry point is for callers under graph capture: after one eager call (the array's address is looked up
+    outside a capture), two calls with different patterns are recorded on one stream and the graph is replayed several
+    times with eager work in between; every replay equals the eager results bit for bit."""
+    L = _lib.lib()
+    V = 8
+    pa = _pattern(300, 6000, V, seed=31, long_rows=24)
+    pb = _pattern(90, 3000, V, seed=32, long_rows=5)
+    Ba, Bb = dev(synth.dense_rhs(6000, 128, seed=3)), dev(synth.dense_rhs(3000, 64, seed=4))
+    arrs = [(p, dev(p.row_offsets), dev(p.col_idx), dev(p.values)) for p in (pa, pb)]
+
+    def call(i, B, N, out, stream):
+        p, ro, ci, vv = arrs[i]
+        rc = L.sspmm_noalloc_f16_f32(p.m_vec, V, N, p.K, ro.data_ptr(), ci.data_ptr(), vv.data_ptr(), B.data_ptr(),
+                                     out.data_ptr(), stream)
+        assert rc == 0, rc
+
+    eager = [torch.empty(pa.m_vec * V, 128, device="cuda"), torch.empty(pb.m_vec * V, 64, device="cuda")]
+    s0 = torch.cuda.current_stream().cuda_stream
+    call(0, Ba, 128, eager[0], s0)
+    call(1, Bb, 64, eager[1], s0)
+    torch.cuda.synchronize()
+    outs = [torch.zeros_like(e) for e in eager]
+    side = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side):
+        st = torch.cuda.current_stream().cuda_stream
+        call(0, Ba, 128, outs[0], st)
+        call(1, Bb, 64, outs[1], st)
+    for replay in range(4):
+        for o in outs:
+            o.fill_(float(replay))          # eager work of the program's own between the replays
+        call(1, Bb, 64, eager[1], s0)       # ... including a call that leaves another schedule in the array
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(outs[0], eager[0]), replay
+        assert torch.equal(outs[1], eager[1]), replay

@@ -343,6 +343,21 @@ def run_cfg1(L, torch, synth, sspmm_amd, O, st, wu):
            "cpu_pipeline_ms": sorted(py)[len(py) // 2] + cpu_spmm_ms,
            "svc_bit_exact_vs_python": bool(same), "spmm_max_rel_err_vs_host_loop": err}
     res["speedup_pipeline"] = res["cpu_pipeline_ms"] / t_pipe
+    res["svc_speedup_vs_python_one_matrix_per_call"] = res["cpu_python_rowmerge_ms"] / t_svc
+    # one such matrix is three launches and a chain of LDS round trips on an idle chip; the reference's job is a
+    # dataset of them, so: 96 matrices of this configuration (seeds 1 .. 96) as one stack through svc_batched
+    many = [synth.expand_to_csr(synth.vector_sparse(512, K, V, 0.9, seed=s)) for s in range(1, 97)]
+    mat_rows, K_max, s_rp, s_ci, _ = sspmm_amd.stack_csr([(c.M, c.K, c.row_ptr, c.col_ind, None) for c in many])
+    d_rp, d_ci = torch.from_numpy(s_rp).cuda(), torch.from_numpy(s_ci).cuda()
+    t_stack = time_launches(lambda: sspmm_amd.svc_batched(mat_rows, K_max, d_rp, d_ci, None, V), 20, 3)
+    t0 = time.perf_counter()
+    want96 = [O.rowmerge_python(c.M, V, O.csr_col_lists(c.M, c.row_ptr, c.col_ind)) for c in many]
+    py96 = (time.perf_counter() - t0) * 1e3
+    got96 = sspmm_amd.svc_batched(mat_rows, K_max, d_rp, d_ci, None, V).to_host()
+    res["svc_stack_of_96_such_matrices"] = {
+        "gpu_ms": t_stack, "gpu_ms_per_matrix": t_stack / 96, "python_rowmerge_ms": py96,
+        "speedup_vs_python": py96 / t_stack,
+        "bit_exact_vs_python": bool(all(g[0].tolist() == w[0] and g[1].tolist() == w[1] for g, w in zip(got96, want96)))}
     res["spmm"] = figures(t_spmm, by, 2.0 * vs.nnz * N)
     return res
 
@@ -473,6 +488,59 @@ def run_cfg4(L, torch, synth, sspmm_amd, O, st, wu):
                                         rd.vec_col.cpu().numpy().tolist() == d_want_cols),
             "nnz": int(d_col.size), "nvec": int(rd.num_vec),
         }
+    return out
+
+
+def run_svc_batched(L, torch, synth, sspmm_amd, O):
+    """The shape of the reference's RowMerge job (a loop over a dataset of small pruned-weight matrices,
+    sparse_matrix_format.py:190-250): 96 seeded unstructured matrices of the dataset's shapes (512x512, 2048x512,
+    512x2048) at 50 to 98 % sparsity, V = 8 and 16, as ONE stack through svc_batched against the Python RowMerge loop
+    over the same matrices, single thread."""
+    shapes = [(512, 512), (2048, 512), (512, 2048)]
+    sparsities = [0.5, 0.7, 0.8, 0.9, 0.95, 0.98]
+    rng = np.random.default_rng(96)
+    mats = []
+    for i in range(96):
+        M, K = shapes[i % 3]
+        mask = rng.random((M, K)) >= sparsities[(i // 3) % 6]
+        ptr = np.concatenate([[0], np.cumsum(mask.sum(axis=1))]).astype(np.int32)
+        mats.append((M, K, ptr, np.nonzero(mask)[1].astype(np.int32), None))
+    mat_rows, K_max, rp, ci, _ = sspmm_amd.stack_csr(mats)
+    d_rp, d_ci = torch.from_numpy(rp).cuda(), torch.from_numpy(ci).cuda()
+    lists = [O.csr_col_lists(m[0], m[2], m[3]) for m in mats]
+    out = {"workload": "96 unstructured matrices (512x512, 2048x512, 512x2048; 50-98 %% sparse), nnz %d in all, one stack" % ci.size,
+           "matrices": len(mats), "nnz": int(ci.size)}
+    for V in (8, 16):
+        batch = sspmm_amd.svc_batched(mat_rows, K_max, d_rp, d_ci, None, V)
+        torch.cuda.synchronize()
+        gpu_ms = time_launches(lambda: sspmm_amd.svc_batched(mat_rows, K_max, d_rp, d_ci, None, V), 10, 2)
+        # the whole job as the converter runs it: stack on the host, upload, merge, one copy back, split per matrix
+        t0 = time.perf_counter()
+        mr2, km2, rp2, ci2, _ = sspmm_amd.stack_csr(mats)
+        host = sspmm_amd.svc_batched(mr2, km2, torch.from_numpy(rp2).cuda(), torch.from_numpy(ci2).cuda(), None, V).to_host()
+        job_ms = (time.perf_counter() - t0) * 1e3
+        # one matrix per call, as before (read-back of nvec per matrix)
+        dm = [(torch.from_numpy(m[2]).cuda(), torch.from_numpy(m[3]).cuda()) for m in mats]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for (M, K, _p, _c, _v), (a, b) in zip(mats, dm):
+            sspmm_amd.svc(a, b, None, M, K, V)
+        torch.cuda.synchronize()
+        loop_ms = (time.perf_counter() - t0) * 1e3
+        t0 = time.perf_counter()
+        want = [O.rowmerge_python(m[0], V, l) for m, l in zip(mats, lists)]
+        py_ms = (time.perf_counter() - t0) * 1e3
+        same = all(h[0].tolist() == w[0] and h[1].tolist() == w[1] for h, w in zip(host, want))
+        nvec = int(sum(len(w[1]) for w in want))
+        alg = sum(synth.svc_algorithmic_bytes(m[0], int(m[3].size), -(-m[0] // V), len(w[1]), V) for m, w in zip(mats, want))
+        out["v%d" % V] = {"gpu_ms": gpu_ms, "gpu_ms_one_call_per_matrix": loop_ms,
+                          "gpu_ms_whole_job_with_stacking_upload_and_copy_back": job_ms,
+                          "python_rowmerge_ms": py_ms, "speedup_vs_python": py_ms / gpu_ms,
+                          "speedup_vs_python_whole_job": py_ms / job_ms, "bit_exact_vs_python": bool(same), "nvec": nvec,
+                          "alg_bytes": alg, "hbm_frac": alg / gpu_ms / 1e6 / HBM_PEAK_GBPS}
+        del batch, host, dm
+    out["speedup_vs_python"] = min(out["v8"]["speedup_vs_python"], out["v16"]["speedup_vs_python"])
+    out["cpu_cores"] = 1
     return out
 
 
@@ -614,7 +682,7 @@ def run_reorder(L, torch, synth, sspmm_amd):
 
 
 ATTENTION = "sparse_attention_seq4096_d64_v8_s0.9_heads48"
-GROUPS = ["cfg1_rowmerge_then_spmm_512x512", "cfg4", "cfg5_encoder_layer_v16_s0.9_tokens4096", ATTENTION,
+GROUPS = ["cfg1_rowmerge_then_spmm_512x512", "cfg4", "svc_batched_dlmc_shapes", "cfg5_encoder_layer_v16_s0.9_tokens4096", ATTENTION,
           "reorder_clustered_16384_v8", "headline_batched_cold"]
 
 
@@ -663,6 +731,8 @@ def run_extra(name, env):
         return {name: run_cfg1(L, torch, synth, sspmm_amd, O, st, wu)}
     if name == "cfg4":
         return run_cfg4(L, torch, synth, sspmm_amd, O, st, wu)
+    if name == "svc_batched_dlmc_shapes":
+        return {name: run_svc_batched(L, torch, synth, sspmm_amd, O)}
     if name == "cfg5_encoder_layer_v16_s0.9_tokens4096":
         return {name: run_cfg5_layer(L, torch, synth, st, wu)}
     if name == ATTENTION:
@@ -906,6 +976,7 @@ def short_extra(extra):
         "cfg4_spmm_with_plan_ms": ("cfg4_spmm_on_svc_output_with_plan", "ms"),
         "svc_cfg4_speedup_vs_python": ("svc_cfg4_zipf_16384_v8", "speedup_vs_python"),
         "svc_batched_dlmc_shapes_speedup_vs_python": ("svc_batched_dlmc_shapes", "speedup_vs_python"),
+        "cfg1_svc_stack_of_96_speedup_vs_python": ("cfg1_rowmerge_then_spmm_512x512", "svc_stack_of_96_such_matrices", "speedup_vs_python"),
         "cfg5_layer_speedup_vs_dense_in_a_graph": ("cfg5_encoder_layer_v16_s0.9_tokens4096", "speedup_vs_dense_layer_in_a_graph"),
         "sparse_attention_forward_seq4096_ms": ("sparse_attention_forward_seq4096_h4_e256_s0.9_b2_l4", "ms"),
     }

@@ -257,6 +257,40 @@ int svc_fill(int M, int K, int V, const int32_t *row_ptr, const int32_t *col_ind
              sspmm_half_t *vec_val, void *hip_stream);
 
 /* ------------------------------------------------------------------------------------------
+ * The SVC of many matrices in one chain of launches.  The reference's RowMerge job is a loop
+ * over a dataset of small matrices, one CVSE per file (generate_CVSE_file, reference
+ * RowMerge/sparse_matrix_format.py:190-250: 2688 matrices, driven twice by RowMerge/row_merge.py:
+ * 16-18); one matrix at a time leaves a GPU idle behind launch latencies.  Here the matrices are
+ * stacked along the rows into one CSR:
+ *   mat_rows[count + 1]  device: first row of matrix i in the stack, mat_rows[count] = M_total
+ *   row_ptr[M_total + 1] device: row pointer of the stack (entry offsets into col_ind / csr_val of
+ *                        the whole stack), col_ind[nnz], csr_val[nnz]
+ *   K_max                the largest column count of the stack (column indices of every matrix lie
+ *                        below its own K, so below K_max)
+ *   groups               sum over the matrices of ceil(rows / V), computed by the caller
+ * A matrix whose row count is not a multiple of V ends with a short group, as it does on its own
+ * (sparse_matrix_format.py:109), and the next matrix starts a new one.  Outputs, in the stack's order:
+ *   mat_groups[count + 1]    first group of matrix i; mat_groups[count] is the group count the device
+ *                            arrived at (equal to `groups` unless the caller miscounted)
+ *   vec_row_ptr[groups + 1]  over all groups: matrix i's own row pointer is
+ *                            vec_row_ptr[mat_groups[i] + j] - vec_row_ptr[mat_groups[i]]
+ *   vec_col / vec_val        the matrices' vectors one after the other; sized for the bound nvec <= nnz
+ *                            nothing has to be read back between the two phases
+ * Workspace of svc_batched_workspace_bytes(count, M_total, nnz, V) bytes, the same for both phases.
+ * Results per matrix are those of svc_count / svc_fill on that matrix alone, bit for bit.
+ * ---------------------------------------------------------------------------------------- */
+size_t svc_batched_workspace_bytes(int count, int M_total, int64_t nnz, int V);
+
+int svc_count_batched(int count, int groups, const int32_t *mat_rows, int M_total, int K_max, int V,
+                      const int32_t *row_ptr, const int32_t *col_ind, int64_t nnz, int order, int32_t *mat_groups,
+                      int32_t *vec_row_ptr, void *workspace, void *hip_stream);
+
+int svc_fill_batched(int count, int groups, const int32_t *mat_rows, int M_total, int K_max, int V,
+                     const int32_t *row_ptr, const int32_t *col_ind, const sspmm_half_t *csr_val, int64_t nnz, int order,
+                     const int32_t *vec_row_ptr, void *workspace, int32_t *vec_col, sspmm_half_t *vec_val,
+                     void *hip_stream);
+
+/* ------------------------------------------------------------------------------------------
  * Row reordering ahead of the SVC: the step the reference runs as `python row_merge_reorder.py`
  * (reference README.md:36) to write its dataset-v8 / dataset-v16 folders, which the harness
  * reads when its `reorder` argument is 1 (reference SSpMM/sspmm_test.cpp:304, 313-320).  The

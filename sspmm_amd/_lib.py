@@ -36,6 +36,9 @@ SIGNATURES = {
     "svc_workspace_bytes": (ctypes.c_size_t, [_int, _i64, _int]),
     "svc_count": (_int, [_int, _int, _int, _vp, _vp, _i64, _int, _vp, _vp, _vp]),
     "svc_fill": (_int, [_int, _int, _int, _vp, _vp, _vp, _i64, _int, _vp, _vp, _vp, _vp, _vp]),
+    "svc_batched_workspace_bytes": (ctypes.c_size_t, [_int, _int, _i64, _int]),
+    "svc_count_batched": (_int, [_int, _int, _vp, _int, _int, _int, _vp, _vp, _i64, _int, _vp, _vp, _vp, _vp]),
+    "svc_fill_batched": (_int, [_int, _int, _vp, _int, _int, _int, _vp, _vp, _vp, _i64, _int, _vp, _vp, _vp, _vp, _vp]),
     "sspmm_add_layernorm_f16": (_int, [_int, _int, _vp, _vp, _vp, _vp, ctypes.c_float, _vp, _vp]),
     "sspmm_linear_f16": (_int, [_int, _int, _int, _int, _vp, _vp, _vp, _vp, _vp, _int, _vp, _vp]),
     "sspmm_attention_fm_f16": (_int, [_int, _int, _int, _int, _vp, _vp, _vp, ctypes.c_int64, _vp, ctypes.c_int64, ctypes.c_float, _vp]),

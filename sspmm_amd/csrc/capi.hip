@@ -316,6 +316,72 @@ int svc_fill(int M, int K, int V, const int32_t *row_ptr, const int32_t *col_ind
                                      static_cast<hipStream_t>(hip_stream));
 }
 
+// A stack of matrices: the single-matrix workspace for the stacked CSR with room for one short group per matrix,
+// then the table of every group's first row.
+static size_t svc_batched_layout(int count, int M_total, int64_t nnz, int V, size_t *off_group_rows) {
+  const int groups_bound = M_total / V + count;
+  const size_t base = sspmm::svc_workspace_layout(nnz, groups_bound, nullptr, nullptr, nullptr);
+  if (off_group_rows) *off_group_rows = base;
+  return base + (((size_t)groups_bound + 2) * 4 + 255) / 256 * 256;
+}
+
+size_t svc_batched_workspace_bytes(int count, int M_total, int64_t nnz, int V) {
+  if (count < 0 || M_total < 0 || V < 1) return 0;
+  return svc_batched_layout(count, M_total, nnz, V, nullptr);
+}
+
+static int svc_batched_args(int count, int groups, const int32_t *mat_rows, int M_total, int K_max, int V,
+                            const int32_t *row_ptr, const int32_t *col_ind, int64_t nnz, void *workspace,
+                            sspmm::SvcArgs *a, int32_t **group_rows) {
+  if (count < 0 || groups < 0 || groups > M_total / (V > 0 ? V : 1) + count || !mat_rows) return kInvalid;
+  const int rc = svc_args(M_total, K_max, V, row_ptr, col_ind, nnz, workspace, a);
+  if (rc) return rc;
+  // (the views of the single-matrix layout, laid out for the most groups the stack can have)
+  size_t off_pos, off_tables, off_lists, off_group_rows;
+  const int groups_bound = M_total / V + count;
+  sspmm::svc_workspace_layout(nnz, groups_bound, &off_pos, &off_tables, &off_lists);
+  svc_batched_layout(count, M_total, nnz, V, &off_group_rows);
+  unsigned char *w = static_cast<unsigned char *>(workspace);
+  a->class_counts = reinterpret_cast<int32_t *>(w + off_lists);
+  a->class_lists = a->class_counts + 64;
+  a->list_stride = groups_bound > 0 ? groups_bound : 1;
+  *group_rows = reinterpret_cast<int32_t *>(w + off_group_rows);
+  a->group_rows = *group_rows;
+  a->groups = groups;
+  return 0;
+}
+
+int svc_count_batched(int count, int groups, const int32_t *mat_rows, int M_total, int K_max, int V,
+                      const int32_t *row_ptr, const int32_t *col_ind, int64_t nnz, int order, int32_t *mat_groups,
+                      int32_t *vec_row_ptr, void *workspace, void *hip_stream) {
+  sspmm::SvcArgs a{};
+  int32_t *group_rows = nullptr;
+  if (order != SVC_ORDER_CPYTHON && order != SVC_ORDER_SORTED) return kInvalid;
+  if (!vec_row_ptr || !mat_groups) return kInvalid;
+  const int rc = svc_batched_args(count, groups, mat_rows, M_total, K_max, V, row_ptr, col_ind, nnz, workspace, &a, &group_rows);
+  if (rc) return rc;
+  a.vec_row_ptr = vec_row_ptr;
+  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+  const hipError_t e = sspmm::launch_svc_group_rows(count, V, groups, mat_rows, group_rows, mat_groups, stream);
+  if (e != hipSuccess) return (int)e;
+  return (int)sspmm::launch_svc_count(a, order, stream);
+}
+
+int svc_fill_batched(int count, int groups, const int32_t *mat_rows, int M_total, int K_max, int V,
+                     const int32_t *row_ptr, const int32_t *col_ind, const sspmm_half_t *csr_val, int64_t nnz, int order,
+                     const int32_t *vec_row_ptr, void *workspace, int32_t *vec_col, sspmm_half_t *vec_val,
+                     void *hip_stream) {
+  sspmm::SvcArgs a{};
+  int32_t *group_rows = nullptr;
+  if (order != SVC_ORDER_CPYTHON && order != SVC_ORDER_SORTED) return kInvalid;
+  if (!vec_row_ptr) return kInvalid;
+  if (csr_val && !vec_val) return kInvalid;
+  const int rc = svc_batched_args(count, groups, mat_rows, M_total, K_max, V, row_ptr, col_ind, nnz, workspace, &a, &group_rows);
+  if (rc) return rc;
+  if (groups == 0) return 0;
+  return (int)sspmm::launch_svc_fill(a, order, csr_val, vec_row_ptr, vec_col, vec_val, static_cast<hipStream_t>(hip_stream));
+}
+
 size_t svc_reorder_workspace_bytes(int M) { return sspmm::reorder_workspace_bytes(M); }
 
 int svc_reorder_minhash(int M, const int32_t *row_ptr, const int32_t *col_ind, int32_t *perm, void *workspace,

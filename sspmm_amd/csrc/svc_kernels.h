@@ -28,6 +28,9 @@ struct SvcArgs {
   int32_t *class_counts;         // [5]
   int32_t *class_lists;          // [5][list_stride]
   int list_stride;
+  // a stack of matrices (batched entry points): first row of every group, [groups + 1]; null for a single matrix
+  const int32_t *group_rows;
+  int groups;
 };
 
 // True when svc_count only counts (bitmap pass) and svc_fill runs the merge and writes the outputs directly.
@@ -36,6 +39,9 @@ bool svc_direct(int order, int K);
 // Total workspace bytes; optional byte offsets of the pos, table and class-list views.
 size_t svc_workspace_layout(int64_t nnz, int m_vec, size_t *off_pos, size_t *off_tables, size_t *off_lists);
 
+// group_rows[groups + 1] and mat_groups[count + 1] of a stack of matrices from mat_rows[count + 1] (device arrays).
+hipError_t launch_svc_group_rows(int count, int V, int groups, const int32_t *mat_rows, int32_t *group_rows,
+                                 int32_t *mat_groups, hipStream_t stream);
 hipError_t launch_svc_count(const SvcArgs &a, int order, hipStream_t stream);
 hipError_t launch_svc_fill(const SvcArgs &a, int order, const uint16_t *csr_val, const int32_t *vec_row_ptr,
                            int32_t *vec_col, uint16_t *vec_val, hipStream_t stream);

@@ -217,6 +217,40 @@ __device__ __forceinline__ uint32_t rebuild_set(u64 *table, int *list, int &n, i
   }
 }
 
+// First member row of group grp (grp = number of groups: one past the last row).  A single matrix's groups are V
+// rows each, the last one what is left; a stack of matrices (the batched entry points) brings a table, because a
+// matrix whose row count is not a multiple of V ends with a short group and the next one starts a new group.
+__device__ __forceinline__ int group_first_row(const SvcArgs &a, int grp) {
+  return a.group_rows ? a.group_rows[grp] : min(a.M, grp * a.V);
+}
+
+// The table of a stack of `count` matrices: mat_rows[i] is the first row of matrix i in the stack (mat_rows[count]
+// the total), group_rows[g] the first row of group g, group_rows[groups] the total, mat_groups[i] the first group of
+// matrix i.  One workgroup; matrices in tiles of 1024.
+__global__ __launch_bounds__(1024) void svc_group_rows_kernel(int count, int V, int groups, const int32_t *mat_rows,
+                                                              int32_t *group_rows, int32_t *mat_groups) {
+  __shared__ int scratch[32];
+  int carry = 0;
+  for (int base = 0; base < count; base += 1024) {
+    const int i = base + (int)threadIdx.x;
+    const int r0 = i < count ? mat_rows[i] : 0, r1 = i < count ? mat_rows[i + 1] : 0;
+    const int n = (r1 - r0 + V - 1) / V;
+    int total;
+    const int first = carry + block_exclusive_scan<1024>(n, &total, scratch);
+    if (i < count) {
+      mat_groups[i] = first;
+      // (never past the table the caller sized for `groups` groups: a wrong count shows in mat_groups[count])
+      for (int g = 0; g < n && first + g < groups; ++g) group_rows[first + g] = r0 + g * V;
+    }
+    carry += total;
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    mat_groups[count] = carry;
+    group_rows[groups] = mat_rows[count];
+  }
+}
+
 // Class of a vector-row group by its key bound: which kernel instance handles it.
 __device__ __forceinline__ bool in_class(int bound, int lo, int hi) { return bound > lo && bound <= hi; }
 
@@ -225,7 +259,7 @@ template <int THREADS>
 __global__ __launch_bounds__(THREADS) void svc_count_distinct_kernel(const SvcArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int grp = blockIdx.x;
-  const int r0 = grp * a.V, r1 = min(a.M, r0 + a.V);
+  const int r0 = group_first_row(a, grp), r1 = group_first_row(a, grp + 1);
   const int e0 = a.row_ptr[r0], e1 = a.row_ptr[r1];
   if (e1 - e0 <= 1) {  // nothing to deduplicate
     if (threadIdx.x == 0) a.vec_row_ptr[grp + 1] = e1 - e0;
@@ -314,10 +348,10 @@ __global__ __launch_bounds__(THREADS) void svc_merge_cpython_kernel(const SvcArg
   // Direct mode walks the list of the groups of its class (kClassBeyond); otherwise there is one workgroup per
   // group, which leaves unless the group's bound on its columns falls into the launch's class.
   const bool listed = a.scanned != nullptr;
-  const int n_groups = listed ? a.class_counts[kClassBeyond] : (a.M + a.V - 1) / a.V;
+  const int n_groups = listed ? a.class_counts[kClassBeyond] : (a.group_rows ? a.groups : (a.M + a.V - 1) / a.V);
   for (int li = blockIdx.x; li < n_groups; li += gridDim.x) {
   const int grp = listed ? a.class_lists[(int64_t)kClassBeyond * a.list_stride + li] : li;
-  const int r0 = grp * a.V, r1 = min(a.M, r0 + a.V);
+  const int r0 = group_first_row(a, grp), r1 = group_first_row(a, grp + 1);
   const int e0 = a.row_ptr[r0], e1 = a.row_ptr[r1];
   const int bound = listed ? a.scanned[grp + 1] - a.scanned[grp] : min(e1 - e0, a.K);
   if (!listed && !in_class(bound, class_lo, class_hi)) continue;  // uniform over the group
@@ -765,7 +799,7 @@ __global__ __launch_bounds__(THREADS) void svc_merge_fast_kernel(const SvcArgs a
   int c = cls, at = li;
   while (at >= a.class_counts[c]) at -= a.class_counts[c--];
   const int grp = a.class_lists[(int64_t)c * a.list_stride + at];
-  const int r0 = grp * a.V, r1 = min(a.M, r0 + a.V);
+  const int r0 = group_first_row(a, grp), r1 = group_first_row(a, grp + 1);
   const int count = a.scanned[grp + 1] - a.scanned[grp];
   const int e0 = a.row_ptr[r0];
 
@@ -871,7 +905,7 @@ template <int THREADS>
 __global__ __launch_bounds__(THREADS) void svc_merge_sorted_kernel(const SvcArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int grp = blockIdx.x;
-  const int r0 = grp * a.V, r1 = min(a.M, r0 + a.V);
+  const int r0 = group_first_row(a, grp), r1 = group_first_row(a, grp + 1);
   const int e0 = a.row_ptr[r0], e1 = a.row_ptr[r1];
   const int words = (a.K + 31) / 32;
   int *scratch = reinterpret_cast<int *>(smem);
@@ -963,7 +997,7 @@ __global__ __launch_bounds__(THREADS) void svc_fill_kernel(const SvcArgs a, cons
                                                           const int32_t *vec_row_ptr, int32_t *vec_col,
                                                           uint16_t *vec_val) {
   const int grp = blockIdx.x;
-  const int r0 = grp * a.V, r1 = min(a.M, r0 + a.V);
+  const int r0 = group_first_row(a, grp), r1 = group_first_row(a, grp + 1);
   const int e0 = a.row_ptr[r0];
   const int v0 = vec_row_ptr[grp], n = vec_row_ptr[grp + 1] - v0;
   if (vec_col)
@@ -1130,8 +1164,14 @@ static hipError_t join_streams(SideStreams *ss, hipStream_t stream, int helpers 
   return hipSuccess;
 }
 
+hipError_t launch_svc_group_rows(int count, int V, int groups, const int32_t *mat_rows, int32_t *group_rows,
+                                 int32_t *mat_groups, hipStream_t stream) {
+  hipLaunchKernelGGL(svc_group_rows_kernel, dim3(1), dim3(1024), 0, stream, count, V, groups, mat_rows, group_rows, mat_groups);
+  return hipGetLastError();
+}
+
 hipError_t launch_svc_count(const SvcArgs &a, int order, hipStream_t stream) {
-  const int m_vec = (a.M + a.V - 1) / a.V;
+  const int m_vec = a.group_rows ? a.groups : (a.M + a.V - 1) / a.V;
   hipError_t e;
   if (m_vec == 0) {
     // no groups: only the scan runs, which writes vec_row_ptr[0] = 0 (and empty class lists)
@@ -1181,7 +1221,7 @@ hipError_t launch_svc_count(const SvcArgs &a, int order, hipStream_t stream) {
 
 hipError_t launch_svc_fill(const SvcArgs &args, int order, const uint16_t *csr_val, const int32_t *vec_row_ptr,
                            int32_t *vec_col, uint16_t *vec_val, hipStream_t stream) {
-  const int m_vec = (args.M + args.V - 1) / args.V;
+  const int m_vec = args.group_rows ? args.groups : (args.M + args.V - 1) / args.V;
   if (!svc_direct(order, args.K)) {
     hipLaunchKernelGGL((svc_fill_kernel<512>), dim3(m_vec), dim3(512), 0, stream, args, csr_val, vec_row_ptr, vec_col,
                        csr_val ? vec_val : nullptr);

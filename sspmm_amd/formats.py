@@ -24,6 +24,13 @@ def read_smtx(path):
     return M, K, nnz, row_ptr, col_ind
 
 
+def read_smtx_header(path):
+    """-> (M, K, nnz) of a `.smtx` file: its first line alone."""
+    with open(path) as f:
+        M, K, nnz = (int(x) for x in f.readline().split(", "))
+    return M, K, nnz
+
+
 def write_smtx(path, M, K, row_ptr, col_ind):
     with open(path, "w") as f:
         f.write("%d, %d, %d\n" % (M, K, len(col_ind)))

@@ -72,17 +72,65 @@ def convert_file(src_path, dest_path, vec_len, order="cpython", reorder=False):
     return statistics(M, K, nnz, vec_len, vec_row_ptr)
 
 
+# entries of one batched call: the stack's CSR, the workspace (16 x) and the outputs stay well inside a GPU's memory
+BATCH_NNZ = 32 << 20
+
+
+def convert_files(src_paths, dest_paths, vec_len, order="cpython"):
+    """Many `.smtx` files -> as many CVSE files with ONE chain of GPU launches: the matrices are read, stacked along
+    the rows, merged by svc_batched, brought back with one copy and written.  Returns the statistics dicts."""
+    import torch
+
+    from . import formats
+    from .svc import stack_csr, svc_batched
+    mats = []
+    for p in src_paths:
+        M, K, nnz, row_ptr, col_ind = formats.read_smtx(p)
+        mats.append((M, K, row_ptr, col_ind, None))
+    mat_rows, K_max, rp, ci, _ = stack_csr(mats)
+    batch = svc_batched(mat_rows, K_max, torch.from_numpy(rp).cuda(), torch.from_numpy(ci).cuda(), None, vec_len, order=order)
+    stats = []
+    for (M, K, row_ptr, col_ind, _), dest, (vec_row_ptr, vec_col, _v) in zip(mats, dest_paths, batch.to_host()):
+        os.makedirs(os.path.dirname(os.path.abspath(dest)), exist_ok=True)
+        formats.write_cvse(dest, vec_row_ptr.size - 1, K, int(col_ind.size), vec_row_ptr, vec_col)
+        stats.append(statistics(M, K, int(col_ind.size), vec_len, vec_row_ptr))
+    return stats
+
+
 def generate_cvse_files(src_dir, dest_dir, paths_txt, vec_len, csv_path=None, order="cpython", log=None,
                         reorder=False):
-    """Every file named in paths_txt (first token of each line, relative to src_dir / dest_dir)."""
+    """Every file named in paths_txt (first token of each line, relative to src_dir / dest_dir).  Without
+    `reorder` the files go through the GPU in stacks (convert_files) of up to BATCH_NNZ entries, so the dataset
+    costs a handful of launch chains instead of one per file."""
     with open(paths_txt) as f:
         names = [line.split()[0] for line in f if line.split()]
     rows = []
-    for i, name in enumerate(names):
-        stats = convert_file(os.path.join(src_dir, name), os.path.join(dest_dir, name), vec_len, order, reorder)
-        rows.append(csv_row(i, stats))
-        if log:
-            log("No. %d  OK  %s" % (i, os.path.join(dest_dir, name)))
+    if reorder:
+        for i, name in enumerate(names):
+            stats = convert_file(os.path.join(src_dir, name), os.path.join(dest_dir, name), vec_len, order, reorder)
+            rows.append(csv_row(i, stats))
+            if log:
+                log("No. %d  OK  %s" % (i, os.path.join(dest_dir, name)))
+    else:
+        from . import formats
+        start = 0
+        while start < len(names):
+            # a stack ends before the file that would take it past BATCH_NNZ entries (the header line names the count)
+            end, total = start, 0
+            while end < len(names):
+                n = formats.read_smtx_header(os.path.join(src_dir, names[end]))[2]
+                if end > start and total + n > BATCH_NNZ:
+                    break
+                total += n
+                end += 1
+            chunk = names[start:end]
+            stats = convert_files([os.path.join(src_dir, n) for n in chunk], [os.path.join(dest_dir, n) for n in chunk],
+                                  vec_len, order)
+            for k, st in enumerate(stats):
+                rows.append(csv_row(start + k, st))
+                if log:
+                    log("No. %d  OK  %s" % (start + k, os.path.join(dest_dir, chunk[k])))
+            start = end
     if csv_path:
         with open(csv_path, "a", newline="") as f:  # the reference appends too
             csv.writer(f).writerows(rows)

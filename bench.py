@@ -270,6 +270,10 @@ def single_launch_cases(batch):
             if (M, K, s) != (2048, 512, 0.9):
                 cases["cfg2_%dx%d_v8_s%g_batched" % (M, K, s)] = dict(M=M, K=K, V=8, sparsity=s, N=256, batch=batch,
                                                                       out_f32=True, std=0.02, seed=2)
+    # cfg2's shapes at N = 512, the width of the reference's published sweep (SSpMM/Makefile_ampere:55-60)
+    for (M, K) in ((2048, 512), (512, 2048), (2048, 2048)):
+        cases["dlmc_shape_%dx%d_v8_s0.9_n512_batched" % (M, K)] = dict(M=M, K=K, V=8, sparsity=0.9, N=512, batch=batch // 2,
+                                                                       out_f32=False, std=0.02, seed=2)
     cases["cfg2_batched_fp16_out"] = dict(M=2048, K=512, V=8, sparsity=0.9, N=256, batch=batch, out_f32=False, std=0.02, seed=2)
     cases["cfg2_shape_v16_batched"] = dict(M=2048, K=512, V=16, sparsity=0.9, N=256, batch=batch, out_f32=True, std=0.02, seed=2)
     cases["cfg2_shape_v16_batched_fp16_out"] = dict(M=2048, K=512, V=16, sparsity=0.9, N=256, batch=batch, out_f32=False,
@@ -350,8 +354,9 @@ def run_cfg1(L, torch, synth, sspmm_amd, O, st, wu):
     mat_rows, K_max, s_rp, s_ci, _ = sspmm_amd.stack_csr([(c.M, c.K, c.row_ptr, c.col_ind, None) for c in many])
     d_rp, d_ci = torch.from_numpy(s_rp).cuda(), torch.from_numpy(s_ci).cuda()
     t_stack = time_launches(lambda: sspmm_amd.svc_batched(mat_rows, K_max, d_rp, d_ci, None, V), 20, 3)
+    lists96 = [O.csr_col_lists(c.M, c.row_ptr, c.col_ind) for c in many]
     t0 = time.perf_counter()
-    want96 = [O.rowmerge_python(c.M, V, O.csr_col_lists(c.M, c.row_ptr, c.col_ind)) for c in many]
+    want96 = [O.rowmerge_python(c.M, V, l) for c, l in zip(many, lists96)]
     py96 = (time.perf_counter() - t0) * 1e3
     got96 = sspmm_amd.svc_batched(mat_rows, K_max, d_rp, d_ci, None, V).to_host()
     res["svc_stack_of_96_such_matrices"] = {
@@ -644,6 +649,55 @@ def run_cfg5_layer(L, torch, synth, st, wu):
             "projections": per}
 
 
+def run_attention_forward(torch, sparsity, bsz, st, wu, seq=4096, heads=4, embed=256, mlp=1024):
+    """The forward pass of the reference's end-to-end sparse attention model (end2end/sspmm_e2e/end_to_end.py:123-203:
+    4 blocks, fp16, V = 8 masks drawn at random per block) at the configurations its results are published for,
+    timed with a device synchronisation either side (the reference's loop has none, end_to_end.py:198-203), eager
+    and replayed from a HIP graph; the same model with dense unmasked attention in torch beside it (the reference's
+    "PyTorch" column)."""
+    from sspmm_amd.attention import SparseAttentionEncoder
+    torch.manual_seed(0)
+    model = SparseAttentionEncoder(257, embed, heads, sparsity, seq, mlp, mlp, vec_length=8, layers=4, seed=20).cuda().half().eval()
+    tokens = torch.randint(0, 257, (bsz, seq), device="cuda")
+
+    def dense_forward():
+        # the same weights with torch's dense attention (no mask): what the reference's dense model computes
+        out = model.encoder(tokens) * (embed ** 0.5)
+        out = out.transpose(0, 1) + model.pe[:seq].to(out.dtype)
+        d = embed // heads
+        for blk in model.blocks:
+            q, k, v = blk.in_proj(blk.layer_norm1(out)).chunk(3, dim=-1)
+            q, k, v = (t.contiguous().view(seq, bsz * heads, d).transpose(0, 1) for t in (q, k, v))
+            a = torch.nn.functional.scaled_dot_product_attention(q, k, v).transpose(0, 1).contiguous().view(seq, bsz, embed)
+            h1 = blk.out_proj(a) + out
+            out = blk.linear2(blk.linear1(blk.layer_norm2(h1))) + out
+        return model.linear(model.layer_norm(out))
+
+    def graphed(fn):
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            fn()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            fn()
+        return g.replay
+
+    with torch.no_grad():
+        y = model(tokens)
+        ms = time_launches(lambda: model(tokens), st, wu)
+        ms_g = time_launches(graphed(lambda: model(tokens)), st, wu)
+        dense_ms = time_launches(dense_forward, max(3, st // 4), 2)
+        blk = model.blocks[0]
+        x0 = torch.randn(seq, bsz, embed, device="cuda").half()
+        att_ms = time_launches(graphed(lambda: blk.attention(x0)), st, wu)
+    nvec = int(model.blocks[0].column_indices.numel())
+    return {"workload": "4 blocks, seq %d, %d heads / embed %d, mlp %d, mask sparsity %g (V=8, %d vectors per block), batch %d, fp16"
+                        % (seq, heads, embed, mlp, sparsity, nvec, bsz),
+            "ms": ms, "ms_in_a_graph": ms_g, "dense_unmasked_torch_ms": dense_ms, "speedup_vs_dense_unmasked_torch": dense_ms / ms_g,
+            "attention_of_one_block_ms_in_a_graph": att_ms, "output_is_finite": bool(torch.isfinite(y).all())}
+
+
 def run_reorder(L, torch, synth, sspmm_amd):
     """Row reordering ahead of the SVC: 16384 rows that are noisy copies of 256 prototype rows, shuffled."""
     rc_csr = synth.clustered_csr(16384, 16384, 256, 128, seed=6, keep=0.9, extras=1)
@@ -682,7 +736,8 @@ def run_reorder(L, torch, synth, sspmm_amd):
 
 
 ATTENTION = "sparse_attention_seq4096_d64_v8_s0.9_heads48"
-GROUPS = ["cfg1_rowmerge_then_spmm_512x512", "cfg4", "svc_batched_dlmc_shapes", "cfg5_encoder_layer_v16_s0.9_tokens4096", ATTENTION,
+ATTENTION_FORWARD = {"sparse_attention_forward_seq4096_h4_e256_s%g_b%d_l4" % (s, b): (s, b) for s in (0.9, 0.95) for b in (2, 8)}
+GROUPS = ["cfg1_rowmerge_then_spmm_512x512", "cfg4", "svc_batched_dlmc_shapes", *ATTENTION_FORWARD, "cfg5_encoder_layer_v16_s0.9_tokens4096", ATTENTION,
           "reorder_clustered_16384_v8", "headline_batched_cold"]
 
 
@@ -731,6 +786,8 @@ def run_extra(name, env):
         return {name: run_cfg1(L, torch, synth, sspmm_amd, O, st, wu)}
     if name == "cfg4":
         return run_cfg4(L, torch, synth, sspmm_amd, O, st, wu)
+    if name in ATTENTION_FORWARD:
+        return {name: run_attention_forward(torch, *ATTENTION_FORWARD[name], st=min(st, 50), wu=min(wu, 10))}
     if name == "svc_batched_dlmc_shapes":
         return {name: run_svc_batched(L, torch, synth, sspmm_amd, O)}
     if name == "cfg5_encoder_layer_v16_s0.9_tokens4096":
@@ -969,7 +1026,6 @@ def short_extra(extra):
         "headline_cold_hbm_frac": ("headline_batched_cold", "hbm_frac"),
         "cfg3_1024x2304_s0.8_n3136_hbm_frac": ("cfg3_1024x2304_v16_s0.8_n3136", "hbm_frac"),
         "cfg3_1024x2304_s0.8_n3136_ms": ("cfg3_1024x2304_v16_s0.8_n3136", "ms"),
-        "cfg3_2048x1024_s0.95_n3136_hbm_frac": ("cfg3_2048x1024_v16_s0.95_n3136", "hbm_frac"),
         "cfg5_ffn1_hbm_frac": ("cfg5_ffn1_3072x768_v16_s0.9_n4096", "hbm_frac"),
         "cfg5_ffn2_hbm_frac": ("cfg5_ffn2_768x3072_v16_s0.9_n4096", "hbm_frac"),
         "cfg4_spmm_with_plan_hbm_frac": ("cfg4_spmm_on_svc_output_with_plan", "hbm_frac"),
@@ -978,7 +1034,7 @@ def short_extra(extra):
         "svc_batched_dlmc_shapes_speedup_vs_python": ("svc_batched_dlmc_shapes", "speedup_vs_python"),
         "cfg1_svc_stack_of_96_speedup_vs_python": ("cfg1_rowmerge_then_spmm_512x512", "svc_stack_of_96_such_matrices", "speedup_vs_python"),
         "cfg5_layer_speedup_vs_dense_in_a_graph": ("cfg5_encoder_layer_v16_s0.9_tokens4096", "speedup_vs_dense_layer_in_a_graph"),
-        "sparse_attention_forward_seq4096_ms": ("sparse_attention_forward_seq4096_h4_e256_s0.9_b2_l4", "ms"),
+        "sparse_attention_forward_s0.9_b2_ms": ("sparse_attention_forward_seq4096_h4_e256_s0.9_b2_l4", "ms_in_a_graph"),
     }
     out = {}
     for name, keys in picks.items():

@@ -84,3 +84,97 @@ def sparse_attention(row_indices, row_offsets, column_indices, q, k, v, scaling,
     w = bcsr_softmax(row_indices, row_offsets, w, scaling, vec_length, w.size(0))
     _check_inputs(row_indices, row_offsets, column_indices, w, v, vec_length)
     return bspmm(row_indices, row_offsets, column_indices, w, v, vec_length)
+
+
+def static_random_mask(m_vec, n, sparsity, seed=0):
+    """A vector-sparse attention mask as the reference's end-to-end model draws it (verify/static_mask.py:7-27:
+    scipy.sparse.random of m_vec x n with density 1 - sparsity, i.e. round(density * m_vec * n) positions drawn uniformly
+    without replacement, CSR with ascending columns; row_indices = vector-rows by ascending length).  Seeded numpy
+    in place of scipy's global state.  Returns (column_indices, row_offsets, row_indices) as int32 numpy arrays."""
+    import numpy as np
+    rng = np.random.default_rng(seed)
+    k = int(round((1.0 - sparsity) * m_vec * n))
+    flat = np.sort(rng.choice(m_vec * n, size=k, replace=False))
+    rows, cols = flat // n, flat % n
+    row_offsets = np.concatenate([[0], np.cumsum(np.bincount(rows, minlength=m_vec))]).astype(np.int32)
+    row_indices = np.argsort(np.diff(row_offsets), kind="stable").astype(np.int32)
+    return cols.astype(np.int32), row_offsets, row_indices
+
+
+class SparseAttentionBlock(torch.nn.Module):
+    """One block of the reference's end-to-end model (SparseTransformerBlock, end2end/sspmm_e2e/end_to_end.py:45-78):
+    LayerNorm -> multi-head attention on a static vector-sparse mask (bsddmm -> bcsr_softmax -> bspmm,
+    spattention.py:151-186) -> + x -> LayerNorm -> linear1 -> linear2 -> + x, on [seq, batch, embed] activations.
+    The block's arithmetic follows the reference as written, including the second residual adding the block's input
+    and the two linear layers without an activation between them."""
+
+    def __init__(self, embed_dim, mlp_dim, num_heads, column_indices, row_offsets, row_indices, vec_length=8):
+        super().__init__()
+        if embed_dim % num_heads:
+            raise ValueError("embed_dim must be a multiple of num_heads")
+        self.embed_dim, self.num_heads, self.vec_length = embed_dim, num_heads, vec_length
+        self.in_proj = torch.nn.Linear(embed_dim, 3 * embed_dim)
+        self.out_proj = torch.nn.Linear(embed_dim, embed_dim)
+        self.layer_norm1 = torch.nn.LayerNorm(embed_dim)
+        self.layer_norm2 = torch.nn.LayerNorm(embed_dim)
+        self.linear1 = torch.nn.Linear(embed_dim, mlp_dim)
+        self.linear2 = torch.nn.Linear(mlp_dim, embed_dim)
+        self.register_buffer("column_indices", column_indices)
+        self.register_buffer("row_offsets", row_offsets)
+        self.register_buffer("row_indices", row_indices)
+
+    def attention(self, x, dense_mask=None):
+        """x [seq, batch, embed] -> [seq, batch, embed].  With dense_mask (bool [seq, seq]) the three sparse steps
+        are replaced by dense masked attention in fp32 (for checks)."""
+        seq, bsz, E = x.shape
+        h, d = self.num_heads, E // self.num_heads
+        q, k, v = self.in_proj(x).chunk(3, dim=-1)
+        # [seq, batch * heads, d] -> [batch * heads, seq, d] (spattention.py:151-157)
+        q, k, v = (t.contiguous().view(seq, bsz * h, d).transpose(0, 1).contiguous() for t in (q, k, v))
+        scaling = float(d) ** -0.5
+        if dense_mask is None:
+            out = sparse_attention(self.row_indices, self.row_offsets, self.column_indices, q, k, v, scaling, self.vec_length)
+        else:
+            s = (q.float() @ k.float().transpose(1, 2)) * scaling
+            s = s.masked_fill(~dense_mask, float("-inf"))
+            out = (torch.softmax(s, dim=-1) @ v.float()).to(x.dtype)
+        out = out.transpose(0, 1).contiguous().view(seq, bsz, E)
+        return self.out_proj(out)
+
+    def forward(self, x, dense_mask=None):
+        out = self.attention(self.layer_norm1(x), dense_mask) + x
+        out = self.linear2(self.linear1(self.layer_norm2(out)))
+        return out + x
+
+
+class SparseAttentionEncoder(torch.nn.Module):
+    """The reference's end-to-end model (SparseTransformerEncoder, end_to_end.py:123-153): embedding * sqrt(embed),
+    sinusoidal positions, four SparseAttentionBlocks each with a mask of its own, LayerNorm, linear head."""
+
+    def __init__(self, vocab_size, embed_dim, num_heads, sparsity, seq_len, mlp_dim, num_class, vec_length=8, layers=4, seed=0):
+        super().__init__()
+        import math
+        self.embed_dim = embed_dim
+        self.encoder = torch.nn.Embedding(vocab_size, embed_dim)
+        pe = torch.zeros(seq_len, embed_dim)
+        pos = torch.arange(0, seq_len, dtype=torch.float).unsqueeze(1)
+        div = torch.exp(torch.arange(0, embed_dim, 2).float() * (-math.log(10000.0) / embed_dim))
+        pe[:, 0::2] = torch.sin(pos * div)
+        pe[:, 1::2] = torch.cos(pos * div)
+        self.register_buffer("pe", pe.unsqueeze(1))
+        blocks = []
+        for i in range(layers):
+            cols, offs, rows = static_random_mask(seq_len // vec_length, seq_len, sparsity, seed=seed + i)
+            blocks.append(SparseAttentionBlock(embed_dim, mlp_dim, num_heads, torch.from_numpy(cols), torch.from_numpy(offs),
+                                               torch.from_numpy(rows), vec_length))
+        self.blocks = torch.nn.ModuleList(blocks)
+        self.layer_norm = torch.nn.LayerNorm(embed_dim)
+        self.linear = torch.nn.Linear(embed_dim, num_class)
+
+    def forward(self, tokens, dense_masks=None):
+        """tokens: int [batch, seq] -> [seq, batch, num_class]."""
+        out = self.encoder(tokens) * (self.embed_dim ** 0.5)
+        out = out.transpose(0, 1) + self.pe[:tokens.size(1)].to(out.dtype)
+        for i, blk in enumerate(self.blocks):
+            out = blk(out, None if dense_masks is None else dense_masks[i])
+        return self.linear(self.layer_norm(out))

@@ -127,3 +127,30 @@ def test_argument_errors(built_library):
         sspmm_amd.csr_softmax(None, off, torch.zeros(0, device="cuda"), 1.0, 8)
     with pytest.raises(RuntimeError):  # F must be a multiple of 8
         sspmm_amd.sddmm(None, off, col, torch.zeros(16, 12, device="cuda").half(), torch.zeros(8, 12, device="cuda").half(), 8)
+
+
+def test_sparse_attention_encoder_matches_dense_masked_attention(built_library):
+    """The end-to-end model of the reference (four blocks, each with its own static mask) against the same model
+    whose attention is dense fp32 arithmetic with the mask applied as -inf (the recipe of the reference's own checks,
+    verify/softmax.py:36-38, verify/spmm.py:36-41)."""
+    from sspmm_amd.attention import SparseAttentionEncoder
+    torch.manual_seed(3)
+    seq, V = 512, 8
+    model = SparseAttentionEncoder(vocab_size=257, embed_dim=128, num_heads=2, sparsity=0.9, seq_len=seq, mlp_dim=256,
+                                   num_class=16, vec_length=V, layers=4, seed=11).cuda().half().eval()
+    tokens = torch.randint(0, 257, (2, seq), device="cuda", generator=torch.Generator("cuda").manual_seed(4))
+    masks = []
+    for blk in model.blocks:
+        off, col = blk.row_offsets.cpu().numpy(), blk.column_indices.cpu().numpy()
+        assert off[-1] == col.size == round(0.1 * (seq // V) * seq)
+        dense = np.zeros((seq, seq), bool)
+        for i in range(seq // V):
+            dense[i * V:(i + 1) * V, col[off[i]:off[i + 1]]] = True
+        assert np.array_equal(np.sort(np.diff(off)[blk.row_indices.cpu().numpy()]), np.diff(off)[blk.row_indices.cpu().numpy()])
+        masks.append(torch.from_numpy(dense).cuda())
+    with torch.no_grad():
+        got = model(tokens)
+        want = model(tokens, dense_masks=masks)
+    assert got.shape == (seq, 2, 16) and got.dtype == torch.float16
+    assert torch.isfinite(got).all()
+    assert max_rel_err(got.float().cpu().numpy(), want.float().cpu().numpy()) <= 1e-2

@@ -61,7 +61,8 @@ hipError_t plan_create(int m_vec, int V, int K, const int32_t *row_offsets, int 
   const size_t n_items = (size_t)pl->header[kHdrItems], n_split = (size_t)pl->header[kHdrSplitRows];
   const size_t n_slots = (size_t)pl->header[kHdrSlots];
   const size_t units = (size_t)(pl->tiles_max > 0 ? pl->tiles_max : 1) * (size_t)(max_batch > 0 ? max_batch : 1);
-  const size_t off_items = 256;
+  const size_t off_bundles = 256;
+  const size_t off_items = off_bundles + align256((n_items - n_slots + 2) * sizeof(int32_t));
   const size_t off_counters = off_items + align256(n_items * sizeof(ScheduleItem));
   pl->counters = n_split * units;
   const size_t off_partials = off_counters + align256(pl->counters * 4);
@@ -72,11 +73,15 @@ hipError_t plan_create(int m_vec, int V, int K, const int32_t *row_offsets, int 
   }
   unsigned char *base = static_cast<unsigned char *>(pl->memory);
   pl->view.header = reinterpret_cast<int32_t *>(base);
+  pl->view.bundles = reinterpret_cast<int32_t *>(base + off_bundles);
   pl->view.items = reinterpret_cast<ScheduleItem *>(base + off_items);
   pl->view.counters = reinterpret_cast<int32_t *>(base + off_counters);
   pl->view.partials = base + off_partials;
   e = hipMemcpyAsync(pl->view.header, pl->header, sizeof(pl->header), hipMemcpyHostToDevice, stream);
-  if (e == hipSuccess) e = launch_schedule_fill(m_vec, row_offsets, pl->view, (int64_t)n_items, (int64_t)pl->counters, 0, stream);
+  if (e == hipSuccess)
+    e = launch_schedule_fill(m_vec, row_offsets, pl->view, (int64_t)n_items, (int64_t)pl->counters, 0, kScheduleBundleSteps, stream);
+  // (the fill leaves the number of bundles in the header)
+  if (e == hipSuccess) e = hipMemcpyAsync(pl->header, pl->view.header, sizeof(pl->header), hipMemcpyDeviceToHost, stream);
   if (e == hipSuccess) e = hipStreamSynchronize(stream);  // products with the plan may come on any stream
   if (e != hipSuccess) {
     (void)hipFree(pl->memory);
@@ -103,7 +108,9 @@ hipError_t launch_spmm_planned(const Plan &pl, const SpmmArgs &a, bool out_f16, 
   const bool skewed = pl.header[kHdrSplitRows] > 0;
   const bool epilogue = a.bias != nullptr || a.act != 0;  // (the load-balanced kernel does not apply one)
   if (can_balance && !epilogue && (forced == 7 || (forced == 0 && skewed)))
-    return launch_spmm_balanced(a, pl.V, out_f16, pl.view, pl.header[kHdrItems], false, stream);
+    return launch_spmm_balanced(a, pl.V, out_f16, pl.view,
+                                pl.header[kHdrBundles] > 0 ? pl.header[kHdrSlots] + pl.header[kHdrBundles] : pl.header[kHdrItems],
+                                false, stream, pl.header[kHdrBundles] > 0 ? pl.header[kHdrSlots] : -1);
   SpmmArgs b = a;
   // (at least 1: an empty pattern is as sparse as it gets, and 0 would say the density is unknown)
   b.mean_row_vectors = pl.m_vec > 0 ? (int)((int64_t)pl.header[kHdrNvec] / pl.m_vec) + 1 : 0;
@@ -165,6 +172,7 @@ hipError_t launch_spmm_static(const SpmmArgs &a, int V, bool out_f16, hipStream_
   if (e != hipSuccess) return e;
   ScheduleView view;
   view.header = reinterpret_cast<int32_t *>(base);
+  view.bundles = nullptr;
   view.items = reinterpret_cast<ScheduleItem *>(base + kStaticItemsOff);
   view.counters = reinterpret_cast<int32_t *>(base + kStaticCountersOff);
   view.partials = base + kStaticPartialsOff;

@@ -25,6 +25,7 @@ enum {
   kHdrNvec = 4,        // stored vectors of the pattern
   kHdrMaxSteps = 5,    // steps of the longest vector-row
   kHdrTotalSteps = 6,  // steps of all vector-rows (an empty row counts one: its zeros are written)
+  kHdrBundles = 7,     // bundles the rows that were left whole are filed in (0: no bundle table)
   kHdrWords = 8
 };
 
@@ -38,13 +39,23 @@ struct ScheduleItem {
 
 static constexpr int kScheduleMinBudget = 8;      // steps: shorter panels are all overhead
 static constexpr int kScheduleTargetItems = 512;   // panels of cut rows wanted at most (before the memory cap)
+// Steps a bundle of short rows aims at.  Measured on a 16384 x 16384 matrix of power-law rows (2048 vector-rows, 1930
+// of them whole, 2.1 steps each on average): 5 and 6 steps 18.2-18.9 us, 8 steps 17.2, 10 17.5, 12 18.3, 16 17.2-20.5,
+// against 18.0 with one wave per row.
+static constexpr int kScheduleBundleSteps = 8;
 
 // A partial tile: the accumulators of one wave (V rows x 64 columns, fp32) as they lie in its registers,
 // 4 x (lanes that hold rows) x 16 bytes.
 static constexpr size_t partial_tile_bytes(int V) { return V == 8 ? 4u * 32u * 16u : 4u * 64u * 16u; }
 
+// Bundles: a wave that starts for one short row spends most of its life waiting for two dependent round trips to
+// memory (column indices, then the rows of B they name) with nothing else in flight, and a pattern of skewed rows is
+// mostly short rows.  The rows that stay whole are therefore filed, in row order, in bundles of about `bundle_steps`
+// steps; one wave takes a bundle and runs its rows as one stream of steps, the loads of a row in flight while the
+// row before it is contracted.  bundles[b] = first item of bundle b, bundles[header[kHdrBundles]] = item count.
 struct ScheduleView {
   int32_t *header;           // kHdrWords ints
+  int32_t *bundles;          // header[kHdrBundles] + 1 ints, or null (every row that stays whole is a unit of its own)
   ScheduleItem *items;
   int32_t *counters;         // panels that have delivered, per (batch element, column tile, cut row); zero between launches
   unsigned char *partials;   // partial tiles, per (batch element, column tile, slot)
@@ -58,8 +69,11 @@ hipError_t launch_schedule_measure(int m_vec, const int32_t *row_offsets, int bu
 // Writes the items for the budget the header holds (at most item_cap of them: the caller sizes from the header,
 // or passes bounds that hold for every pattern), and clears `counters_to_clear` counters, or when that is
 // negative the counters_per_cut_row counters of every cut row the header reports.  One workgroup.
+// With view.bundles set, also files the rows that stay whole in bundles of about bundle_steps steps (at most 64
+// rows each) and leaves their number in header[kHdrBundles].
 hipError_t launch_schedule_fill(int m_vec, const int32_t *row_offsets, const ScheduleView &view, int64_t item_cap,
-                                int64_t counters_to_clear, int64_t counters_per_cut_row, hipStream_t stream);
+                                int64_t counters_to_clear, int64_t counters_per_cut_row, int bundle_steps,
+                                hipStream_t stream);
 
 // launch_schedule_measure (budget chosen from the pattern) and launch_schedule_fill (clearing the counters of the
 // cut rows) as one launch; up to 4096 vector-rows by a kernel of its own that writes the same schedule sooner.

@@ -118,11 +118,19 @@ __device__ __forceinline__ unsigned long long block_exclusive_scan64(unsigned lo
 __device__ __forceinline__ void schedule_fill(int m_vec, const int32_t *__restrict__ row_offsets, const int32_t *header,
                                               ScheduleItem *__restrict__ items, long long item_cap,
                                               int32_t *__restrict__ counters, long long counters_to_clear,
-                                              long long counters_per_cut_row, unsigned long long *scratch) {
+                                              long long counters_per_cut_row, unsigned long long *scratch,
+                                              int32_t *__restrict__ bundles = nullptr, int bundle_steps = 0,
+                                              int32_t *header_out = nullptr) {
   if (counters_to_clear < 0) counters_to_clear = (long long)header[kHdrSplitRows] * counters_per_cut_row;
   for (long long i = threadIdx.x; i < counters_to_clear; i += kBuildThreads) counters[i] = 0;
   const int budget = header[kHdrBudget];
-  const long long n_slots = header[kHdrSlots];
+  const long long n_slots = header[kHdrSlots], n_items = header[kHdrItems];
+  const bool bundling = bundles != nullptr && bundle_steps > 0;
+  if (bundling && threadIdx.x == 0) {  // (what a pattern without whole rows leaves: no bundle)
+    bundles[0] = (int)n_slots;
+    header_out[kHdrBundles] = 0;
+  }
+  unsigned long long carry_enders = 0;
   // Two scans per 1024 rows: the panels of cut rows together with the number of cut rows (panels in bits 0-39 of
   // the running sum, cut rows from bit 40 on), and the rows that stay whole.
   unsigned long long carry_slots_split = 0, carry_whole = 0;
@@ -138,7 +146,24 @@ __device__ __forceinline__ void schedule_fill(int m_vec, const int32_t *__restri
     unsigned long long t1, t2;
     const unsigned long long ex1 =
         block_exclusive_scan64(r < m_vec && pcs ? (unsigned long long)pcs + (1ull << 40) : 0ull, &t1, scratch);
-    const unsigned long long ex2 = block_exclusive_scan64(r < m_vec && !pcs ? 1ull : 0ull, &t2, scratch);
+    // (rows that stay whole: their number in the low half, their steps in the high half)
+    const unsigned long long ex2 =
+        block_exclusive_scan64(r < m_vec && !pcs ? 1ull + ((unsigned long long)steps << 32) : 0ull, &t2, scratch);
+    // Bundles of the rows that stay whole: a row whose steps reach or cross a multiple of bundle_steps in the
+    // running sum of steps, or that is the 64th of its bundle (the rows of a bundle are held one per lane), ends
+    // its bundle; so does a row of more than half a bundle's steps and the row in front of one (such a row is a
+    // bundle of its own: a bundle then never holds more than a bundle and a half).  The number of such rows before
+    // a row is the row's bundle.
+    unsigned long long ex3 = 0, t3 = 0;
+    bool ender = false;
+    if (bundling) {  // (uniform)
+      const unsigned long long before = (carry_whole + ex2) >> 32, count_before = (carry_whole + ex2) & 0xffffffffull;
+      const int next_steps = r + 1 < m_vec ? steps_of(row_offsets[r + 2] - end) : 0;
+      ender = r < m_vec && !pcs &&
+              ((before + (unsigned long long)steps) / (unsigned)bundle_steps > before / (unsigned)bundle_steps ||
+               (count_before & 63ull) == 63ull || 2 * steps > bundle_steps || 2 * next_steps > bundle_steps);
+      ex3 = block_exclusive_scan64(ender ? 1ull : 0ull, &t3, scratch);
+    }
     if (r < m_vec) {
       if (pcs) {
         const unsigned long long at = carry_slots_split + ex1;
@@ -159,7 +184,15 @@ __device__ __forceinline__ void schedule_fill(int m_vec, const int32_t *__restri
           items[first_slot + pc] = it;
         }
       } else {
-        const long long at = n_slots + (long long)(carry_whole + ex2);
+        const long long at = n_slots + (long long)((carry_whole + ex2) & 0xffffffffull);
+        if (bundling && at < item_cap) {
+          const long long b = (long long)(carry_enders + ex3);
+          if (ender) bundles[b + 1] = (int)(at + 1);
+          if (at == n_items - 1) {  // the last row that stays whole closes the table
+            bundles[b + 1] = (int)n_items;
+            header_out[kHdrBundles] = (int)(b + 1);
+          }
+        }
         if (at < item_cap) {
           ScheduleItem it;
           it.row = r;
@@ -176,6 +209,7 @@ __device__ __forceinline__ void schedule_fill(int m_vec, const int32_t *__restri
     }
     carry_slots_split += t1;
     carry_whole += t2;
+    carry_enders += t3;
   }
 }
 
@@ -183,9 +217,12 @@ __global__ __launch_bounds__(kBuildThreads) void schedule_fill_kernel(int m_vec,
                                                                       const int32_t *__restrict__ header,
                                                                       ScheduleItem *__restrict__ items, long long item_cap,
                                                                       int32_t *__restrict__ counters, long long counters_to_clear,
-                                                                      long long counters_per_cut_row) {
+                                                                      long long counters_per_cut_row,
+                                                                      int32_t *__restrict__ bundles, int bundle_steps,
+                                                                      int32_t *__restrict__ header_out) {
   __shared__ unsigned long long scratch[kBuildThreads / 64];
-  schedule_fill(m_vec, row_offsets, header, items, item_cap, counters, counters_to_clear, counters_per_cut_row, scratch);
+  schedule_fill(m_vec, row_offsets, header, items, item_cap, counters, counters_to_clear, counters_per_cut_row, scratch,
+                bundles, bundle_steps, header_out);
 }
 
 // Both steps in one launch (the header passes through global memory inside the one workgroup).
@@ -416,10 +453,11 @@ hipError_t launch_schedule_measure(int m_vec, const int32_t *row_offsets, int bu
 }
 
 hipError_t launch_schedule_fill(int m_vec, const int32_t *row_offsets, const ScheduleView &view, int64_t item_cap,
-                                int64_t counters_to_clear, int64_t counters_per_cut_row, hipStream_t stream) {
+                                int64_t counters_to_clear, int64_t counters_per_cut_row, int bundle_steps,
+                                hipStream_t stream) {
   hipLaunchKernelGGL(schedule_fill_kernel, dim3(1), dim3(kBuildThreads), 0, stream, m_vec, row_offsets, view.header,
                      view.items, (long long)item_cap, view.counters, (long long)counters_to_clear,
-                     (long long)counters_per_cut_row);
+                     (long long)counters_per_cut_row, view.bundles, bundle_steps, view.header);
   return hipGetLastError();
 }
 

@@ -47,8 +47,10 @@ int last_kernel();
 // Only where balanced_kernel_applies (the MFMA kernels' alignment and size conditions).
 struct ScheduleView;
 bool balanced_kernel_applies(const SpmmArgs &args, int V, bool out_f16);
+// bundle_base >= 0: the schedule files its whole rows in bundles, units 0 .. bundle_base - 1 are the panels of cut
+// rows (one item each), unit bundle_base + b is bundle b, and n_items counts units.
 hipError_t launch_spmm_balanced(const SpmmArgs &args, int V, bool out_f16, const ScheduleView &schedule, int n_items,
-                                bool device_count, hipStream_t stream);
+                                bool device_count, hipStream_t stream, int bundle_base = -1);
 int kernel_override();
 
 hipError_t launch_sorted_row_swizzle(int m_vec, const int32_t *row_offsets, int32_t *row_indices,

@@ -1292,6 +1292,122 @@ __device__ __forceinline__ void stage_accumulate(floatx4 (&acc)[4], const StageL
   }
 }
 
+// The same pipeline over a bundle of whole vector-rows (items first .. first + count - 1 of a schedule, count <= 64):
+// the steps of all the rows are one stream, so that the column indices of a row's first step and the rows of B they
+// name are in flight while the row before it is contracted, and a row's V x 64 tile of C is stored when its last
+// step has been.  A row of no vectors is one step of zeros.  Each row's sums are formed exactly as stage_accumulate
+// forms them (same steps, same order).
+template <int V, typename OutT>
+__device__ __forceinline__ void stage_stream(const StageLane<V> &x, const int32_t *col_idx, const uint16_t *vals,
+                                             __amdgpu_buffer_rsrc_t srd_b, uint32_t lane_n2, uint32_t lane_col_off, uint32_t b_bytes,
+                                             const void *first_item, int count, int lane, const SlabStore<V, OutT, 4> &out,
+                                             __amdgpu_buffer_rsrc_t srd_c, uint32_t c_vrow_bytes) {
+  // the bundle's items, one per lane (row, first vector, end): a uniform index reads one back without memory
+  const uintx4 mine = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(
+                                                     make_srd(first_item, (uint32_t)count * 32u), (uint32_t)lane * 32u, 0, 0));
+  struct Step {  // (uniform)
+    int row, kc, end;
+    bool valid;
+  };
+  int j = 0;
+  Step cur;
+  cur.row = __builtin_amdgcn_readlane((int)mine[0], 0);
+  cur.kc = __builtin_amdgcn_readlane((int)mine[1], 0);
+  cur.end = __builtin_amdgcn_readlane((int)mine[2], 0);
+  cur.valid = true;
+  const auto next = [&]() {
+    const Step d = cur;
+    if (cur.valid) {
+      cur.kc += 32;
+      if (cur.kc >= cur.end) {
+        ++j;
+        cur.valid = j < count;
+        const int jj = cur.valid ? j : 0;
+        cur.row = __builtin_amdgcn_readlane((int)mine[0], jj);
+        cur.kc = __builtin_amdgcn_readlane((int)mine[1], jj);
+        cur.end = __builtin_amdgcn_readlane((int)mine[2], jj);
+      }
+    }
+    return d;
+  };
+  // (a step past the bundle's end has no vectors to its name: descriptors of zero bytes, every load reads zeros)
+  const auto load_head = [&](StageHead<V> &h, const Step &d) {
+    const uint32_t recs = d.valid ? (uint32_t)d.end : 0u;
+    h.kc = d.kc;
+    h.cols = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(make_srd(col_idx, recs * 4u), (d.kc + 4 * x.j) * 4, 0, 0));
+    h.vraw = SlabVals<V>::load(make_srd(vals, recs * (V * 2u)), (uint32_t)d.kc * (V * 2u) + x.vals_lane_off);
+  };
+  const auto load_body = [&](StageBody<V> &c, const StageHead<V> &h, const Step &d) {
+    uint32_t off[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) off[i] = __umul24(h.cols[i], lane_n2) + lane_col_off;
+    if (h.kc + 32 > d.end) {  // wave-uniform: only the last step of a vector-row can be partial
+#pragma unroll
+      for (int i = 0; i < 4; ++i) off[i] = (h.kc + 4 * x.j + i < d.end) ? off[i] : b_bytes;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      c.piece[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_b, off[i], 0, 0));
+    c.vraw = h.vraw;
+  };
+  floatx4 acc[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
+  const auto contract = [&](const StageBody<V> &c, const Step &d) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<uintx4 *>(x.stage_dst + i * kStagePitch) = c.piece[i];
+    *reinterpret_cast<typename SlabVals<V>::type *>(x.tile_dst) = c.vraw;
+    Half8Bits a;
+    {
+      const uintx2 lo = lds_read_tr(x.val_tile, x.a_off);
+      const uintx2 hi = lds_read_tr(x.val_tile, x.a_off + 4u * (V * 2u));
+      a.u[0] = lo[0]; a.u[1] = lo[1]; a.u[2] = hi[0]; a.u[3] = hi[1];
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      Half8Bits b;
+      const uintx2 lo = lds_read_tr_abs(x.b_rd + 32u * q);
+      const uintx2 hi = lds_read_tr_abs(x.b_rd + 4u * kStagePitch + 32u * q);
+      b.u[0] = lo[0]; b.u[1] = lo[1]; b.u[2] = hi[0]; b.u[3] = hi[1];
+      acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(b.h, a.h, acc[q], 0, 0, 0);
+    }
+    if (d.kc + 32 >= d.end) {  // the row's last step: its tile of C, and the next row starts from zero
+      out.store(acc, srd_c, (uint32_t)d.row * c_vrow_bytes);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) acc[q] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+  };
+  // Heads run two steps ahead of the arithmetic, bodies one; loads are only issued on the paths that use them, so
+  // that the waits in front of every use count exactly the loads behind it.
+  StageHead<V> h0, h1;
+  StageBody<V> c0, c1;
+  Step d0 = next();
+  load_head(h0, d0);
+  Step d1 = next();
+  load_head(h1, d1);
+  load_body(c0, h0, d0);
+  for (;;) {
+    if (!d1.valid) {
+      contract(c0, d0);
+      break;
+    }
+    const Step d2 = next();
+    load_head(h0, d2);
+    load_body(c1, h1, d1);
+    contract(c0, d0);
+    if (!d2.valid) {
+      contract(c1, d1);
+      break;
+    }
+    const Step d3 = next();
+    load_head(h1, d3);
+    load_body(c0, h0, d2);
+    contract(c1, d1);
+    d0 = d2;
+    d1 = d3;
+  }
+}
+
 template <int V, typename OutT>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(V == 8 ? 5 : 4, V == 8 ? 5 : 4))) void spmm_stage_kernel(const SpmmArgs p) {
   __shared__ __align__(16) unsigned char stage[32 * kStagePitch];
@@ -1371,8 +1487,10 @@ struct BalancedArgs {
   const ScheduleItem *items;
   int32_t *counters;
   unsigned char *partials;
-  int n_items;            // items the grid covers: the schedule's count, or an upper bound of it
+  int n_items;            // units the grid covers: the schedule's count, or an upper bound of it
   uint32_t tiles_padded;
+  const int32_t *bundles; // first item of every bundle of whole rows, or null: every item is a unit
+  int bundle_base;        // with bundles: units below this are single items (the panels of cut rows)
 };
 
 // Partial tiles travel between workgroups that may sit on different XCDs, each with an L2 of its own.  They are
@@ -1427,9 +1545,25 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(4, 4))) void
   {
     const uint32_t id = blockIdx.x;
     const uint32_t batch = id / per_batch, rem = id % per_batch;
-    const uint32_t tile = rem % s.tiles_padded, item = rem / s.tiles_padded;
+    const uint32_t tile = rem % s.tiles_padded, unit = rem / s.tiles_padded;
     if (tile >= p.n_tiles) return;
-    if (DEVICE_COUNT && item >= (uint32_t)s.header[kHdrItems]) return;
+    if (DEVICE_COUNT && unit >= (uint32_t)s.header[kHdrItems]) return;
+    uint32_t item = unit;
+    if (!DEVICE_COUNT && s.bundles != nullptr && unit >= (uint32_t)s.bundle_base) {
+      // a bundle of rows that stay whole: one stream of steps
+      const int32_t *bp = s.bundles + (unit - (uint32_t)s.bundle_base);
+      const int first = __builtin_amdgcn_readfirstlane(bp[0]), last = __builtin_amdgcn_readfirstlane(bp[1]);
+      const int ncol = (int)tile * 64 + 8 * x.pc;
+      const bool col_ok = ncol < p.N;
+      SlabStore<V, OutT, 4> out;
+      out.init(lane, (int)tile * 64, p.N);
+      stage_stream<V, OutT>(x, p.col_idx, p.values + (int64_t)batch * p.stride_values,
+                            make_srd(p.B + (int64_t)batch * p.stride_B, b_bytes), col_ok ? (uint32_t)p.N * 2u : 0u,
+                            col_ok ? (uint32_t)ncol * 2u : b_bytes, b_bytes, s.items + first, last - first, lane, out,
+                            make_srd(reinterpret_cast<OutT *>(p.C) + (int64_t)batch * p.stride_C, (uint32_t)p.m_vec * c_vrow_bytes),
+                            c_vrow_bytes);
+      return;
+    }
     const ScheduleItem *ip = s.items + item;
     // (the item is the same for the whole wave: scalar registers)
     const int row = __builtin_amdgcn_readfirstlane(ip->row), kbeg = __builtin_amdgcn_readfirstlane(ip->kbeg),
@@ -1694,7 +1828,7 @@ static void launch_balanced_v(const SpmmArgs &p, const BalancedArgs &s, uint32_t
 }
 
 hipError_t launch_spmm_balanced(const SpmmArgs &a, int V, bool out_f16, const ScheduleView &sv, int n_items,
-                                bool device_count, hipStream_t stream) {
+                                bool device_count, hipStream_t stream, int bundle_base) {
   SpmmArgs p = a;
   p.n_tiles = (uint32_t)((a.N + 63) / 64);
   BalancedArgs s;
@@ -1704,6 +1838,8 @@ hipError_t launch_spmm_balanced(const SpmmArgs &a, int V, bool out_f16, const Sc
   s.partials = sv.partials;
   s.n_items = n_items;
   s.tiles_padded = padded_tiles(p.n_tiles);
+  s.bundles = bundle_base >= 0 ? sv.bundles : nullptr;
+  s.bundle_base = bundle_base;
   const uint64_t units = (uint64_t)n_items * s.tiles_padded * (uint64_t)a.batch;
   if (units >= (1ull << 31)) return hipErrorInvalidValue;
   if (units == 0) return hipSuccess;

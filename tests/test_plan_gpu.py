@@ -311,3 +311,41 @@ def test_many_panels_give_the_same_bits_twenty_times_in_a_row(oracle, built_libr
     want = oracle.spmm(vs.m_vec, V, N, K, vs.row_offsets, vs.col_idx, vals[1], B[1], threads=8)
     assert max_rel_err(first[1].cpu().numpy(), want) <= TIGHT_F32
     plan.destroy()
+
+
+@pytest.mark.parametrize("V", [8, 16])
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16])
+def test_short_rows_run_in_bundles_with_the_same_bits(oracle, built_library, V, out_dtype):
+    """The rows that stay whole are filed in bundles (a wave runs the rows of a bundle as one stream of steps): runs of
+    more than 64 one-step rows (a bundle holds at most 64), empty rows at the start, in the middle and at the end of
+    bundles, rows of more than half a bundle's steps (bundles of their own), partial last steps, a partial last column
+    tile.  Every row that is not cut must equal the staged gather kernel's row bit for bit, and all of it the oracle."""
+    K, N = 4000, 200
+    rng = np.random.default_rng(31 + V)
+    lens = rng.integers(0, 34, 700)
+    lens[100:180] = rng.integers(1, 20, 80)          # eighty one-step rows in a row
+    lens[300:310] = 0
+    lens[rng.choice(700, 40, replace=False)] = rng.integers(130, 330, 40)   # five to eleven steps
+    lens[[5, 350, 699]] = [2500, 3100, 1800]         # cut
+    lens[[0, 698]] = 0
+    vs = ragged(len(lens), K, V, lens, seed=32 + V)
+    B = synth.dense_rhs(K, N, seed=33)
+    plan = Plan(dev(vs.row_offsets), V, K, max_N=N)
+    assert plan.info().cut_rows >= 3
+    L = _lib.lib()
+    got = run(vs, B, out_dtype, plan)
+    assert L.sspmm_last_kernel() == BALANCED
+    L.sspmm_select_kernel(6)
+    try:
+        base = run(vs, B, out_dtype)
+        assert L.sspmm_last_kernel() == 6
+    finally:
+        L.sspmm_select_kernel(0)
+    cut = steps_of(lens) > plan.info().panel_steps
+    for i in np.flatnonzero(~cut):
+        assert np.array_equal(got[i * V:(i + 1) * V], base[i * V:(i + 1) * V]), i
+    want = oracle.spmm(vs.m_vec, V, N, K, vs.row_offsets, vs.col_idx, vs.values, B, threads=8)
+    assert max_rel_err(got, want) <= (TIGHT_F32 if out_dtype == torch.float32 else TIGHT_F16)
+    for _ in range(2):
+        assert np.array_equal(run(vs, B, out_dtype, plan), got)
+    plan.destroy()

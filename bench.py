@@ -226,7 +226,8 @@ def spmm_case(L, torch, synth, M, K, V, sparsity, N, batch, out_f32, std, seed, 
 
 
 def attention_block(torch, synth, sspmm_amd, st, wu):
-    """Times the three steps of the reference's sparse attention block; returns a dict of figures."""
+    """Times the three steps of the reference's sparse attention block, one by one and as the one launch that stands
+    for the chain; returns a dict of figures."""
     # the sparse attention block of the reference (bsddmm -> bcsr_softmax -> bspmm) on one mask shared by
     # 48 heads: 4096 tokens, head size 64, V=8, 90 % of the vectors masked out
     seqA, dA, VA, bA = 4096, 64, 8, 48
@@ -240,6 +241,10 @@ def attention_block(torch, synth, sspmm_amd, st, wu):
     t_soft = time_launches(lambda: sspmm_amd.bcsr_softmax(None, offA, wA, 0.125, VA, bA), st, wu)
     t_av = time_launches(lambda: sspmm_amd.bspmm(None, offA, colA, pA, vA, VA), st, wu)
     t_dense = time_launches(lambda: torch.nn.functional.scaled_dot_product_attention(qA, kA, vA), max(5, st // 10), 2)
+    t_one = time_launches(lambda: sspmm_amd.fused_sparse_attention(None, offA, colA, qA, kA, vA, 0.125, VA), st, wu)
+    chain = sspmm_amd.bspmm(None, offA, colA, pA, vA, VA).float()
+    one = sspmm_amd.fused_sparse_attention(None, offA, colA, qA, kA, vA, 0.125, VA).float()
+    by_one = bA * 4 * 2 * seqA * dA + 4 * nvA + 4 * (mk_a.m_vec + 1)   # q, k, v read and the output written, once each
     by_sddmm = bA * (2 * seqA * dA * 2 + 2 * nvA * VA) + 4 * nvA + 4 * (mk_a.m_vec + 1)
     by_soft = bA * 2 * 2 * nvA * VA + 4 * (mk_a.m_vec + 1)
     by_av = bA * (2 * nvA * VA + 2 * seqA * dA + 2 * seqA * dA) + 4 * nvA + 4 * (mk_a.m_vec + 1)
@@ -249,6 +254,11 @@ def attention_block(torch, synth, sspmm_amd, st, wu):
         "bcsr_softmax_alg_bytes": by_soft,
         "bspmm_ms": t_av, "bspmm_hbm_frac": by_av / t_av / 1e6 / HBM_PEAK_GBPS, "bspmm_alg_bytes": by_av,
         "block_ms": t_sddmm + t_soft + t_av, "dense_sdpa_ms": t_dense, "nvec": int(nvA),
+        "one_launch_ms": t_one, "one_launch_alg_bytes": by_one, "one_launch_hbm_frac": by_one / t_one / 1e6 / HBM_PEAK_GBPS,
+        # rows of k and of v fetched from the caches, 128 bytes per stored vector each: what bounds the launch
+        "one_launch_gathered_tb_per_s": bA * 2 * nvA * 2 * dA / t_one / 1e9,
+        "one_launch_speedup_vs_three": (t_sddmm + t_soft + t_av) / t_one,
+        "one_launch_max_rel_err_vs_three": float((one - chain).abs().max() / chain.abs().max()),
     }
     del qA, kA, vA, wA, pA
     return res
@@ -1012,7 +1022,7 @@ def parity_failures(tree, path=""):
 
 
 def short_extra(extra):
-    """At most a dozen scalars of the full result dictionary for the line on stdout (single-launch fractions of the
+    """About a dozen scalars of the full result dictionary for the line on stdout (single-launch fractions of the
     HBM peak, SVC speed-ups over the Python RowMerge); absent entries are left out."""
     def get(*keys):
         node = extra
@@ -1035,6 +1045,7 @@ def short_extra(extra):
         "cfg1_svc_stack_of_96_speedup_vs_python": ("cfg1_rowmerge_then_spmm_512x512", "svc_stack_of_96_such_matrices", "speedup_vs_python"),
         "cfg5_layer_speedup_vs_dense_in_a_graph": ("cfg5_encoder_layer_v16_s0.9_tokens4096", "speedup_vs_dense_layer_in_a_graph"),
         "sparse_attention_forward_s0.9_b2_ms": ("sparse_attention_forward_seq4096_h4_e256_s0.9_b2_l4", "ms_in_a_graph"),
+        "sparse_attention_block_one_launch_ms": (ATTENTION, "one_launch_ms"),
     }
     out = {}
     for name, keys in picks.items():

@@ -221,6 +221,21 @@ int sspmm_softmax_batched_f16(int batch, int m_vec, int V, const int32_t *row_in
                               const sspmm_half_t *values, float scaler, sspmm_half_t *out_values, int64_t stride,
                               void *hip_stream);
 
+/*
+ * The three steps of the attention block in one launch, for heads of F = 64 features:
+ * out[b, i*V + v, :] = sum_j softmax_j(scale * q[b, i*V + v, :] . k[b, col_j, :]) * v[b, col_j, :] over the
+ * vectors j of vector-row i; a row with no stored vectors gives zeros.  q, out: [batch][m_vec*V][64];
+ * k, v: [batch][n_keys][64]; strides in elements.  Stands for the chain bsddmm -> bcsr_softmax -> bspmm of
+ * reference end2end/sspmm_e2e/spattention.py:167-179 (which has no single operator for it): the scores and the
+ * probabilities stay on the CU, in fp32, and the probabilities enter the product rounded to fp16 before the
+ * division by their sum, so results differ from the chain's by fp16 rounding, not bit for bit.
+ * Returns invalid-value for any other F; 16-byte aligned pointers, strides multiples of 8, scale > 0.
+ */
+int sspmm_sparse_attention_f16(int batch, int m_vec, int V, int F, int n_keys, const int32_t *row_indices,
+                               const int32_t *row_offsets, const int32_t *col_idx, const sspmm_half_t *q, int64_t stride_q,
+                               const sspmm_half_t *k, int64_t stride_k, const sspmm_half_t *v, int64_t stride_v, float scale,
+                               sspmm_half_t *out, int64_t stride_out, void *hip_stream);
+
 /* ------------------------------------------------------------------------------------------
  * Sparse Vector Compression (RowMerge): CSR -> CVSE.  Replaces the Python pass
  * CVSE.__init__, reference RowMerge/sparse_matrix_format.py:94-123 (merge at :110), and adds

@@ -76,10 +76,43 @@ def csr_softmax(row_indices, row_offsets, values, scaler, vec_length):
     return bcsr_softmax(row_indices, row_offsets, values, scaler, vec_length, 1)
 
 
-def sparse_attention(row_indices, row_offsets, column_indices, q, k, v, scaling, vec_length):
+def fused_sparse_attention(row_indices, row_offsets, column_indices, q, k, v, scaling, vec_length):
+    """The block's three steps in one launch (heads of 64 features only): scores and probabilities never leave the
+    chip.  Same arguments and result shape as `sparse_attention`; differs from the three-step chain by fp16 rounding
+    of intermediate values only (the chain rounds the scores and the normalised probabilities to fp16, this rounds
+    the probabilities before the division by their sum)."""
+    _check_pattern(row_indices, row_offsets, column_indices, vec_length)
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        _check_half(name, t)
+    m, d, n = q.size(-2), q.size(-1), k.size(-2)
+    if d != 64 or k.size(-1) != 64 or v.size(-1) != 64:
+        raise ValueError("fused_sparse_attention takes heads of 64 features")
+    if v.size(-2) != n:
+        raise ValueError("k and v must have the same number of rows")
+    m_vec = row_offsets.numel() - 1
+    if m != m_vec * vec_length:
+        raise ValueError("q must have m_vec * vec_length = %d rows, got %d" % (m_vec * vec_length, m))
+    batch = q.numel() // (m * d) if m > 0 else 1
+    if k.numel() != batch * n * d or v.numel() != batch * n * d:
+        raise ValueError("q, k and v must have the same batch size")
+    out = torch.empty(q.shape, dtype=torch.float16, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = _lib.lib().sspmm_sparse_attention_f16(batch, m_vec, vec_length, d, n, _ptr(row_indices), _ptr(row_offsets),
+                                                   _ptr(column_indices), _ptr(q), m * d, _ptr(k), n * d, _ptr(v), n * d,
+                                                   float(scaling), _ptr(out), m * d, _stream())
+    _lib.check(rc, "sspmm_sparse_attention")
+    return out
+
+
+def sparse_attention(row_indices, row_offsets, column_indices, q, k, v, scaling, vec_length, fused=None):
     """softmax(mask(q k^T) * scaling) v on a vector-sparse mask shared by the batch:
     q [batch, tgt, d], k [batch, src, d], v [batch, src, d_v] -> fp16 [batch, tgt, d_v]; the three
-    steps of the reference's block (spattention.py:167-179)."""
+    steps of the reference's block (spattention.py:167-179).  fused: None = one launch where the shapes allow it
+    (d = d_v = 64), False = always the three operators, True = one launch or an error."""
+    if fused is None:
+        fused = q.size(-1) == 64 and v.size(-1) == 64 and row_offsets.numel() > 1 and q.numel() > 0
+    if fused:
+        return fused_sparse_attention(row_indices, row_offsets, column_indices, q, k, v, scaling, vec_length)
     w = bsddmm(row_indices, row_offsets, column_indices, q, k, vec_length)
     w = bcsr_softmax(row_indices, row_offsets, w, scaling, vec_length, w.size(0))
     _check_inputs(row_indices, row_offsets, column_indices, w, v, vec_length)

@@ -32,9 +32,26 @@ struct SoftmaxArgs {
   uint32_t total_work, per_xcd;
 };
 
+struct AttentionArgs {
+  int m_vec, n_keys, batch;
+  const int32_t *row_indices;  // nullable
+  const int32_t *row_offsets;
+  const int32_t *col_idx;
+  const uint16_t *q;  // [batch][m_vec*V][64]
+  const uint16_t *k;  // [batch][n_keys][64]
+  const uint16_t *v;  // [batch][n_keys][64]
+  uint16_t *out;      // [batch][m_vec*V][64]
+  int64_t stride_q, stride_k, stride_v, stride_out;  // per-batch strides in elements
+  float scale;
+  uint32_t total_work, per_xcd;  // filled by the launcher
+};
+
 // V must be 8 or 16; F a multiple of 8 up to 256; 16-byte aligned operands and strides.
 hipError_t launch_sddmm(const SddmmArgs &args, int V, hipStream_t stream);
 hipError_t launch_softmax(const SoftmaxArgs &args, int V, hipStream_t stream);
+// sddmm, softmax and the product with v in one kernel, for 64 features per row of q, k and v.  16-byte aligned
+// operands and strides; n_keys * 128 bytes below 2 GiB.
+hipError_t launch_sparse_attention(const AttentionArgs &args, int V, hipStream_t stream);
 
 }  // namespace sspmm
 #endif

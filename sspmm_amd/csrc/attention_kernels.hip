@@ -372,4 +372,217 @@ hipError_t launch_softmax(const SoftmaxArgs &a, int V, hipStream_t stream) {
   return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------- the three steps in one
+// softmax(mask(q k^T) * scale) v per vector-row without the scores ever leaving the CU, for heads of 64 features
+// (the three launches of the block, reference end2end/sspmm_e2e/spattention.py:167-179, move the scores and the
+// probabilities through memory twice each: 2 * V bytes per stored vector four times over).
+//
+// One wave per (vector-row, batch element), a step is 32 stored vectors.  The rows of k and of v the step names
+// are fetched as in the staged SpMM kernel (eight lanes on the eight 16-byte pieces of one 128-byte row, lane
+// (j, pc) = rows of k slots 4j .. 4j+3, piece pc) and written to two LDS stages with padded rows.
+//   scores:  the staged rows of k are the MFMA's first operand (lane (n, g): features 32c + 8g .. of staged row
+//            16t + n), the V rows of q the second, held in registers for the whole row; the lane ends up with the
+//            scores of query n against staged rows 16t + 4g + r, r = 0 .. 3, t = 0, 1.
+//   softmax: running maximum and running sum per query in base 2 (the scale carries log2 e); a query's scores
+//            sit in the four lanes n, n + 16, n + 32, n + 48, which exchange their maxima with two lane swaps.
+//            When the maximum moves, the sums so far are scaled down by 2^(old - new).
+//   product: the eight probabilities of a lane are, in this order, the second operand's k slots 8g .. 8g+7 of
+//            query n; the first operand is the transpose read of the staged rows of v in the matching order
+//            (rows 4g .. 4g+3, then 16 + 4g .. 16 + 4g + 3).  Lane (n, g) accumulates features 16u + 4g + r of
+//            query n, u = 0 .. 3, divides by the sum at the end and stores four times 8 bytes.
+// The probabilities enter the product rounded to fp16 before the division by the sum (the three launches round
+// after it); sums are fp32 throughout.
+// The launch is bound by the stream of gathered rows from the L2 into the CUs (256 bytes per stored vector and batch
+// element; measured 21 TB/s on 4096 keys, 90 % masked, 48 heads), not by waves in flight: two waves per SIMD with
+// the registers that allows measured 2-7 % faster than three, and four (which spills) 75 % slower.
+namespace {
+
+typedef __attribute__((address_space(3))) short lds_short4 __attribute__((ext_vector_type(4)));
+typedef short shortx4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uintx2 lds_read_tr(const unsigned char *p) {
+  const shortx4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) shortx4 *)p);
+  return __builtin_bit_cast(uintx2, v);
+}
+
+// max / sum over the four lanes n, n + 16, n + 32, n + 48, in each of them
+__device__ __forceinline__ float quad_rows_max(float x) {
+  const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float quad_rows_sum(float x) {
+  const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+static constexpr uint32_t kAttnPitch = 144;  // bytes per staged row: 64 features and 16 of padding
+
+}  // namespace
+
+template <int V>
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void sparse_attention_kernel(const AttentionArgs p) {
+  __shared__ __align__(16) unsigned char stage_k[32 * kAttnPitch];
+  __shared__ __align__(16) unsigned char stage_v[32 * kAttnPitch];
+  const uint32_t w = xcd_work_index(p.per_xcd);
+  if (w >= p.total_work) return;
+  const uint32_t r = w % (uint32_t)p.m_vec;
+  const uint32_t batch = w / (uint32_t)p.m_vec;
+  const int row = __builtin_amdgcn_readfirstlane(p.row_indices ? p.row_indices[r] : (int)r);
+  const int beg = p.row_offsets[row], end = p.row_offsets[row + 1];
+  const int lane = threadIdx.x, n = lane & 15, g = lane >> 4, j = lane >> 3, pc = lane & 7;
+
+  uint16_t *out = p.out + (int64_t)batch * p.stride_out + ((int64_t)row * V + n) * 64 + 4 * g;
+  if (beg == end) {  // a query that attends to nothing: zeros, as the product with no stored vectors gives
+    if (n < V) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) *reinterpret_cast<uintx2 *>(out + 16 * u) = uintx2{0u, 0u};
+    }
+    return;
+  }
+  const __amdgpu_buffer_rsrc_t srd_q = make_srd(p.q + (int64_t)batch * p.stride_q + (int64_t)row * V * 64, (uint32_t)V * 128u);
+  const uint32_t kv_bytes = (uint32_t)p.n_keys * 128u;
+  const __amdgpu_buffer_rsrc_t srd_k = make_srd(p.k + (int64_t)batch * p.stride_k, kv_bytes);
+  const __amdgpu_buffer_rsrc_t srd_v = make_srd(p.v + (int64_t)batch * p.stride_v, kv_bytes);
+  const __amdgpu_buffer_rsrc_t srd_cols = make_srd(p.col_idx, (uint32_t)end * 4u);  // past the row: reads 0
+
+  half8 q[2];
+#pragma unroll
+  for (int c = 0; c < 2; ++c)  // (rows past V: beyond the descriptor, zeros)
+    q[c] = __builtin_bit_cast(half8, __builtin_amdgcn_raw_buffer_load_b128(srd_q, (uint32_t)n * 128u + (32u * c + 8u * g) * 2u, 0, 0));
+
+  unsigned char *const k_dst = stage_k + (uint32_t)(4 * j) * kAttnPitch + (uint32_t)pc * 16u;
+  unsigned char *const v_dst = stage_v + (uint32_t)(4 * j) * kAttnPitch + (uint32_t)pc * 16u;
+  const unsigned char *const k_rd = stage_k + (uint32_t)n * kAttnPitch + (uint32_t)g * 16u;
+  const unsigned char *const v_rd = stage_v + (uint32_t)(4 * g + (n >> 2)) * kAttnPitch + (uint32_t)(n & 3) * 8u;
+  const uint32_t piece_off = (uint32_t)pc * 16u;
+  const float scale2 = p.scale * 1.4426950408889634f;
+
+  struct Body {
+    uintx4 k[4], v[4];
+  };
+  const auto load_head = [&](int kc) {
+    return __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_cols, (kc + 4 * j) * 4, 0, 0));
+  };
+  const auto load_body = [&](Body &b, const uintx4 &cols, int kc) {
+    uint32_t off[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) off[i] = cols[i] * 128u + piece_off;
+    if (kc + 32 > end) {  // (uniform) the row's last step: slots past its end fetch zeros
+#pragma unroll
+      for (int i = 0; i < 4; ++i) off[i] = (kc + 4 * j + i < end) ? off[i] : kv_bytes;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) b.k[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_k, off[i], 0, 0));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) b.v[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_v, off[i], 0, 0));
+  };
+
+  floatx4 acc[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) acc[u] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float run_max = -INFINITY, run_sum = 0.f;  // of query n; the sum only over this lane's share of the keys
+
+  const auto contract = [&](const Body &b, int kc) {
+    // (LDS operations of a wave execute in order: these writes land behind the previous step's reads)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<uintx4 *>(k_dst + i * kAttnPitch) = b.k[i];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<uintx4 *>(v_dst + i * kAttnPitch) = b.v[i];
+    float x[8];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      floatx4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        const half8 a = *reinterpret_cast<const half8 *>(k_rd + (uint32_t)t * (16u * kAttnPitch) + (uint32_t)c * 64u);
+        s = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, q[c], s, 0, 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) x[4 * t + i] = s[i] * scale2;
+    }
+    if (kc + 32 > end) {  // (uniform)
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (kc + 16 * t + 4 * g + i >= end) x[4 * t + i] = -INFINITY;
+    }
+    float mx = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+    mx = quad_rows_max(mx);  // finite: the step's first slot is always a stored vector
+    const float new_max = fmaxf(run_max, mx);
+    if (__builtin_amdgcn_ballot_w64(new_max > run_max)) {  // (uniform) some query's maximum moved
+      const float alpha = __builtin_amdgcn_exp2f(run_max - new_max);
+      run_sum *= alpha;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) acc[u] *= alpha;
+      run_max = new_max;
+    }
+    float e[8], sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      e[i] = __builtin_amdgcn_exp2f(x[i] - run_max);
+      sum += e[i];
+    }
+    run_sum += sum;
+    const half8 pb = {(_Float16)e[0], (_Float16)e[1], (_Float16)e[2], (_Float16)e[3],
+                      (_Float16)e[4], (_Float16)e[5], (_Float16)e[6], (_Float16)e[7]};
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const uintx2 lo = lds_read_tr(v_rd + 32u * u);
+      const uintx2 hi = lds_read_tr(v_rd + 16u * kAttnPitch + 32u * u);
+      const uintx4 a = {lo[0], lo[1], hi[0], hi[1]};
+      acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), pb, acc[u], 0, 0, 0);
+    }
+  };
+
+  // Column indices run two steps ahead of the arithmetic, the rows of k and v one (two sets, used alternately).
+  Body b0, b1;
+  uintx4 h0 = load_head(beg), h1 = load_head(beg + 32);
+  load_body(b0, h0, beg);
+  int kc = beg;  // the step held in b0
+  for (;;) {
+    if (kc + 32 >= end) {
+      contract(b0, kc);
+      break;
+    }
+    h0 = load_head(kc + 64);
+    load_body(b1, h1, kc + 32);
+    contract(b0, kc);
+    kc += 32;
+    if (kc + 32 >= end) {
+      contract(b1, kc);
+      break;
+    }
+    h1 = load_head(kc + 64);
+    load_body(b0, h0, kc + 32);
+    contract(b1, kc);
+    kc += 32;
+  }
+
+  const float inv = 1.0f / quad_rows_sum(run_sum);
+  if (n < V) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const half4 h = {(_Float16)(acc[u][0] * inv), (_Float16)(acc[u][1] * inv), (_Float16)(acc[u][2] * inv), (_Float16)(acc[u][3] * inv)};
+      *reinterpret_cast<uintx2 *>(out + 16 * u) = __builtin_bit_cast(uintx2, h);
+    }
+  }
+}
+
+hipError_t launch_sparse_attention(const AttentionArgs &a, int V, hipStream_t stream) {
+  AttentionArgs p = a;
+  p.total_work = (uint32_t)a.m_vec * (uint32_t)a.batch;
+  p.per_xcd = (p.total_work + 7u) / 8u;
+  if (p.total_work == 0) return hipSuccess;
+  if (V == 8)
+    hipLaunchKernelGGL(sparse_attention_kernel<8>, dim3(p.per_xcd * 8u), dim3(64), 0, stream, p);
+  else
+    hipLaunchKernelGGL(sparse_attention_kernel<16>, dim3(p.per_xcd * 8u), dim3(64), 0, stream, p);
+  return hipGetLastError();
+}
+
 }  // namespace sspmm

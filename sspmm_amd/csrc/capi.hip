@@ -262,6 +262,40 @@ int sspmm_softmax_f16(int m_vec, int V, const int32_t *row_indices, const int32_
   return sspmm_softmax_batched_f16(1, m_vec, V, row_indices, row_offsets, values, scaler, out_values, 0, hip_stream);
 }
 
+int sspmm_sparse_attention_f16(int batch, int m_vec, int V, int F, int n_keys, const int32_t *row_indices,
+                               const int32_t *row_offsets, const int32_t *col_idx, const sspmm_half_t *q, int64_t stride_q,
+                               const sspmm_half_t *k, int64_t stride_k, const sspmm_half_t *v, int64_t stride_v, float scale,
+                               sspmm_half_t *out, int64_t stride_out, void *hip_stream) {
+  if (V != 8 && V != 16) return kInvalid;
+  if (F != 64) return kInvalid;
+  if (batch < 0 || m_vec < 0 || n_keys < 0) return kInvalid;
+  if (!(scale > 0.f) || !std::isfinite(scale)) return kInvalid;
+  if (batch == 0 || m_vec == 0) return 0;
+  if (!row_offsets || !col_idx || !q || !k || !v || !out) return kInvalid;
+  if ((int64_t)m_vec * batch >= (1ll << 31) - 8 || (int64_t)n_keys * 128 >= (1ll << 31)) return kInvalid;
+  if (reinterpret_cast<uintptr_t>(q) % 16 || reinterpret_cast<uintptr_t>(k) % 16 || reinterpret_cast<uintptr_t>(v) % 16 ||
+      reinterpret_cast<uintptr_t>(out) % 16 || stride_q % 8 || stride_k % 8 || stride_v % 8 || stride_out % 8)
+    return kInvalid;
+  if (batch > 1 && stride_out < (int64_t)m_vec * V * 64) return kInvalid;  // (the batch elements' outputs must not overlap)
+  sspmm::AttentionArgs a{};
+  a.m_vec = m_vec;
+  a.n_keys = n_keys;
+  a.batch = batch;
+  a.row_indices = row_indices;
+  a.row_offsets = row_offsets;
+  a.col_idx = col_idx;
+  a.q = q;
+  a.k = k;
+  a.v = v;
+  a.out = out;
+  a.stride_q = stride_q;
+  a.stride_k = stride_k;
+  a.stride_v = stride_v;
+  a.stride_out = stride_out;
+  a.scale = scale;
+  return (int)sspmm::launch_sparse_attention(a, V, static_cast<hipStream_t>(hip_stream));
+}
+
 size_t svc_workspace_bytes(int M, int64_t nnz, int V) {
   if (M < 0 || V < 1) return 0;
   return sspmm::svc_workspace_layout(nnz, (M + V - 1) / V, nullptr, nullptr, nullptr);

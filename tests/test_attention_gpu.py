@@ -97,14 +97,16 @@ def test_batched_ops_match_looped_single_calls(oracle, built_library):
         assert torch.equal(p[b], sspmm_amd.csr_softmax(None, off, w[b].contiguous(), 0.125, V))
 
 
+@pytest.mark.parametrize("fused", [False, True])
 @pytest.mark.parametrize("V", [8, 16])
-def test_sparse_attention_matches_dense_masked_attention(built_library, V):
-    """The reference's block (sddmm -> softmax -> spmm) against torch attention with a -inf mask."""
+def test_sparse_attention_matches_dense_masked_attention(built_library, V, fused):
+    """The reference's block (sddmm -> softmax -> spmm), as three launches and as one, against torch attention
+    with a -inf mask."""
     seq, d, batch = 256, 64, 6
     vs = _pattern(seq // V, seq, V, 0.8, seed=11)
     g = torch.Generator("cuda").manual_seed(12)
     q, k, v = (torch.randn(batch, seq, d, device="cuda", generator=g).half() for _ in range(3))
-    out = sspmm_amd.sparse_attention(None, dev(vs.row_offsets), dev(vs.col_idx), q, k, v, 1.0 / math.sqrt(d), V)
+    out = sspmm_amd.sparse_attention(None, dev(vs.row_offsets), dev(vs.col_idx), q, k, v, 1.0 / math.sqrt(d), V, fused=fused)
     torch.cuda.synchronize()
     mask = torch.full((seq, seq), float("-inf"), device="cuda")
     for i in range(vs.m_vec):
@@ -116,6 +118,67 @@ def test_sparse_attention_matches_dense_masked_attention(built_library, V):
     assert max_rel_err(out.float().cpu().numpy(), want.cpu().numpy()) <= 1e-2
 
 
+def _dense_attention(off, cols, V, q, k, v, scale):
+    """float64 numpy: per vector-row, softmax over the stored columns, rows without any give zeros."""
+    batch, m, d = q.shape
+    out = np.zeros((batch, m, v.shape[-1]))
+    q64, k64, v64 = (t.astype(np.float64) for t in (q, k, v))
+    for i in range(len(off) - 1):
+        c = cols[off[i]:off[i + 1]]
+        if c.size == 0:
+            continue
+        s = np.einsum("bvd,bjd->bvj", q64[:, i * V:(i + 1) * V], k64[:, c]) * scale
+        e = np.exp(s - s.max(axis=-1, keepdims=True))
+        out[:, i * V:(i + 1) * V] = np.einsum("bvj,bjd->bvd", e / e.sum(axis=-1, keepdims=True), v64[:, c])
+    return out
+
+
+@pytest.mark.parametrize("V", [8, 16])
+def test_one_launch_attention_row_lengths_permutation_and_large_scores(built_library, V):
+    """Rows of every length around the kernel's step of 32 vectors (none, one, a full step, one more, several steps
+    and a tail), visited through a permutation, with scores large enough that the running maximum has to move by
+    hundreds between steps; against float64 arithmetic and against the three launches."""
+    n_keys, d, batch = 200, 64, 3
+    lens = [0, 1, 2, 31, 32, 33, 63, 64, 65, 96, 100, 200, 0, 7]
+    rng = np.random.default_rng(40 + V)
+    cols = np.concatenate([np.sort(rng.permutation(n_keys)[:n]) for n in lens]).astype(np.int32)
+    off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    m = len(lens) * V
+    q = (rng.standard_normal((batch, m, d)) * 3).astype(np.float16)
+    k = (rng.standard_normal((batch, n_keys, d)) * 3).astype(np.float16)
+    v = rng.standard_normal((batch, n_keys, d)).astype(np.float16)
+    perm = dev(rng.permutation(len(lens)).astype(np.int32))
+    for scale in (0.125, 2.0):  # scores up to a few hundred, then a few thousand
+        want = _dense_attention(off, cols, V, q, k, v, scale)
+        for ri in (None, perm):
+            print("attention V=%d scale=%g permuted=%s" % (V, scale, ri is not None), flush=True)
+            got = sspmm_amd.fused_sparse_attention(ri, dev(off), dev(cols), dev(q), dev(k), dev(v), scale, V)
+            torch.cuda.synchronize()
+            got = got.cpu().numpy().astype(np.float64)
+            assert np.isfinite(got).all()
+            assert np.abs(got - want).max() <= 4e-3 * max(1.0, np.abs(want).max())
+            for i, n in enumerate(lens):
+                if n == 0:
+                    assert not got[:, i * V:(i + 1) * V].any()
+    chain = sspmm_amd.sparse_attention(None, dev(off), dev(cols), dev(q), dev(k), dev(v), 0.125, V, fused=False)
+    one = sspmm_amd.sparse_attention(None, dev(off), dev(cols), dev(q), dev(k), dev(v), 0.125, V)  # picks the one launch
+    assert torch.equal(one, sspmm_amd.fused_sparse_attention(None, dev(off), dev(cols), dev(q), dev(k), dev(v), 0.125, V))
+    # (the chain rounds scores of magnitude up to ~100 to fp16, a step of 1/16 in the exponent's argument before the scale)
+    assert (one.float() - chain.float()).abs().max().item() <= 3e-2
+
+
+def test_one_launch_attention_of_a_single_key_returns_its_value_row(built_library):
+    """A query that attends to one key gets that row of v back exactly (probability one, fp16 in and out)."""
+    V, n_keys, m_vec = 8, 50, 5
+    rng = np.random.default_rng(3)
+    cols = rng.integers(0, n_keys, m_vec).astype(np.int32)
+    off = np.arange(m_vec + 1, dtype=np.int32)
+    q, k, v = (rng.standard_normal((2, n, 64)).astype(np.float16) for n in (m_vec * V, n_keys, n_keys))
+    got = sspmm_amd.fused_sparse_attention(None, dev(off), dev(cols), dev(q), dev(k), dev(v), 0.125, V).cpu().numpy()
+    for i in range(m_vec):
+        assert np.array_equal(got[:, i * V:(i + 1) * V], np.repeat(v[:, cols[i]][:, None], V, axis=1))
+
+
 def test_argument_errors(built_library):
     off = torch.zeros(3, dtype=torch.int32, device="cuda")
     col = torch.zeros(0, dtype=torch.int32, device="cuda")
@@ -125,6 +188,10 @@ def test_argument_errors(built_library):
         sspmm_amd.sddmm(None, off, col, torch.zeros(16, 64, device="cuda").half(), torch.zeros(8, 32, device="cuda").half(), 8)
     with pytest.raises(TypeError):
         sspmm_amd.csr_softmax(None, off, torch.zeros(0, device="cuda"), 1.0, 8)
+    with pytest.raises(ValueError):  # the one-launch block takes heads of 64 features only
+        sspmm_amd.fused_sparse_attention(None, off, col, *(torch.zeros(1, 16, 32, device="cuda").half() for _ in range(3)), 1.0, 8)
+    with pytest.raises(RuntimeError):  # scale must be positive
+        sspmm_amd.fused_sparse_attention(None, off, col, *(torch.zeros(1, 16, 64, device="cuda").half() for _ in range(3)), 0.0, 8)
     with pytest.raises(RuntimeError):  # F must be a multiple of 8
         sspmm_amd.sddmm(None, off, col, torch.zeros(16, 12, device="cuda").half(), torch.zeros(8, 12, device="cuda").half(), 8)
 

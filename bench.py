@@ -1022,7 +1022,7 @@ def parity_failures(tree, path=""):
 
 
 def short_extra(extra):
-    """About a dozen scalars of the full result dictionary for the line on stdout (single-launch fractions of the
+    """At most a dozen scalars of the full result dictionary for the line on stdout (single-launch fractions of the
     HBM peak, SVC speed-ups over the Python RowMerge); absent entries are left out."""
     def get(*keys):
         node = extra
@@ -1042,7 +1042,6 @@ def short_extra(extra):
         "cfg4_spmm_with_plan_ms": ("cfg4_spmm_on_svc_output_with_plan", "ms"),
         "svc_cfg4_speedup_vs_python": ("svc_cfg4_zipf_16384_v8", "speedup_vs_python"),
         "svc_batched_dlmc_shapes_speedup_vs_python": ("svc_batched_dlmc_shapes", "speedup_vs_python"),
-        "cfg1_svc_stack_of_96_speedup_vs_python": ("cfg1_rowmerge_then_spmm_512x512", "svc_stack_of_96_such_matrices", "speedup_vs_python"),
         "cfg5_layer_speedup_vs_dense_in_a_graph": ("cfg5_encoder_layer_v16_s0.9_tokens4096", "speedup_vs_dense_layer_in_a_graph"),
         "sparse_attention_forward_s0.9_b2_ms": ("sparse_attention_forward_seq4096_h4_e256_s0.9_b2_l4", "ms_in_a_graph"),
         "sparse_attention_block_one_launch_ms": (ATTENTION, "one_launch_ms"),

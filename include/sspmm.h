@@ -236,6 +236,22 @@ int sspmm_sparse_attention_f16(int batch, int m_vec, int V, int F, int n_keys, c
                                const sspmm_half_t *k, int64_t stride_k, const sspmm_half_t *v, int64_t stride_v, float scale,
                                sspmm_half_t *out, int64_t stride_out, void *hip_stream);
 
+/*
+ * The same launch on operands that hold several heads side by side, so that a model's fused projection can be used
+ * where it lies: row r of (batch element e, head h) starts at x + e*stride_x + h*head_x + r*ld_x (elements; 64
+ * features each), for x = q, k, v and out.  The mask is shared by all batch * heads pairs.  For the output of a
+ * projection [seq][batch][3 * heads * 64] (reference spattention.py:151-157 copies q, k and v out of it and into
+ * [batch * heads][seq][64] first): q = qkv, k = qkv + heads*64, v = qkv + 2*heads*64, stride = 3*heads*64,
+ * head = 64, ld = batch*3*heads*64.  Strides non-negative multiples of 8, ld >= 64; the caller sees to it that no two
+ * rows of out overlap.  No counterpart in the reference.
+ */
+int sspmm_sparse_attention_heads_f16(int batch, int heads, int m_vec, int V, int F, int n_keys, const int32_t *row_indices,
+                                     const int32_t *row_offsets, const int32_t *col_idx, const sspmm_half_t *q,
+                                     int64_t stride_q, int64_t head_q, int64_t ld_q, const sspmm_half_t *k, int64_t stride_k,
+                                     int64_t head_k, int64_t ld_k, const sspmm_half_t *v, int64_t stride_v, int64_t head_v,
+                                     int64_t ld_v, float scale, sspmm_half_t *out, int64_t stride_out, int64_t head_out,
+                                     int64_t ld_out, void *hip_stream);
+
 /* ------------------------------------------------------------------------------------------
  * Sparse Vector Compression (RowMerge): CSR -> CVSE.  Replaces the Python pass
  * CVSE.__init__, reference RowMerge/sparse_matrix_format.py:94-123 (merge at :110), and adds

@@ -11,7 +11,7 @@ operator raises.
 from .spmm import spmm, bspmm, sorted_row_swizzle  # noqa: F401
 from .plan import Plan, PlanInfo  # noqa: F401
 from .svc import svc, svc_batched, stack_csr, SvcBatch, SvcResult  # noqa: F401
-from .attention import sddmm, bsddmm, csr_softmax, bcsr_softmax, sparse_attention, fused_sparse_attention  # noqa: F401
+from .attention import sddmm, bsddmm, csr_softmax, bcsr_softmax, sparse_attention, fused_sparse_attention, sparse_attention_packed  # noqa: F401
 from .reorder import minhash_order, permute_csr, svc_reordered  # noqa: F401
 from .layers import SparseLinear, SparseEncoderLayer  # noqa: F401
 from .formats import Cvse, read_smtx, write_smtx, read_cvse, write_cvse, cvse_text  # noqa: F401

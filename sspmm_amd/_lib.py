@@ -35,6 +35,8 @@ SIGNATURES = {
     "sspmm_softmax_batched_f16": (_int, [_int, _int, _int, _vp, _vp, _vp, ctypes.c_float, _vp, _i64, _vp]),
     "sspmm_sparse_attention_f16": (_int, [_int, _int, _int, _int, _int, _vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64,
                                           ctypes.c_float, _vp, _i64, _vp]),
+    "sspmm_sparse_attention_heads_f16": (_int, [_int, _int, _int, _int, _int, _int, _vp, _vp, _vp, _vp, _i64, _i64, _i64,
+                                                _vp, _i64, _i64, _i64, _vp, _i64, _i64, _i64, ctypes.c_float, _vp, _i64, _i64, _i64, _vp]),
     "svc_workspace_bytes": (ctypes.c_size_t, [_int, _i64, _int]),
     "svc_count": (_int, [_int, _int, _int, _vp, _vp, _i64, _int, _vp, _vp, _vp]),
     "svc_fill": (_int, [_int, _int, _int, _vp, _vp, _vp, _i64, _int, _vp, _vp, _vp, _vp, _vp]),

@@ -104,6 +104,31 @@ def fused_sparse_attention(row_indices, row_offsets, column_indices, q, k, v, sc
     return out
 
 
+def sparse_attention_packed(row_indices, row_offsets, column_indices, qkv, num_heads, scaling, vec_length):
+    """Multi-head attention on a vector-sparse mask straight from a fused projection: qkv [seq, batch, 3 * embed] (q,
+    k and v side by side in the last dimension, heads of 64 features side by side in each) -> [seq, batch, embed],
+    in one launch and without the copies into [batch * heads, seq, 64] and back that the reference's module makes
+    around its three operators (spattention.py:151-157 and 181-184)."""
+    _check_pattern(row_indices, row_offsets, column_indices, vec_length)
+    _check_half("qkv", qkv)
+    if qkv.dim() != 3 or qkv.size(-1) != 3 * num_heads * 64:
+        raise ValueError("qkv must be [seq, batch, 3 * num_heads * 64]")
+    seq, bsz, three_e = qkv.shape
+    e = three_e // 3
+    m_vec = row_offsets.numel() - 1
+    if seq != m_vec * vec_length:
+        raise ValueError("qkv must have m_vec * vec_length = %d rows, got %d" % (m_vec * vec_length, seq))
+    out = torch.empty((seq, bsz, e), dtype=torch.float16, device=qkv.device)
+    base, ld = qkv.data_ptr(), bsz * three_e
+    with torch.cuda.device(qkv.device):
+        rc = _lib.lib().sspmm_sparse_attention_heads_f16(
+            bsz, num_heads, m_vec, vec_length, 64, seq, _ptr(row_indices), _ptr(row_offsets), _ptr(column_indices),
+            base, three_e, 64, ld, base + 2 * e, three_e, 64, ld, base + 4 * e, three_e, 64, ld, float(scaling),
+            _ptr(out), e, 64, bsz * e, _stream())
+    _lib.check(rc, "sspmm_sparse_attention_heads")
+    return out
+
+
 def sparse_attention(row_indices, row_offsets, column_indices, q, k, v, scaling, vec_length, fused=None):
     """softmax(mask(q k^T) * scaling) v on a vector-sparse mask shared by the batch:
     q [batch, tgt, d], k [batch, src, d], v [batch, src, d_v] -> fp16 [batch, tgt, d_v]; the three
@@ -161,10 +186,15 @@ class SparseAttentionBlock(torch.nn.Module):
         are replaced by dense masked attention in fp32 (for checks)."""
         seq, bsz, E = x.shape
         h, d = self.num_heads, E // self.num_heads
-        q, k, v = self.in_proj(x).chunk(3, dim=-1)
+        scaling = float(d) ** -0.5
+        qkv = self.in_proj(x)
+        if dense_mask is None and d == 64 and qkv.dtype == torch.float16:
+            # the heads are read where the projection left them and written where the output projection wants them
+            return self.out_proj(sparse_attention_packed(self.row_indices, self.row_offsets, self.column_indices,
+                                                         qkv.contiguous(), h, scaling, self.vec_length))
+        q, k, v = qkv.chunk(3, dim=-1)
         # [seq, batch * heads, d] -> [batch * heads, seq, d] (spattention.py:151-157)
         q, k, v = (t.contiguous().view(seq, bsz * h, d).transpose(0, 1).contiguous() for t in (q, k, v))
-        scaling = float(d) ** -0.5
         if dense_mask is None:
             out = sparse_attention(self.row_indices, self.row_offsets, self.column_indices, q, k, v, scaling, self.vec_length)
         else:

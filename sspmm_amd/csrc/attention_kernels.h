@@ -33,15 +33,17 @@ struct SoftmaxArgs {
 };
 
 struct AttentionArgs {
-  int m_vec, n_keys, batch;
+  int m_vec, n_keys, batch, heads;  // batch counts (batch element, head) pairs: element = index / heads, head = index % heads
   const int32_t *row_indices;  // nullable
   const int32_t *row_offsets;
   const int32_t *col_idx;
-  const uint16_t *q;  // [batch][m_vec*V][64]
-  const uint16_t *k;  // [batch][n_keys][64]
-  const uint16_t *v;  // [batch][n_keys][64]
-  uint16_t *out;      // [batch][m_vec*V][64]
-  int64_t stride_q, stride_k, stride_v, stride_out;  // per-batch strides in elements
+  const uint16_t *q;  // row r of (element e, head h) at q + e * stride_q + h * head_q + r * ld_q, 64 features each
+  const uint16_t *k;  // n_keys rows per (element, head), addressed the same way
+  const uint16_t *v;
+  uint16_t *out;      // m_vec * V rows per (element, head)
+  int64_t stride_q, stride_k, stride_v, stride_out;  // between batch elements, in elements
+  int64_t head_q, head_k, head_v, head_out;          // between the heads of an element
+  int64_t ld_q, ld_k, ld_v, ld_out;                  // between rows
   float scale;
   uint32_t total_work, per_xcd;  // filled by the launcher
 };
@@ -50,7 +52,7 @@ struct AttentionArgs {
 hipError_t launch_sddmm(const SddmmArgs &args, int V, hipStream_t stream);
 hipError_t launch_softmax(const SoftmaxArgs &args, int V, hipStream_t stream);
 // sddmm, softmax and the product with v in one kernel, for 64 features per row of q, k and v.  16-byte aligned
-// operands and strides; n_keys * 128 bytes below 2 GiB.
+// operands and strides; the rows of one (element, head) span less than 2 GiB.
 hipError_t launch_sparse_attention(const AttentionArgs &args, int V, hipStream_t stream);
 
 }  // namespace sspmm

@@ -435,7 +435,8 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   const int beg = p.row_offsets[row], end = p.row_offsets[row + 1];
   const int lane = threadIdx.x, n = lane & 15, g = lane >> 4, j = lane >> 3, pc = lane & 7;
 
-  uint16_t *out = p.out + (int64_t)batch * p.stride_out + ((int64_t)row * V + n) * 64 + 4 * g;
+  const uint32_t elem = batch / (uint32_t)p.heads, head = batch % (uint32_t)p.heads;
+  uint16_t *out = p.out + (int64_t)elem * p.stride_out + (int64_t)head * p.head_out + ((int64_t)row * V + n) * p.ld_out + 4 * g;
   if (beg == end) {  // a query that attends to nothing: zeros, as the product with no stored vectors gives
     if (n < V) {
 #pragma unroll
@@ -443,16 +444,19 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     }
     return;
   }
-  const __amdgpu_buffer_rsrc_t srd_q = make_srd(p.q + (int64_t)batch * p.stride_q + (int64_t)row * V * 64, (uint32_t)V * 128u);
-  const uint32_t kv_bytes = (uint32_t)p.n_keys * 128u;
-  const __amdgpu_buffer_rsrc_t srd_k = make_srd(p.k + (int64_t)batch * p.stride_k, kv_bytes);
-  const __amdgpu_buffer_rsrc_t srd_v = make_srd(p.v + (int64_t)batch * p.stride_v, kv_bytes);
+  // (descriptors end with the last row's 128 bytes; between the rows of a strided operand lies what belongs to other heads)
+  const uint32_t q_row = (uint32_t)p.ld_q * 2u, k_row = (uint32_t)p.ld_k * 2u, v_row = (uint32_t)p.ld_v * 2u;
+  const __amdgpu_buffer_rsrc_t srd_q = make_srd(p.q + (int64_t)elem * p.stride_q + (int64_t)head * p.head_q + (int64_t)row * V * p.ld_q,
+                                                (uint32_t)(V - 1) * q_row + 128u);
+  const uint32_t k_bytes = (uint32_t)(p.n_keys - 1) * k_row + 128u, v_bytes = (uint32_t)(p.n_keys - 1) * v_row + 128u;
+  const __amdgpu_buffer_rsrc_t srd_k = make_srd(p.k + (int64_t)elem * p.stride_k + (int64_t)head * p.head_k, k_bytes);
+  const __amdgpu_buffer_rsrc_t srd_v = make_srd(p.v + (int64_t)elem * p.stride_v + (int64_t)head * p.head_v, v_bytes);
   const __amdgpu_buffer_rsrc_t srd_cols = make_srd(p.col_idx, (uint32_t)end * 4u);  // past the row: reads 0
 
   half8 q[2];
 #pragma unroll
   for (int c = 0; c < 2; ++c)  // (rows past V: beyond the descriptor, zeros)
-    q[c] = __builtin_bit_cast(half8, __builtin_amdgcn_raw_buffer_load_b128(srd_q, (uint32_t)n * 128u + (32u * c + 8u * g) * 2u, 0, 0));
+    q[c] = __builtin_bit_cast(half8, __builtin_amdgcn_raw_buffer_load_b128(srd_q, n < V ? (uint32_t)n * q_row + (32u * c + 8u * g) * 2u : 0xfffffff0u, 0, 0));
 
   unsigned char *const k_dst = stage_k + (uint32_t)(4 * j) * kAttnPitch + (uint32_t)pc * 16u;
   unsigned char *const v_dst = stage_v + (uint32_t)(4 * j) * kAttnPitch + (uint32_t)pc * 16u;
@@ -468,17 +472,24 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     return __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_cols, (kc + 4 * j) * 4, 0, 0));
   };
   const auto load_body = [&](Body &b, const uintx4 &cols, int kc) {
-    uint32_t off[4];
+    uint32_t ok[4], ov[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) off[i] = cols[i] * 128u + piece_off;
+    for (int i = 0; i < 4; ++i) {
+      ok[i] = __umul24(cols[i], k_row) + piece_off;  // (both factors below 2^24: the launcher's caller checks the row pitch)
+      ov[i] = __umul24(cols[i], v_row) + piece_off;
+    }
     if (kc + 32 > end) {  // (uniform) the row's last step: slots past its end fetch zeros
 #pragma unroll
-      for (int i = 0; i < 4; ++i) off[i] = (kc + 4 * j + i < end) ? off[i] : kv_bytes;
+      for (int i = 0; i < 4; ++i) {
+        const bool live = kc + 4 * j + i < end;
+        ok[i] = live ? ok[i] : k_bytes;
+        ov[i] = live ? ov[i] : v_bytes;
+      }
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) b.k[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_k, off[i], 0, 0));
+    for (int i = 0; i < 4; ++i) b.k[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_k, ok[i], 0, 0));
 #pragma unroll
-    for (int i = 0; i < 4; ++i) b.v[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_v, off[i], 0, 0));
+    for (int i = 0; i < 4; ++i) b.v[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_v, ov[i], 0, 0));
   };
 
   floatx4 acc[4];

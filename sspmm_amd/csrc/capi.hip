@@ -262,25 +262,36 @@ int sspmm_softmax_f16(int m_vec, int V, const int32_t *row_indices, const int32_
   return sspmm_softmax_batched_f16(1, m_vec, V, row_indices, row_offsets, values, scaler, out_values, 0, hip_stream);
 }
 
-int sspmm_sparse_attention_f16(int batch, int m_vec, int V, int F, int n_keys, const int32_t *row_indices,
-                               const int32_t *row_offsets, const int32_t *col_idx, const sspmm_half_t *q, int64_t stride_q,
-                               const sspmm_half_t *k, int64_t stride_k, const sspmm_half_t *v, int64_t stride_v, float scale,
-                               sspmm_half_t *out, int64_t stride_out, void *hip_stream) {
+int sspmm_sparse_attention_heads_f16(int batch, int heads, int m_vec, int V, int F, int n_keys, const int32_t *row_indices,
+                                     const int32_t *row_offsets, const int32_t *col_idx, const sspmm_half_t *q,
+                                     int64_t stride_q, int64_t head_q, int64_t ld_q, const sspmm_half_t *k, int64_t stride_k,
+                                     int64_t head_k, int64_t ld_k, const sspmm_half_t *v, int64_t stride_v, int64_t head_v,
+                                     int64_t ld_v, float scale, sspmm_half_t *out, int64_t stride_out, int64_t head_out,
+                                     int64_t ld_out, void *hip_stream) {
   if (V != 8 && V != 16) return kInvalid;
   if (F != 64) return kInvalid;
-  if (batch < 0 || m_vec < 0 || n_keys < 0) return kInvalid;
+  if (batch < 0 || heads < 1 || m_vec < 0 || n_keys < 0) return kInvalid;
   if (!(scale > 0.f) || !std::isfinite(scale)) return kInvalid;
   if (batch == 0 || m_vec == 0) return 0;
   if (!row_offsets || !col_idx || !q || !k || !v || !out) return kInvalid;
-  if ((int64_t)m_vec * batch >= (1ll << 31) - 8 || (int64_t)n_keys * 128 >= (1ll << 31)) return kInvalid;
+  if ((int64_t)m_vec * batch * heads >= (1ll << 31) - 8) return kInvalid;
+  const int64_t strides[] = {stride_q, head_q, ld_q, stride_k, head_k, ld_k, stride_v, head_v, ld_v, stride_out, head_out, ld_out};
+  for (int64_t x : strides)
+    if (x % 8 || x < 0) return kInvalid;
+  if (ld_q < 64 || ld_k < 64 || ld_v < 64 || ld_out < 64) return kInvalid;
+  if (ld_k >= (1 << 23) || ld_v >= (1 << 23) || n_keys >= (1 << 24)) return kInvalid;  // (24-bit multiplies of column by row pitch)
+  // one buffer descriptor spans the rows of an (element, head) pair
+  const int64_t rows_q = (int64_t)m_vec * V, limit = (1ll << 31) - 256;
+  if (n_keys > 0 && ((n_keys - 1) * ld_k * 2 >= limit || (n_keys - 1) * ld_v * 2 >= limit)) return kInvalid;
+  if ((rows_q - 1) * ld_q * 2 >= limit) return kInvalid;
   if (reinterpret_cast<uintptr_t>(q) % 16 || reinterpret_cast<uintptr_t>(k) % 16 || reinterpret_cast<uintptr_t>(v) % 16 ||
-      reinterpret_cast<uintptr_t>(out) % 16 || stride_q % 8 || stride_k % 8 || stride_v % 8 || stride_out % 8)
+      reinterpret_cast<uintptr_t>(out) % 16)
     return kInvalid;
-  if (batch > 1 && stride_out < (int64_t)m_vec * V * 64) return kInvalid;  // (the batch elements' outputs must not overlap)
   sspmm::AttentionArgs a{};
   a.m_vec = m_vec;
   a.n_keys = n_keys;
-  a.batch = batch;
+  a.batch = batch * heads;
+  a.heads = heads;
   a.row_indices = row_indices;
   a.row_offsets = row_offsets;
   a.col_idx = col_idx;
@@ -292,8 +303,25 @@ int sspmm_sparse_attention_f16(int batch, int m_vec, int V, int F, int n_keys, c
   a.stride_k = stride_k;
   a.stride_v = stride_v;
   a.stride_out = stride_out;
+  a.head_q = head_q;
+  a.head_k = head_k;
+  a.head_v = head_v;
+  a.head_out = head_out;
+  a.ld_q = ld_q;
+  a.ld_k = ld_k;
+  a.ld_v = ld_v;
+  a.ld_out = ld_out;
   a.scale = scale;
   return (int)sspmm::launch_sparse_attention(a, V, static_cast<hipStream_t>(hip_stream));
+}
+
+int sspmm_sparse_attention_f16(int batch, int m_vec, int V, int F, int n_keys, const int32_t *row_indices,
+                               const int32_t *row_offsets, const int32_t *col_idx, const sspmm_half_t *q, int64_t stride_q,
+                               const sspmm_half_t *k, int64_t stride_k, const sspmm_half_t *v, int64_t stride_v, float scale,
+                               sspmm_half_t *out, int64_t stride_out, void *hip_stream) {
+  if (batch > 1 && stride_out < (int64_t)m_vec * V * 64) return kInvalid;  // (the batch elements' outputs must not overlap)
+  return sspmm_sparse_attention_heads_f16(batch, 1, m_vec, V, F, n_keys, row_indices, row_offsets, col_idx, q, stride_q, 0, 64,
+                                          k, stride_k, 0, 64, v, stride_v, 0, 64, scale, out, stride_out, 0, 64, hip_stream);
 }
 
 size_t svc_workspace_bytes(int M, int64_t nnz, int V) {

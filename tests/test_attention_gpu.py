@@ -179,6 +179,27 @@ def test_one_launch_attention_of_a_single_key_returns_its_value_row(built_librar
         assert np.array_equal(got[:, i * V:(i + 1) * V], np.repeat(v[:, cols[i]][:, None], V, axis=1))
 
 
+@pytest.mark.parametrize("V", [8, 16])
+def test_packed_heads_give_the_bits_of_the_copied_out_heads(built_library, V):
+    """The launch on a fused projection [seq, batch, 3 * heads * 64] against the same launch on q, k and v copied out
+    into [batch * heads, seq, 64] as the reference's module lays them out (spattention.py:151-157, 181-184)."""
+    seq, bsz, heads = 192, 3, 5
+    E = heads * 64
+    vs = _pattern(seq // V, seq, V, 0.7, seed=21)
+    off, col = dev(vs.row_offsets), dev(vs.col_idx)
+    g = torch.Generator("cuda").manual_seed(22)
+    qkv = torch.randn(seq, bsz, 3 * E, device="cuda", generator=g).half()
+    got = sspmm_amd.sparse_attention_packed(None, off, col, qkv, heads, 0.125, V)
+    torch.cuda.synchronize()
+    q, k, v = (t.contiguous().view(seq, bsz * heads, 64).transpose(0, 1).contiguous() for t in qkv.chunk(3, dim=-1))
+    want = sspmm_amd.fused_sparse_attention(None, off, col, q, k, v, 0.125, V)
+    want = want.transpose(0, 1).contiguous().view(seq, bsz, E)
+    assert got.shape == (seq, bsz, E)
+    assert torch.equal(got, want)
+    with pytest.raises(ValueError):
+        sspmm_amd.sparse_attention_packed(None, off, col, qkv, heads + 1, 0.125, V)
+
+
 def test_argument_errors(built_library):
     off = torch.zeros(3, dtype=torch.int32, device="cuda")
     col = torch.zeros(0, dtype=torch.int32, device="cuda")

@@ -75,6 +75,11 @@ def test_argument_errors_without_device_work(built_library):
     for bad_scale in (0.0, -0.125, float("nan"), float("inf")):
         assert sa(scale=bad_scale) == 1
     assert L.sspmm_sparse_attention_f16(0, 4, 8, 64, 8, None, None, None, None, 0, None, 0, None, 0, 0.125, None, 0, None) == 0
+    # ... and its form for heads that lie side by side: no heads, a row pitch below the head's width, a pitch that is not a
+    # multiple of 8, a negative stride
+    sh = lambda heads=2, ld=384, head=64, stride=128: L.sspmm_sparse_attention_heads_f16(  # noqa: E731
+        1, heads, 1, 8, 64, 8, None, 16, 16, 16, stride, head, ld, 16, stride, head, ld, 16, stride, head, ld, 0.125, 16, stride, head, ld, None)
+    assert sh(heads=0) == 1 and sh(ld=32) == 1 and sh(ld=388) == 1 and sh(stride=-128) == 1 and sh(ld=1 << 23) == 1
     assert L.svc_workspace_bytes(16, 100, 8) >= 100 * 8
     assert b"invalid" in L.sspmm_error_string(1)
     assert L.sspmm_error_string(0) == b"success"

@@ -187,6 +187,16 @@ int sspmm_noalloc_f16_f32(int m_vec, int V, int N, int K, const int32_t *row_off
  */
 int sspmm_sorted_row_swizzle(int m_vec, const int32_t *row_offsets, int32_t *row_indices, void *hip_stream);
 
+/*
+ * The same order (ties included) for patterns of very many vector-rows: the entry above compares every pair of
+ * rows in one launch, which suits the 10^2 - 10^4 vector-rows of this format's matrices; this one sorts by
+ * length with a stable radix sort in `workspace` (at least sspmm_sorted_row_swizzle_workspace_bytes(m_vec)
+ * bytes of device memory, 256-byte aligned), linear in m_vec, several launches on `hip_stream`.
+ */
+size_t sspmm_sorted_row_swizzle_workspace_bytes(int m_vec);
+int sspmm_sorted_row_swizzle_ws(int m_vec, const int32_t *row_offsets, int32_t *row_indices, void *workspace,
+                                size_t workspace_bytes, void *hip_stream);
+
 /* ------------------------------------------------------------------------------------------
  * The two steps either side of the batched SpMM in the reference's sparse attention block
  * (end2end/sspmm_e2e/spattention.py:167-179), on the same pattern arrays.

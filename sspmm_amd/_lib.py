@@ -24,6 +24,8 @@ SIGNATURES = {
     "sspmm_batched_f16_f32": (_int, [_int] * 5 + [_vp, _vp, _vp, _vp, _i64, _vp, _i64, _vp, _i64, _vp]),
     "sspmm_noalloc_f16_f32": (_int, [_int] * 4 + [_vp] * 6),
     "sspmm_sorted_row_swizzle": (_int, [_int, _vp, _vp, _vp]),
+    "sspmm_sorted_row_swizzle_workspace_bytes": (ctypes.c_size_t, [_int]),
+    "sspmm_sorted_row_swizzle_ws": (_int, [_int, _vp, _vp, _vp, ctypes.c_size_t, _vp]),
     "sspmm_plan_create": (_int, [_int, _int, _int, _vp, _int, _int, _int, _vp, ctypes.POINTER(ctypes.c_void_p)]),
     "sspmm_plan_destroy": (_int, [_vp]),
     "sspmm_plan_info": (_int, [_vp, ctypes.POINTER(ctypes.c_int64)]),

@@ -195,6 +195,19 @@ int sspmm_sorted_row_swizzle(int m_vec, const int32_t *row_offsets, int32_t *row
   return (int)sspmm::launch_sorted_row_swizzle(m_vec, row_offsets, row_indices, static_cast<hipStream_t>(hip_stream));
 }
 
+size_t sspmm_sorted_row_swizzle_workspace_bytes(int m_vec) {
+  return m_vec < 0 ? 0 : sspmm::sorted_row_swizzle_workspace_bytes(m_vec);
+}
+
+int sspmm_sorted_row_swizzle_ws(int m_vec, const int32_t *row_offsets, int32_t *row_indices, void *workspace,
+                                size_t workspace_bytes, void *hip_stream) {
+  if (m_vec < 0) return kInvalid;
+  if (m_vec == 0) return 0;
+  if (!row_offsets || !row_indices || !workspace) return kInvalid;
+  return (int)sspmm::launch_sorted_row_swizzle_ws(m_vec, row_offsets, row_indices, workspace, workspace_bytes,
+                                                  static_cast<hipStream_t>(hip_stream));
+}
+
 int sspmm_sddmm_batched_f16(int batch, int m_vec, int V, int F, int n_rhs, const int32_t *row_indices,
                             const int32_t *row_offsets, const int32_t *col_idx, const sspmm_half_t *lhs,
                             int64_t stride_lhs, const sspmm_half_t *rhs, int64_t stride_rhs, sspmm_half_t *out_values,

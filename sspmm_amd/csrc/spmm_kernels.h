@@ -55,6 +55,10 @@ int kernel_override();
 
 hipError_t launch_sorted_row_swizzle(int m_vec, const int32_t *row_offsets, int32_t *row_indices,
                                      hipStream_t stream);
+// The same order from a stable radix sort in caller-provided scratch memory (linear in m_vec).
+size_t sorted_row_swizzle_workspace_bytes(int m_vec);
+hipError_t launch_sorted_row_swizzle_ws(int m_vec, const int32_t *row_offsets, int32_t *row_indices, void *workspace,
+                                        size_t workspace_bytes, hipStream_t stream);
 
 }  // namespace sspmm
 #endif

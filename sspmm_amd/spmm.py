@@ -128,6 +128,9 @@ def bspmm(row_indices, row_offsets, column_indices, values, rhs_matrix, vec_leng
     return out
 
 
+SWIZZLE_SORT_FROM = 4096  # vector-rows; measured crossover of the two entry points on an MI355X (13 against 17 us at 2048, 48 against 26 at 8192)
+
+
 def sorted_row_swizzle(row_offsets):
     """Vector-rows ordered by descending length (reference SortedRowSwizzle,
     SSpMM/include/bm_test_utils.h:210-225), computed on the GPU."""
@@ -135,7 +138,13 @@ def sorted_row_swizzle(row_offsets):
         raise TypeError("row_offsets must be an int32 GPU tensor")
     m_vec = row_offsets.numel() - 1
     out = torch.empty(max(m_vec, 0), dtype=torch.int32, device=row_offsets.device)
+    L = _lib.lib()
     with torch.cuda.device(row_offsets.device):
-        rc = _lib.lib().sspmm_sorted_row_swizzle(m_vec, _ptr(row_offsets), _ptr(out), _stream())
+        if m_vec > SWIZZLE_SORT_FROM:
+            # every pair of rows compared in one launch grows with the square of m_vec: a radix sort from here on
+            ws = torch.empty(L.sspmm_sorted_row_swizzle_workspace_bytes(m_vec), dtype=torch.uint8, device=row_offsets.device)
+            rc = L.sspmm_sorted_row_swizzle_ws(m_vec, _ptr(row_offsets), _ptr(out), _ptr(ws), ws.numel(), _stream())
+        else:
+            rc = L.sspmm_sorted_row_swizzle(m_vec, _ptr(row_offsets), _ptr(out), _stream())
     _lib.check(rc, "sspmm_sorted_row_swizzle")
     return out

@@ -469,6 +469,24 @@ def test_row_swizzle_matches_oracle(oracle, built_library):
         off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
         got = sspmm_amd.sorted_row_swizzle(dev(off)).cpu().numpy()
         assert np.array_equal(got, oracle.sorted_row_swizzle(off))
+    # the radix-sort entry gives the same order, ties included; the wrapper takes it for many rows
+    from sspmm_amd import _lib
+    from sspmm_amd.spmm import SWIZZLE_SORT_FROM
+    L = _lib.lib()
+    for m_vec in [1, 300, 70000]:
+        lens = rng.integers(0, 40 if m_vec < 1000 else 20000, m_vec)
+        lens[::7] = 13  # plenty of ties
+        off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        d_off = dev(off)
+        out = torch.empty(m_vec, dtype=torch.int32, device="cuda")
+        ws = torch.empty(L.sspmm_sorted_row_swizzle_workspace_bytes(m_vec), dtype=torch.uint8, device="cuda")
+        assert L.sspmm_sorted_row_swizzle_ws(m_vec, d_off.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel() - 1, None) != 0
+        assert L.sspmm_sorted_row_swizzle_ws(m_vec, d_off.data_ptr(), out.data_ptr(), ws.data_ptr(), ws.numel(), None) == 0
+        torch.cuda.synchronize()
+        want = oracle.sorted_row_swizzle(off)
+        assert np.array_equal(out.cpu().numpy(), want)
+        if m_vec > SWIZZLE_SORT_FROM:
+            assert np.array_equal(sspmm_amd.sorted_row_swizzle(d_off).cpu().numpy(), want)
 
 
 @pytest.mark.parametrize("V", [8, 16])

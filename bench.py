@@ -659,7 +659,7 @@ def run_cfg5_layer(L, torch, synth, st, wu):
             "projections": per}
 
 
-def run_attention_forward(torch, sparsity, bsz, st, wu, seq=4096, heads=4, embed=256, mlp=1024):
+def run_attention_forward(torch, sparsity, bsz, seq, heads, embed, st, wu, mlp=1024):
     """The forward pass of the reference's end-to-end sparse attention model (end2end/sspmm_e2e/end_to_end.py:123-203:
     4 blocks, fp16, V = 8 masks drawn at random per block) at the configurations its results are published for,
     timed with a device synchronisation either side (the reference's loop has none, end_to_end.py:198-203), eager
@@ -667,7 +667,7 @@ def run_attention_forward(torch, sparsity, bsz, st, wu, seq=4096, heads=4, embed
     "PyTorch" column)."""
     from sspmm_amd.attention import SparseAttentionEncoder
     torch.manual_seed(0)
-    model = SparseAttentionEncoder(257, embed, heads, sparsity, seq, mlp, mlp, vec_length=8, layers=4, seed=20).cuda().half().eval()
+    model = SparseAttentionEncoder(257, embed, heads, sparsity, seq, mlp, 2, vec_length=8, layers=4, seed=20).cuda().half().eval()
     tokens = torch.randint(0, 257, (bsz, seq), device="cuda")
 
     def dense_forward():
@@ -746,7 +746,9 @@ def run_reorder(L, torch, synth, sspmm_amd):
 
 
 ATTENTION = "sparse_attention_seq4096_d64_v8_s0.9_heads48"
-ATTENTION_FORWARD = {"sparse_attention_forward_seq4096_h4_e256_s%g_b%d_l4" % (s, b): (s, b) for s in (0.9, 0.95) for b in (2, 8)}
+# the eight published configurations of the reference's end-to-end model (mask sparsity, sequence, heads / embed), batch 2 and 8
+ATTENTION_FORWARD = {"sparse_attention_forward_seq%d_h%d_e%d_s%g_b%d_l4" % (seq, h, e, s, b): (s, b, seq, h, e)
+                     for s in (0.9, 0.95) for seq in (4096, 8192) for (h, e) in ((4, 256), (8, 512)) for b in (2, 8)}
 GROUPS = ["cfg1_rowmerge_then_spmm_512x512", "cfg4", "svc_batched_dlmc_shapes", *ATTENTION_FORWARD, "cfg5_encoder_layer_v16_s0.9_tokens4096", ATTENTION,
           "reorder_clustered_16384_v8", "headline_batched_cold"]
 
@@ -797,7 +799,8 @@ def run_extra(name, env):
     if name == "cfg4":
         return run_cfg4(L, torch, synth, sspmm_amd, O, st, wu)
     if name in ATTENTION_FORWARD:
-        return {name: run_attention_forward(torch, *ATTENTION_FORWARD[name], st=min(st, 50), wu=min(wu, 10))}
+        return {name: run_attention_forward(torch, *ATTENTION_FORWARD[name], st=min(st, 50) if ATTENTION_FORWARD[name][2] <= 4096 else min(st, 20),
+                                            wu=min(wu, 10))}
     if name == "svc_batched_dlmc_shapes":
         return {name: run_svc_batched(L, torch, synth, sspmm_amd, O)}
     if name == "cfg5_encoder_layer_v16_s0.9_tokens4096":

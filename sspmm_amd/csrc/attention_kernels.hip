@@ -397,7 +397,6 @@ hipError_t launch_softmax(const SoftmaxArgs &a, int V, hipStream_t stream) {
 // the registers that allows measured 2-7 % faster than three, and four (which spills) 75 % slower.
 namespace {
 
-typedef __attribute__((address_space(3))) short lds_short4 __attribute__((ext_vector_type(4)));
 typedef short shortx4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ uintx2 lds_read_tr(const unsigned char *p) {

@@ -245,6 +245,10 @@ def attention_block(torch, synth, sspmm_amd, st, wu):
     chain = sspmm_amd.bspmm(None, offA, colA, pA, vA, VA).float()
     one = sspmm_amd.fused_sparse_attention(None, offA, colA, qA, kA, vA, 0.125, VA).float()
     by_one = bA * 4 * 2 * seqA * dA + 4 * nvA + 4 * (mk_a.m_vec + 1)   # q, k, v read and the output written, once each
+    # the same block on a V = 16 mask of the same sparsity: every gathered row of k and v serves 16 queries instead of 8
+    mk16 = synth.vector_sparse(seqA, seqA, 16, 0.9, seed=7)
+    off16, col16 = torch.from_numpy(mk16.row_offsets).cuda(), torch.from_numpy(mk16.col_idx).cuda()
+    t_one16 = time_launches(lambda: sspmm_amd.fused_sparse_attention(None, off16, col16, qA, kA, vA, 0.125, 16), st, wu)
     by_sddmm = bA * (2 * seqA * dA * 2 + 2 * nvA * VA) + 4 * nvA + 4 * (mk_a.m_vec + 1)
     by_soft = bA * 2 * 2 * nvA * VA + 4 * (mk_a.m_vec + 1)
     by_av = bA * (2 * nvA * VA + 2 * seqA * dA + 2 * seqA * dA) + 4 * nvA + 4 * (mk_a.m_vec + 1)
@@ -258,6 +262,7 @@ def attention_block(torch, synth, sspmm_amd, st, wu):
         # rows of k and of v fetched from the caches, 128 bytes per stored vector each: what bounds the launch
         "one_launch_gathered_tb_per_s": bA * 2 * nvA * 2 * dA / t_one / 1e9,
         "one_launch_speedup_vs_three": (t_sddmm + t_soft + t_av) / t_one,
+        "one_launch_v16_mask_ms": t_one16, "one_launch_v16_mask_gathered_tb_per_s": bA * 2 * mk16.col_idx.size * 2 * dA / t_one16 / 1e9,
         "one_launch_max_rel_err_vs_three": float((one - chain).abs().max() / chain.abs().max()),
     }
     del qA, kA, vA, wA, pA

@@ -394,7 +394,10 @@ hipError_t launch_softmax(const SoftmaxArgs &a, int V, hipStream_t stream) {
 // after it); sums are fp32 throughout.
 // The launch is bound by the stream of gathered rows from the L2 into the CUs (256 bytes per stored vector and batch
 // element; measured 21 TB/s on 4096 keys, 90 % masked, 48 heads), not by waves in flight: two waves per SIMD with
-// the registers that allows measured 2-7 % faster than three, and four (which spills) 75 % slower.
+// the registers that allows measured 2-7 % faster than three, and four (which spills) 75 % slower.  Column indices
+// fetched in blocks of 64 with one coalesced load and handed out with lane permutes, as the sddmm kernel does, take
+// 11 % of the address unit's work away and cost 10 % in time here (124 -> 137 us): the permutes queue in the LDS pipe
+// behind the stage's writes and reads.
 namespace {
 
 typedef short shortx4 __attribute__((ext_vector_type(4)));

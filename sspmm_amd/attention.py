@@ -104,6 +104,12 @@ def fused_sparse_attention(row_indices, row_offsets, column_indices, q, k, v, sc
     return out
 
 
+def packed_attention_fits(seq, bsz, three_e):
+    """Whether `sparse_attention_packed` takes a projection of this shape: the rows of one (batch element, head) pair,
+    which lie `bsz * three_e` elements apart, must span less than 2 GiB (one 32-bit buffer descriptor)."""
+    return (seq - 1) * bsz * three_e * 2 < (1 << 31) - 256 and bsz * three_e < (1 << 23) and seq < (1 << 24)
+
+
 def sparse_attention_packed(row_indices, row_offsets, column_indices, qkv, num_heads, scaling, vec_length):
     """Multi-head attention on a vector-sparse mask straight from a fused projection: qkv [seq, batch, 3 * embed] (q,
     k and v side by side in the last dimension, heads of 64 features side by side in each) -> [seq, batch, embed],
@@ -188,7 +194,7 @@ class SparseAttentionBlock(torch.nn.Module):
         h, d = self.num_heads, E // self.num_heads
         scaling = float(d) ** -0.5
         qkv = self.in_proj(x)
-        if dense_mask is None and d == 64 and qkv.dtype == torch.float16:
+        if dense_mask is None and d == 64 and qkv.dtype == torch.float16 and packed_attention_fits(seq, bsz, 3 * E):
             # the heads are read where the projection left them and written where the output projection wants them
             return self.out_proj(sparse_attention_packed(self.row_indices, self.row_offsets, self.column_indices,
                                                          qkv.contiguous(), h, scaling, self.vec_length))

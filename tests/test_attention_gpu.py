@@ -198,6 +198,8 @@ def test_packed_heads_give_the_bits_of_the_copied_out_heads(built_library, V):
     assert torch.equal(got, want)
     with pytest.raises(ValueError):
         sspmm_amd.sparse_attention_packed(None, off, col, qkv, heads + 1, 0.125, V)
+    from sspmm_amd.attention import packed_attention_fits
+    assert packed_attention_fits(8192, 8, 3 * 512) and not packed_attention_fits(16384, 32, 3 * 1024)
 
 
 def test_argument_errors(built_library):

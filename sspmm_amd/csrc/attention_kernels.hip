@@ -397,7 +397,9 @@ hipError_t launch_softmax(const SoftmaxArgs &a, int V, hipStream_t stream) {
 // the registers that allows measured 2-7 % faster than three, and four (which spills) 75 % slower.  Column indices
 // fetched in blocks of 64 with one coalesced load and handed out with lane permutes, as the sddmm kernel does, take
 // 11 % of the address unit's work away and cost 10 % in time here (124 -> 137 us): the permutes queue in the LDS pipe
-// behind the stage's writes and reads.
+// behind the stage's writes and reads.  One index per lane of a quad (a 4-byte load) passed round with DPP moves
+// measures the same as the 16-byte load, run against it on one box (128.6 and 128.7 us): it is the 64 bytes a
+// cycle of the cache's data path that bound the launch, not the count of load instructions.
 namespace {
 
 typedef short shortx4 __attribute__((ext_vector_type(4)));

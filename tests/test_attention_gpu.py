@@ -167,6 +167,21 @@ def test_one_launch_attention_row_lengths_permutation_and_large_scores(built_lib
     assert (one.float() - chain.float()).abs().max().item() <= 3e-2
 
 
+@pytest.mark.parametrize("d", [32, 128])
+def test_heads_of_other_widths_take_the_three_operators(built_library, d):
+    """`sparse_attention` with nothing forced: heads that are not 64 wide run the chain, and `fused=True` says so."""
+    V, seq, batch = 8, 128, 2
+    vs = _pattern(seq // V, seq, V, 0.75, seed=31)
+    off, col = dev(vs.row_offsets), dev(vs.col_idx)
+    g = torch.Generator("cuda").manual_seed(32)
+    q, k, v = (torch.randn(batch, seq, d, device="cuda", generator=g).half() for _ in range(3))
+    out = sspmm_amd.sparse_attention(None, off, col, q, k, v, d ** -0.5, V)
+    want = _dense_attention(vs.row_offsets, vs.col_idx, V, *(t.cpu().numpy() for t in (q, k, v)), d ** -0.5)
+    assert np.abs(out.float().cpu().numpy() - want).max() <= 1e-2
+    with pytest.raises(ValueError):
+        sspmm_amd.sparse_attention(None, off, col, q, k, v, d ** -0.5, V, fused=True)
+
+
 def test_one_launch_attention_of_a_single_key_returns_its_value_row(built_library):
     """A query that attends to one key gets that row of v back exactly (probability one, fp16 in and out)."""
     V, n_keys, m_vec = 8, 50, 5

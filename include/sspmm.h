@@ -232,10 +232,10 @@ int sspmm_softmax_batched_f16(int batch, int m_vec, int V, const int32_t *row_in
                               void *hip_stream);
 
 /*
- * The three steps of the attention block in one launch, for heads of F = 64 features:
+ * The three steps of the attention block in one launch, for heads of F = 32, 64 or 128 features:
  * out[b, i*V + v, :] = sum_j softmax_j(scale * q[b, i*V + v, :] . k[b, col_j, :]) * v[b, col_j, :] over the
- * vectors j of vector-row i; a row with no stored vectors gives zeros.  q, out: [batch][m_vec*V][64];
- * k, v: [batch][n_keys][64]; strides in elements.  Stands for the chain bsddmm -> bcsr_softmax -> bspmm of
+ * vectors j of vector-row i; a row with no stored vectors gives zeros.  q, out: [batch][m_vec*V][F];
+ * k, v: [batch][n_keys][F]; strides in elements.  Stands for the chain bsddmm -> bcsr_softmax -> bspmm of
  * reference end2end/sspmm_e2e/spattention.py:167-179 (which has no single operator for it): the scores and the
  * probabilities stay on the CU, in fp32, and the probabilities enter the product rounded to fp16 before the
  * division by their sum, so results differ from the chain's by fp16 rounding, not bit for bit.
@@ -250,9 +250,9 @@ int sspmm_sparse_attention_f16(int batch, int m_vec, int V, int F, int n_keys, c
  * The same launch on operands that hold several heads side by side, so that a model's fused projection can be used
  * where it lies: row r of (batch element e, head h) starts at x + e*stride_x + h*head_x + r*ld_x (elements; 64
  * features each), for x = q, k, v and out.  The mask is shared by all batch * heads pairs.  For the output of a
- * projection [seq][batch][3 * heads * 64] (reference spattention.py:151-157 copies q, k and v out of it and into
- * [batch * heads][seq][64] first): q = qkv, k = qkv + heads*64, v = qkv + 2*heads*64, stride = 3*heads*64,
- * head = 64, ld = batch*3*heads*64.  Strides non-negative multiples of 8, ld >= 64; the caller sees to it that no two
+ * projection [seq][batch][3 * heads * F] (reference spattention.py:151-157 copies q, k and v out of it and into
+ * [batch * heads][seq][F] first): q = qkv, k = qkv + heads*F, v = qkv + 2*heads*F, stride = 3*heads*F,
+ * head = F, ld = batch*3*heads*F.  Strides non-negative multiples of 8, ld >= F; the caller sees to it that no two
  * rows of out overlap.  No counterpart in the reference.
  */
 int sspmm_sparse_attention_heads_f16(int batch, int heads, int m_vec, int V, int F, int n_keys, const int32_t *row_indices,

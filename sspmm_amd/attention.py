@@ -76,8 +76,11 @@ def csr_softmax(row_indices, row_offsets, values, scaler, vec_length):
     return bcsr_softmax(row_indices, row_offsets, values, scaler, vec_length, 1)
 
 
+FUSED_HEAD_WIDTHS = (32, 64, 128)
+
+
 def fused_sparse_attention(row_indices, row_offsets, column_indices, q, k, v, scaling, vec_length):
-    """The block's three steps in one launch (heads of 64 features only): scores and probabilities never leave the
+    """The block's three steps in one launch (heads of 32, 64 or 128 features): scores and probabilities never leave the
     chip.  Same arguments and result shape as `sparse_attention`; differs from the three-step chain by fp16 rounding
     of intermediate values only (the chain rounds the scores and the normalised probabilities to fp16, this rounds
     the probabilities before the division by their sum)."""
@@ -85,8 +88,8 @@ def fused_sparse_attention(row_indices, row_offsets, column_indices, q, k, v, sc
     for name, t in (("q", q), ("k", k), ("v", v)):
         _check_half(name, t)
     m, d, n = q.size(-2), q.size(-1), k.size(-2)
-    if d != 64 or k.size(-1) != 64 or v.size(-1) != 64:
-        raise ValueError("fused_sparse_attention takes heads of 64 features")
+    if d not in FUSED_HEAD_WIDTHS or k.size(-1) != d or v.size(-1) != d:
+        raise ValueError("fused_sparse_attention takes heads of 32, 64 or 128 features, the same for q, k and v")
     if v.size(-2) != n:
         raise ValueError("k and v must have the same number of rows")
     m_vec = row_offsets.numel() - 1
@@ -112,15 +115,16 @@ def packed_attention_fits(seq, bsz, three_e):
 
 def sparse_attention_packed(row_indices, row_offsets, column_indices, qkv, num_heads, scaling, vec_length):
     """Multi-head attention on a vector-sparse mask straight from a fused projection: qkv [seq, batch, 3 * embed] (q,
-    k and v side by side in the last dimension, heads of 64 features side by side in each) -> [seq, batch, embed],
+    k and v side by side in the last dimension, heads of 32, 64 or 128 features side by side in each) -> [seq, batch, embed],
     in one launch and without the copies into [batch * heads, seq, 64] and back that the reference's module makes
     around its three operators (spattention.py:151-157 and 181-184)."""
     _check_pattern(row_indices, row_offsets, column_indices, vec_length)
     _check_half("qkv", qkv)
-    if qkv.dim() != 3 or qkv.size(-1) != 3 * num_heads * 64:
-        raise ValueError("qkv must be [seq, batch, 3 * num_heads * 64]")
+    if qkv.dim() != 3 or qkv.size(-1) % (3 * num_heads) or qkv.size(-1) // (3 * num_heads) not in FUSED_HEAD_WIDTHS:
+        raise ValueError("qkv must be [seq, batch, 3 * num_heads * d] with d = 32, 64 or 128")
     seq, bsz, three_e = qkv.shape
     e = three_e // 3
+    d = e // num_heads
     m_vec = row_offsets.numel() - 1
     if seq != m_vec * vec_length:
         raise ValueError("qkv must have m_vec * vec_length = %d rows, got %d" % (m_vec * vec_length, seq))
@@ -128,9 +132,9 @@ def sparse_attention_packed(row_indices, row_offsets, column_indices, qkv, num_h
     base, ld = qkv.data_ptr(), bsz * three_e
     with torch.cuda.device(qkv.device):
         rc = _lib.lib().sspmm_sparse_attention_heads_f16(
-            bsz, num_heads, m_vec, vec_length, 64, seq, _ptr(row_indices), _ptr(row_offsets), _ptr(column_indices),
-            base, three_e, 64, ld, base + 2 * e, three_e, 64, ld, base + 4 * e, three_e, 64, ld, float(scaling),
-            _ptr(out), e, 64, bsz * e, _stream())
+            bsz, num_heads, m_vec, vec_length, d, seq, _ptr(row_indices), _ptr(row_offsets), _ptr(column_indices),
+            base, three_e, d, ld, base + 2 * e, three_e, d, ld, base + 4 * e, three_e, d, ld, float(scaling),
+            _ptr(out), e, d, bsz * e, _stream())
     _lib.check(rc, "sspmm_sparse_attention_heads")
     return out
 
@@ -139,9 +143,9 @@ def sparse_attention(row_indices, row_offsets, column_indices, q, k, v, scaling,
     """softmax(mask(q k^T) * scaling) v on a vector-sparse mask shared by the batch:
     q [batch, tgt, d], k [batch, src, d], v [batch, src, d_v] -> fp16 [batch, tgt, d_v]; the three
     steps of the reference's block (spattention.py:167-179).  fused: None = one launch where the shapes allow it
-    (d = d_v = 64), False = always the three operators, True = one launch or an error."""
+    (d = d_v = 32, 64 or 128), False = always the three operators, True = one launch or an error."""
     if fused is None:
-        fused = q.size(-1) == 64 and v.size(-1) == 64 and row_offsets.numel() > 1 and q.numel() > 0
+        fused = q.size(-1) in FUSED_HEAD_WIDTHS and v.size(-1) == q.size(-1) and row_offsets.numel() > 1 and q.numel() > 0
     if fused:
         return fused_sparse_attention(row_indices, row_offsets, column_indices, q, k, v, scaling, vec_length)
     w = bsddmm(row_indices, row_offsets, column_indices, q, k, vec_length)
@@ -194,7 +198,7 @@ class SparseAttentionBlock(torch.nn.Module):
         h, d = self.num_heads, E // self.num_heads
         scaling = float(d) ** -0.5
         qkv = self.in_proj(x)
-        if dense_mask is None and d == 64 and qkv.dtype == torch.float16 and packed_attention_fits(seq, bsz, 3 * E):
+        if dense_mask is None and d in FUSED_HEAD_WIDTHS and qkv.dtype == torch.float16 and packed_attention_fits(seq, bsz, 3 * E):
             # the heads are read where the projection left them and written where the output projection wants them
             return self.out_proj(sparse_attention_packed(self.row_indices, self.row_offsets, self.column_indices,
                                                          qkv.contiguous(), h, scaling, self.vec_length))

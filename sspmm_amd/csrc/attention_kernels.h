@@ -37,7 +37,7 @@ struct AttentionArgs {
   const int32_t *row_indices;  // nullable
   const int32_t *row_offsets;
   const int32_t *col_idx;
-  const uint16_t *q;  // row r of (element e, head h) at q + e * stride_q + h * head_q + r * ld_q, 64 features each
+  const uint16_t *q;  // row r of (element e, head h) at q + e * stride_q + h * head_q + r * ld_q, F features each
   const uint16_t *k;  // n_keys rows per (element, head), addressed the same way
   const uint16_t *v;
   uint16_t *out;      // m_vec * V rows per (element, head)
@@ -51,9 +51,9 @@ struct AttentionArgs {
 // V must be 8 or 16; F a multiple of 8 up to 256; 16-byte aligned operands and strides.
 hipError_t launch_sddmm(const SddmmArgs &args, int V, hipStream_t stream);
 hipError_t launch_softmax(const SoftmaxArgs &args, int V, hipStream_t stream);
-// sddmm, softmax and the product with v in one kernel, for 64 features per row of q, k and v.  16-byte aligned
+// sddmm, softmax and the product with v in one kernel, for F = 32, 64 or 128 features per row of q, k and v.  16-byte aligned
 // operands and strides; the rows of one (element, head) span less than 2 GiB.
-hipError_t launch_sparse_attention(const AttentionArgs &args, int V, hipStream_t stream);
+hipError_t launch_sparse_attention(const AttentionArgs &args, int V, int F, hipStream_t stream);
 
 }  // namespace sspmm
 #endif

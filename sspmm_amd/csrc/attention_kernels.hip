@@ -373,7 +373,8 @@ hipError_t launch_softmax(const SoftmaxArgs &a, int V, hipStream_t stream) {
 }
 
 // ---------------------------------------------------------------------- the three steps in one
-// softmax(mask(q k^T) * scale) v per vector-row without the scores ever leaving the CU, for heads of 64 features
+// softmax(mask(q k^T) * scale) v per vector-row without the scores ever leaving the CU, for heads of 32, 64 or 128
+// features (described for 64)
 // (the three launches of the block, reference end2end/sspmm_e2e/spattention.py:167-179, move the scores and the
 // probabilities through memory twice each: 2 * V bytes per stored vector four times over).
 //
@@ -423,97 +424,117 @@ __device__ __forceinline__ float quad_rows_sum(float x) {
   return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
-static constexpr uint32_t kAttnPitch = 144;  // bytes per staged row: 64 features and 16 of padding
 
 }  // namespace
 
-template <int V>
+// F: features per row of q, k and v (32, 64 or 128).  A row is F * 2 bytes = LPR 16-byte pieces, a load instruction
+// brings 64 / LPR rows, a step of 32 rows takes L = LPR / 2 of them per operand; lane (jr, pc) fetches piece pc of the
+// rows of k slots L * jr .. L * jr + L - 1, whose column indices it reads as L consecutive ints.
+template <int V, int F>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void sparse_attention_kernel(const AttentionArgs p) {
-  __shared__ __align__(16) unsigned char stage_k[32 * kAttnPitch];
-  __shared__ __align__(16) unsigned char stage_v[32 * kAttnPitch];
+  constexpr int LPR = F / 8, L = LPR / 2, NC = F / 32, NT = F / 16;
+  constexpr uint32_t kRowBytes = F * 2u, kPitch = kRowBytes + 16u;  // staged rows padded by 16 bytes against bank conflicts
+  __shared__ __align__(16) unsigned char stage_k[32 * kPitch];
+  __shared__ __align__(16) unsigned char stage_v[32 * kPitch];
   const uint32_t w = xcd_work_index(p.per_xcd);
   if (w >= p.total_work) return;
   const uint32_t r = w % (uint32_t)p.m_vec;
   const uint32_t batch = w / (uint32_t)p.m_vec;
   const int row = __builtin_amdgcn_readfirstlane(p.row_indices ? p.row_indices[r] : (int)r);
   const int beg = p.row_offsets[row], end = p.row_offsets[row + 1];
-  const int lane = threadIdx.x, n = lane & 15, g = lane >> 4, j = lane >> 3, pc = lane & 7;
+  const int lane = threadIdx.x, n = lane & 15, g = lane >> 4, jr = lane / LPR, pc = lane % LPR;
 
   const uint32_t elem = batch / (uint32_t)p.heads, head = batch % (uint32_t)p.heads;
   uint16_t *out = p.out + (int64_t)elem * p.stride_out + (int64_t)head * p.head_out + ((int64_t)row * V + n) * p.ld_out + 4 * g;
   if (beg == end) {  // a query that attends to nothing: zeros, as the product with no stored vectors gives
     if (n < V) {
 #pragma unroll
-      for (int u = 0; u < 4; ++u) *reinterpret_cast<uintx2 *>(out + 16 * u) = uintx2{0u, 0u};
+      for (int u = 0; u < NT; ++u) *reinterpret_cast<uintx2 *>(out + 16 * u) = uintx2{0u, 0u};
     }
     return;
   }
-  // (descriptors end with the last row's 128 bytes; between the rows of a strided operand lies what belongs to other heads)
+  // (descriptors end with the last row's bytes; between the rows of a strided operand lies what belongs to other heads)
   const uint32_t q_row = (uint32_t)p.ld_q * 2u, k_row = (uint32_t)p.ld_k * 2u, v_row = (uint32_t)p.ld_v * 2u;
   const __amdgpu_buffer_rsrc_t srd_q = make_srd(p.q + (int64_t)elem * p.stride_q + (int64_t)head * p.head_q + (int64_t)row * V * p.ld_q,
-                                                (uint32_t)(V - 1) * q_row + 128u);
-  const uint32_t k_bytes = (uint32_t)(p.n_keys - 1) * k_row + 128u, v_bytes = (uint32_t)(p.n_keys - 1) * v_row + 128u;
+                                                (uint32_t)(V - 1) * q_row + kRowBytes);
+  const uint32_t k_bytes = (uint32_t)(p.n_keys - 1) * k_row + kRowBytes, v_bytes = (uint32_t)(p.n_keys - 1) * v_row + kRowBytes;
   const __amdgpu_buffer_rsrc_t srd_k = make_srd(p.k + (int64_t)elem * p.stride_k + (int64_t)head * p.head_k, k_bytes);
   const __amdgpu_buffer_rsrc_t srd_v = make_srd(p.v + (int64_t)elem * p.stride_v + (int64_t)head * p.head_v, v_bytes);
   const __amdgpu_buffer_rsrc_t srd_cols = make_srd(p.col_idx, (uint32_t)end * 4u);  // past the row: reads 0
 
-  half8 q[2];
+  half8 q[NC];
 #pragma unroll
-  for (int c = 0; c < 2; ++c)  // (rows past V: beyond the descriptor, zeros)
+  for (int c = 0; c < NC; ++c)  // (rows past V: beyond the descriptor, zeros)
     q[c] = __builtin_bit_cast(half8, __builtin_amdgcn_raw_buffer_load_b128(srd_q, n < V ? (uint32_t)n * q_row + (32u * c + 8u * g) * 2u : 0xfffffff0u, 0, 0));
 
-  unsigned char *const k_dst = stage_k + (uint32_t)(4 * j) * kAttnPitch + (uint32_t)pc * 16u;
-  unsigned char *const v_dst = stage_v + (uint32_t)(4 * j) * kAttnPitch + (uint32_t)pc * 16u;
-  const unsigned char *const k_rd = stage_k + (uint32_t)n * kAttnPitch + (uint32_t)g * 16u;
-  const unsigned char *const v_rd = stage_v + (uint32_t)(4 * g + (n >> 2)) * kAttnPitch + (uint32_t)(n & 3) * 8u;
+  unsigned char *const k_dst = stage_k + (uint32_t)(L * jr) * kPitch + (uint32_t)pc * 16u;
+  unsigned char *const v_dst = stage_v + (uint32_t)(L * jr) * kPitch + (uint32_t)pc * 16u;
+  const unsigned char *const k_rd = stage_k + (uint32_t)n * kPitch + (uint32_t)g * 16u;
+  const unsigned char *const v_rd = stage_v + (uint32_t)(4 * g + (n >> 2)) * kPitch + (uint32_t)(n & 3) * 8u;
   const uint32_t piece_off = (uint32_t)pc * 16u;
   const float scale2 = p.scale * 1.4426950408889634f;
 
+  struct Head {
+    uint32_t c[L];
+  };
   struct Body {
-    uintx4 k[4], v[4];
+    uintx4 k[L], v[L];
   };
   const auto load_head = [&](int kc) {
-    return __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_cols, (kc + 4 * j) * 4, 0, 0));
-  };
-  const auto load_body = [&](Body &b, const uintx4 &cols, int kc) {
-    uint32_t ok[4], ov[4];
+    Head h;
+    const int at = (kc + L * jr) * 4;
+    if (L == 2) {
+      const uintx2 x = __builtin_bit_cast(uintx2, __builtin_amdgcn_raw_buffer_load_b64(srd_cols, at, 0, 0));
+      h.c[0] = x[0]; h.c[1] = x[1];
+    } else {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      ok[i] = __umul24(cols[i], k_row) + piece_off;  // (both factors below 2^24: the launcher's caller checks the row pitch)
-      ov[i] = __umul24(cols[i], v_row) + piece_off;
+      for (int i = 0; i < L; i += 4) {
+        const uintx4 x = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_cols, at + 4 * i, 0, 0));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) h.c[(i + e) % L] = x[e];
+      }
+    }
+    return h;
+  };
+  const auto load_body = [&](Body &b, const Head &h, int kc) {
+    uint32_t ok[L], ov[L];
+#pragma unroll
+    for (int i = 0; i < L; ++i) {
+      ok[i] = __umul24(h.c[i], k_row) + piece_off;  // (both factors below 2^24: the launcher's caller checks the row pitch)
+      ov[i] = __umul24(h.c[i], v_row) + piece_off;
     }
     if (kc + 32 > end) {  // (uniform) the row's last step: slots past its end fetch zeros
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const bool live = kc + 4 * j + i < end;
+      for (int i = 0; i < L; ++i) {
+        const bool live = kc + L * jr + i < end;
         ok[i] = live ? ok[i] : k_bytes;
         ov[i] = live ? ov[i] : v_bytes;
       }
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) b.k[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_k, ok[i], 0, 0));
+    for (int i = 0; i < L; ++i) b.k[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_k, ok[i], 0, 0));
 #pragma unroll
-    for (int i = 0; i < 4; ++i) b.v[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_v, ov[i], 0, 0));
+    for (int i = 0; i < L; ++i) b.v[i] = __builtin_bit_cast(uintx4, __builtin_amdgcn_raw_buffer_load_b128(srd_v, ov[i], 0, 0));
   };
 
-  floatx4 acc[4];
+  floatx4 acc[NT];
 #pragma unroll
-  for (int u = 0; u < 4; ++u) acc[u] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int u = 0; u < NT; ++u) acc[u] = floatx4{0.f, 0.f, 0.f, 0.f};
   float run_max = -INFINITY, run_sum = 0.f;  // of query n; the sum only over this lane's share of the keys
 
   const auto contract = [&](const Body &b, int kc) {
     // (LDS operations of a wave execute in order: these writes land behind the previous step's reads)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) *reinterpret_cast<uintx4 *>(k_dst + i * kAttnPitch) = b.k[i];
+    for (int i = 0; i < L; ++i) *reinterpret_cast<uintx4 *>(k_dst + i * kPitch) = b.k[i];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) *reinterpret_cast<uintx4 *>(v_dst + i * kAttnPitch) = b.v[i];
+    for (int i = 0; i < L; ++i) *reinterpret_cast<uintx4 *>(v_dst + i * kPitch) = b.v[i];
     float x[8];
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       floatx4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        const half8 a = *reinterpret_cast<const half8 *>(k_rd + (uint32_t)t * (16u * kAttnPitch) + (uint32_t)c * 64u);
+      for (int c = 0; c < NC; ++c) {
+        const half8 a = *reinterpret_cast<const half8 *>(k_rd + (uint32_t)t * (16u * kPitch) + (uint32_t)c * 64u);
         s = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, q[c], s, 0, 0, 0);
       }
 #pragma unroll
@@ -533,7 +554,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
       const float alpha = __builtin_amdgcn_exp2f(run_max - new_max);
       run_sum *= alpha;
 #pragma unroll
-      for (int u = 0; u < 4; ++u) acc[u] *= alpha;
+      for (int u = 0; u < NT; ++u) acc[u] *= alpha;
       run_max = new_max;
     }
     float e[8], sum = 0.f;
@@ -546,9 +567,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
     const half8 pb = {(_Float16)e[0], (_Float16)e[1], (_Float16)e[2], (_Float16)e[3],
                       (_Float16)e[4], (_Float16)e[5], (_Float16)e[6], (_Float16)e[7]};
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < NT; ++u) {
       const uintx2 lo = lds_read_tr(v_rd + 32u * u);
-      const uintx2 hi = lds_read_tr(v_rd + 16u * kAttnPitch + 32u * u);
+      const uintx2 hi = lds_read_tr(v_rd + 16u * kPitch + 32u * u);
       const uintx4 a = {lo[0], lo[1], hi[0], hi[1]};
       acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8, a), pb, acc[u], 0, 0, 0);
     }
@@ -556,7 +577,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
 
   // Column indices run two steps ahead of the arithmetic, the rows of k and v one (two sets, used alternately).
   Body b0, b1;
-  uintx4 h0 = load_head(beg), h1 = load_head(beg + 32);
+  Head h0 = load_head(beg), h1 = load_head(beg + 32);
   load_body(b0, h0, beg);
   int kc = beg;  // the step held in b0
   for (;;) {
@@ -581,22 +602,29 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
   const float inv = 1.0f / quad_rows_sum(run_sum);
   if (n < V) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
+    for (int u = 0; u < NT; ++u) {
       const half4 h = {(_Float16)(acc[u][0] * inv), (_Float16)(acc[u][1] * inv), (_Float16)(acc[u][2] * inv), (_Float16)(acc[u][3] * inv)};
       *reinterpret_cast<uintx2 *>(out + 16 * u) = __builtin_bit_cast(uintx2, h);
     }
   }
 }
 
-hipError_t launch_sparse_attention(const AttentionArgs &a, int V, hipStream_t stream) {
+template <int V>
+static void launch_sparse_attention_v(const AttentionArgs &p, int F, hipStream_t stream) {
+  const dim3 grid(p.per_xcd * 8u), block(64);
+  if (F == 32) hipLaunchKernelGGL((sparse_attention_kernel<V, 32>), grid, block, 0, stream, p);
+  else if (F == 64) hipLaunchKernelGGL((sparse_attention_kernel<V, 64>), grid, block, 0, stream, p);
+  else hipLaunchKernelGGL((sparse_attention_kernel<V, 128>), grid, block, 0, stream, p);
+}
+
+hipError_t launch_sparse_attention(const AttentionArgs &a, int V, int F, hipStream_t stream) {
+  if (F != 32 && F != 64 && F != 128) return hipErrorInvalidValue;
   AttentionArgs p = a;
   p.total_work = (uint32_t)a.m_vec * (uint32_t)a.batch;
   p.per_xcd = (p.total_work + 7u) / 8u;
   if (p.total_work == 0) return hipSuccess;
-  if (V == 8)
-    hipLaunchKernelGGL(sparse_attention_kernel<8>, dim3(p.per_xcd * 8u), dim3(64), 0, stream, p);
-  else
-    hipLaunchKernelGGL(sparse_attention_kernel<16>, dim3(p.per_xcd * 8u), dim3(64), 0, stream, p);
+  if (V == 8) launch_sparse_attention_v<8>(p, F, stream);
+  else launch_sparse_attention_v<16>(p, F, stream);
   return hipGetLastError();
 }
 

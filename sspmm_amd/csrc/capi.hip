@@ -282,7 +282,7 @@ int sspmm_sparse_attention_heads_f16(int batch, int heads, int m_vec, int V, int
                                      int64_t ld_v, float scale, sspmm_half_t *out, int64_t stride_out, int64_t head_out,
                                      int64_t ld_out, void *hip_stream) {
   if (V != 8 && V != 16) return kInvalid;
-  if (F != 64) return kInvalid;
+  if (F != 32 && F != 64 && F != 128) return kInvalid;
   if (batch < 0 || heads < 1 || m_vec < 0 || n_keys < 0) return kInvalid;
   if (!(scale > 0.f) || !std::isfinite(scale)) return kInvalid;
   if (batch == 0 || m_vec == 0) return 0;
@@ -291,7 +291,7 @@ int sspmm_sparse_attention_heads_f16(int batch, int heads, int m_vec, int V, int
   const int64_t strides[] = {stride_q, head_q, ld_q, stride_k, head_k, ld_k, stride_v, head_v, ld_v, stride_out, head_out, ld_out};
   for (int64_t x : strides)
     if (x % 8 || x < 0) return kInvalid;
-  if (ld_q < 64 || ld_k < 64 || ld_v < 64 || ld_out < 64) return kInvalid;
+  if (ld_q < F || ld_k < F || ld_v < F || ld_out < F) return kInvalid;
   if (ld_k >= (1 << 23) || ld_v >= (1 << 23) || n_keys >= (1 << 24)) return kInvalid;  // (24-bit multiplies of column by row pitch)
   // one buffer descriptor spans the rows of an (element, head) pair
   const int64_t rows_q = (int64_t)m_vec * V, limit = (1ll << 31) - 256;
@@ -325,16 +325,16 @@ int sspmm_sparse_attention_heads_f16(int batch, int heads, int m_vec, int V, int
   a.ld_v = ld_v;
   a.ld_out = ld_out;
   a.scale = scale;
-  return (int)sspmm::launch_sparse_attention(a, V, static_cast<hipStream_t>(hip_stream));
+  return (int)sspmm::launch_sparse_attention(a, V, F, static_cast<hipStream_t>(hip_stream));
 }
 
 int sspmm_sparse_attention_f16(int batch, int m_vec, int V, int F, int n_keys, const int32_t *row_indices,
                                const int32_t *row_offsets, const int32_t *col_idx, const sspmm_half_t *q, int64_t stride_q,
                                const sspmm_half_t *k, int64_t stride_k, const sspmm_half_t *v, int64_t stride_v, float scale,
                                sspmm_half_t *out, int64_t stride_out, void *hip_stream) {
-  if (batch > 1 && stride_out < (int64_t)m_vec * V * 64) return kInvalid;  // (the batch elements' outputs must not overlap)
-  return sspmm_sparse_attention_heads_f16(batch, 1, m_vec, V, F, n_keys, row_indices, row_offsets, col_idx, q, stride_q, 0, 64,
-                                          k, stride_k, 0, 64, v, stride_v, 0, 64, scale, out, stride_out, 0, 64, hip_stream);
+  if (batch > 1 && stride_out < (int64_t)m_vec * V * F) return kInvalid;  // (the batch elements' outputs must not overlap)
+  return sspmm_sparse_attention_heads_f16(batch, 1, m_vec, V, F, n_keys, row_indices, row_offsets, col_idx, q, stride_q, 0, F,
+                                          k, stride_k, 0, F, v, stride_v, 0, F, scale, out, stride_out, 0, F, hip_stream);
 }
 
 size_t svc_workspace_bytes(int M, int64_t nnz, int V) {

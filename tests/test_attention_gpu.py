@@ -133,25 +133,26 @@ def _dense_attention(off, cols, V, q, k, v, scale):
     return out
 
 
+@pytest.mark.parametrize("d", [32, 64, 128])
 @pytest.mark.parametrize("V", [8, 16])
-def test_one_launch_attention_row_lengths_permutation_and_large_scores(built_library, V):
+def test_one_launch_attention_row_lengths_permutation_and_large_scores(built_library, V, d):
     """Rows of every length around the kernel's step of 32 vectors (none, one, a full step, one more, several steps
     and a tail), visited through a permutation, with scores large enough that the running maximum has to move by
     hundreds between steps; against float64 arithmetic and against the three launches."""
-    n_keys, d, batch = 200, 64, 3
+    n_keys, batch = 200, 3
     lens = [0, 1, 2, 31, 32, 33, 63, 64, 65, 96, 100, 200, 0, 7]
-    rng = np.random.default_rng(40 + V)
+    rng = np.random.default_rng(40 + V + d)
     cols = np.concatenate([np.sort(rng.permutation(n_keys)[:n]) for n in lens]).astype(np.int32)
     off = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
     m = len(lens) * V
-    q = (rng.standard_normal((batch, m, d)) * 3).astype(np.float16)
+    q = (rng.standard_normal((batch, m, d)) * 3 * (64 / d) ** 0.5).astype(np.float16)
     k = (rng.standard_normal((batch, n_keys, d)) * 3).astype(np.float16)
     v = rng.standard_normal((batch, n_keys, d)).astype(np.float16)
     perm = dev(rng.permutation(len(lens)).astype(np.int32))
     for scale in (0.125, 2.0):  # scores up to a few hundred, then a few thousand
         want = _dense_attention(off, cols, V, q, k, v, scale)
         for ri in (None, perm):
-            print("attention V=%d scale=%g permuted=%s" % (V, scale, ri is not None), flush=True)
+            print("attention V=%d d=%d scale=%g permuted=%s" % (V, d, scale, ri is not None), flush=True)
             got = sspmm_amd.fused_sparse_attention(ri, dev(off), dev(cols), dev(q), dev(k), dev(v), scale, V)
             torch.cuda.synchronize()
             got = got.cpu().numpy().astype(np.float64)
@@ -167,9 +168,9 @@ def test_one_launch_attention_row_lengths_permutation_and_large_scores(built_lib
     assert (one.float() - chain.float()).abs().max().item() <= 3e-2
 
 
-@pytest.mark.parametrize("d", [32, 128])
+@pytest.mark.parametrize("d", [40, 256])
 def test_heads_of_other_widths_take_the_three_operators(built_library, d):
-    """`sparse_attention` with nothing forced: heads that are not 64 wide run the chain, and `fused=True` says so."""
+    """`sparse_attention` with nothing forced: heads that are not 32, 64 or 128 wide run the chain, and `fused=True` says so."""
     V, seq, batch = 8, 128, 2
     vs = _pattern(seq // V, seq, V, 0.75, seed=31)
     off, col = dev(vs.row_offsets), dev(vs.col_idx)
@@ -182,31 +183,33 @@ def test_heads_of_other_widths_take_the_three_operators(built_library, d):
         sspmm_amd.sparse_attention(None, off, col, q, k, v, d ** -0.5, V, fused=True)
 
 
-def test_one_launch_attention_of_a_single_key_returns_its_value_row(built_library):
+@pytest.mark.parametrize("d", [32, 64, 128])
+def test_one_launch_attention_of_a_single_key_returns_its_value_row(built_library, d):
     """A query that attends to one key gets that row of v back exactly (probability one, fp16 in and out)."""
     V, n_keys, m_vec = 8, 50, 5
-    rng = np.random.default_rng(3)
+    rng = np.random.default_rng(3 + d)
     cols = rng.integers(0, n_keys, m_vec).astype(np.int32)
     off = np.arange(m_vec + 1, dtype=np.int32)
-    q, k, v = (rng.standard_normal((2, n, 64)).astype(np.float16) for n in (m_vec * V, n_keys, n_keys))
+    q, k, v = (rng.standard_normal((2, n, d)).astype(np.float16) for n in (m_vec * V, n_keys, n_keys))
     got = sspmm_amd.fused_sparse_attention(None, dev(off), dev(cols), dev(q), dev(k), dev(v), 0.125, V).cpu().numpy()
     for i in range(m_vec):
         assert np.array_equal(got[:, i * V:(i + 1) * V], np.repeat(v[:, cols[i]][:, None], V, axis=1))
 
 
+@pytest.mark.parametrize("d", [32, 64, 128])
 @pytest.mark.parametrize("V", [8, 16])
-def test_packed_heads_give_the_bits_of_the_copied_out_heads(built_library, V):
-    """The launch on a fused projection [seq, batch, 3 * heads * 64] against the same launch on q, k and v copied out
-    into [batch * heads, seq, 64] as the reference's module lays them out (spattention.py:151-157, 181-184)."""
+def test_packed_heads_give_the_bits_of_the_copied_out_heads(built_library, V, d):
+    """The launch on a fused projection [seq, batch, 3 * heads * d] against the same launch on q, k and v copied out
+    into [batch * heads, seq, d] as the reference's module lays them out (spattention.py:151-157, 181-184)."""
     seq, bsz, heads = 192, 3, 5
-    E = heads * 64
+    E = heads * d
     vs = _pattern(seq // V, seq, V, 0.7, seed=21)
     off, col = dev(vs.row_offsets), dev(vs.col_idx)
     g = torch.Generator("cuda").manual_seed(22)
     qkv = torch.randn(seq, bsz, 3 * E, device="cuda", generator=g).half()
     got = sspmm_amd.sparse_attention_packed(None, off, col, qkv, heads, 0.125, V)
     torch.cuda.synchronize()
-    q, k, v = (t.contiguous().view(seq, bsz * heads, 64).transpose(0, 1).contiguous() for t in qkv.chunk(3, dim=-1))
+    q, k, v = (t.contiguous().view(seq, bsz * heads, d).transpose(0, 1).contiguous() for t in qkv.chunk(3, dim=-1))
     want = sspmm_amd.fused_sparse_attention(None, off, col, q, k, v, 0.125, V)
     want = want.transpose(0, 1).contiguous().view(seq, bsz, E)
     assert got.shape == (seq, bsz, E)
@@ -226,8 +229,8 @@ def test_argument_errors(built_library):
         sspmm_amd.sddmm(None, off, col, torch.zeros(16, 64, device="cuda").half(), torch.zeros(8, 32, device="cuda").half(), 8)
     with pytest.raises(TypeError):
         sspmm_amd.csr_softmax(None, off, torch.zeros(0, device="cuda"), 1.0, 8)
-    with pytest.raises(ValueError):  # the one-launch block takes heads of 64 features only
-        sspmm_amd.fused_sparse_attention(None, off, col, *(torch.zeros(1, 16, 32, device="cuda").half() for _ in range(3)), 1.0, 8)
+    with pytest.raises(ValueError):  # the one-launch block takes heads of 32, 64 or 128 features
+        sspmm_amd.fused_sparse_attention(None, off, col, *(torch.zeros(1, 16, 48, device="cuda").half() for _ in range(3)), 1.0, 8)
     with pytest.raises(RuntimeError):  # scale must be positive
         sspmm_amd.fused_sparse_attention(None, off, col, *(torch.zeros(1, 16, 64, device="cuda").half() for _ in range(3)), 0.0, 8)
     with pytest.raises(RuntimeError):  # F must be a multiple of 8

@@ -68,10 +68,10 @@ def test_argument_errors_without_device_work(built_library):
     assert L.sspmm_attention_fm_f16(0, 1, 64, 64, None, None, None, 0, None, 0, 0.125, None) == 0
     for bad_scale in (0.0, -0.125, float("nan"), float("inf")):
         assert L.sspmm_attention_fm_f16(1, 1, 64, 64, 16, 16, 16, 64, 16, 64, bad_scale, None) == 1
-    # the one-launch sparse attention block: heads of 64 features, V of 8 or 16, a positive finite scale, aligned operands
+    # the one-launch sparse attention block: heads of 32, 64 or 128 features, V of 8 or 16, a positive finite scale, aligned operands
     sa = lambda V=8, F=64, q=16, stride=512, scale=0.125: L.sspmm_sparse_attention_f16(  # noqa: E731
         1, 1, V, F, 8, None, 16, 16, q, stride, 16, 512, 16, 512, scale, 16, 512, None)
-    assert sa(V=4) == 1 and sa(F=32) == 1 and sa(F=128) == 1 and sa(q=8) == 1 and sa(stride=4) == 1
+    assert sa(V=4) == 1 and sa(F=48) == 1 and sa(F=256) == 1 and sa(q=8) == 1 and sa(stride=4) == 1
     for bad_scale in (0.0, -0.125, float("nan"), float("inf")):
         assert sa(scale=bad_scale) == 1
     assert L.sspmm_sparse_attention_f16(0, 4, 8, 64, 8, None, None, None, None, 0, None, 0, None, 0, 0.125, None, 0, None) == 0

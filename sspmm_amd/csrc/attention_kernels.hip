@@ -431,7 +431,7 @@ __device__ __forceinline__ float quad_rows_sum(float x) {
 // brings 64 / LPR rows, a step of 32 rows takes L = LPR / 2 of them per operand; lane (jr, pc) fetches piece pc of the
 // rows of k slots L * jr .. L * jr + L - 1, whose column indices it reads as L consecutive ints.
 template <int V, int F>
-__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) void sparse_attention_kernel(const AttentionArgs p) {
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(F == 32 ? 4 : 2, F == 32 ? 4 : 2))) void sparse_attention_kernel(const AttentionArgs p) {
   constexpr int LPR = F / 8, L = LPR / 2, NC = F / 32, NT = F / 16;
   constexpr uint32_t kRowBytes = F * 2u, kPitch = kRowBytes + 16u;  // staged rows padded by 16 bytes against bank conflicts
   __shared__ __align__(16) unsigned char stage_k[32 * kPitch];

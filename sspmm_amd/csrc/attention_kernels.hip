@@ -457,7 +457,9 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(F == 32 ? 4 
   const uint32_t q_row = (uint32_t)p.ld_q * 2u, k_row = (uint32_t)p.ld_k * 2u, v_row = (uint32_t)p.ld_v * 2u;
   const __amdgpu_buffer_rsrc_t srd_q = make_srd(p.q + (int64_t)elem * p.stride_q + (int64_t)head * p.head_q + (int64_t)row * V * p.ld_q,
                                                 (uint32_t)(V - 1) * q_row + kRowBytes);
-  const uint32_t k_bytes = (uint32_t)(p.n_keys - 1) * k_row + kRowBytes, v_bytes = (uint32_t)(p.n_keys - 1) * v_row + kRowBytes;
+  // (no keys at all: descriptors of zero bytes, whatever a pattern then names reads as zeros)
+  const uint32_t k_bytes = p.n_keys > 0 ? (uint32_t)(p.n_keys - 1) * k_row + kRowBytes : 0u;
+  const uint32_t v_bytes = p.n_keys > 0 ? (uint32_t)(p.n_keys - 1) * v_row + kRowBytes : 0u;
   const __amdgpu_buffer_rsrc_t srd_k = make_srd(p.k + (int64_t)elem * p.stride_k + (int64_t)head * p.head_k, k_bytes);
   const __amdgpu_buffer_rsrc_t srd_v = make_srd(p.v + (int64_t)elem * p.stride_v + (int64_t)head * p.head_v, v_bytes);
   const __amdgpu_buffer_rsrc_t srd_cols = make_srd(p.col_idx, (uint32_t)end * 4u);  // past the row: reads 0

@@ -168,6 +168,35 @@ def test_one_launch_attention_row_lengths_permutation_and_large_scores(built_lib
     assert (one.float() - chain.float()).abs().max().item() <= 3e-2
 
 
+def test_one_launch_attention_at_full_size_by_its_properties(built_library):
+    """The benchmark's block (4096 tokens, 90 % of the vectors masked out, 48 heads of 64 features): with every row of
+    v the same the probabilities of a row must add up to one, so every query gets that row back; columns stored in
+    another order inside the vector-rows change the sums' order only; a permutation of the vector-rows changes nothing."""
+    V, seq, heads, d = 8, 4096, 48, 64
+    from sspmm_amd.attention import static_random_mask
+    cols, off, rows = static_random_mask(seq // V, seq, 0.9, seed=5)
+    rng = np.random.default_rng(6)
+    shuffled = cols.copy()
+    for i in range(len(off) - 1):
+        rng.shuffle(shuffled[off[i]:off[i + 1]])
+    g = torch.Generator("cuda").manual_seed(7)
+    q, k, v = (torch.randn(heads, seq, d, device="cuda", generator=g).half() for _ in range(3))
+    const = torch.full((d,), 0.0, device="cuda").half()
+    const[::2], const[1::2] = 0.75, -1.5
+    v_const = const.expand(heads, seq, d).contiguous()
+    d_off, d_cols, d_rows, d_shuf = dev(off), dev(cols), dev(rows), dev(shuffled)
+    print("attention at full size: %d vectors per head" % cols.size, flush=True)
+    out = sspmm_amd.fused_sparse_attention(None, d_off, d_cols, q, k, v_const, 0.125, V)
+    assert (out.float() - const.float()).abs().max().item() <= 2e-3
+    a = sspmm_amd.fused_sparse_attention(None, d_off, d_cols, q, k, v, 0.125, V)
+    b = sspmm_amd.fused_sparse_attention(d_rows, d_off, d_cols, q, k, v, 0.125, V)
+    c = sspmm_amd.fused_sparse_attention(None, d_off, d_shuf, q, k, v, 0.125, V)
+    assert torch.equal(a, b)
+    assert (a.float() - c.float()).abs().max().item() <= 2e-3
+    chain = sspmm_amd.sparse_attention(None, d_off, d_cols, q, k, v, 0.125, V, fused=False)
+    assert (a.float() - chain.float()).abs().max().item() <= 4e-3
+
+
 @pytest.mark.parametrize("d", [40, 256])
 def test_heads_of_other_widths_take_the_three_operators(built_library, d):
     """`sparse_attention` with nothing forced: heads that are not 32, 64 or 128 wide run the chain, and `fused=True` says so."""

@@ -672,7 +672,8 @@ def run_attention_forward(torch, sparsity, bsz, seq, heads, embed, st, wu, mlp=1
     "PyTorch" column)."""
     from sspmm_amd.attention import SparseAttentionEncoder
     torch.manual_seed(0)
-    model = SparseAttentionEncoder(257, embed, heads, sparsity, seq, mlp, 2, vec_length=8, layers=4, seed=20).cuda().half().eval()
+    # (the head is as wide as the MLP, as the reference's driver builds it: end_to_end.py:176-185, num_class=args.mlp_dim)
+    model = SparseAttentionEncoder(257, embed, heads, sparsity, seq, mlp, mlp, vec_length=8, layers=4, seed=20).cuda().half().eval()
     tokens = torch.randint(0, 257, (bsz, seq), device="cuda")
 
     def dense_forward():
